@@ -1,0 +1,223 @@
+"""ctypes bindings of the CPU oracle (test infrastructure only).
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
+import this package.  ``libmoe_oracle.so`` is the plain-C restatement in ``moe_oracle.c``;
+``_ref/libck_ref.so`` is Composable Kernel's own host reference compiled from the ck_tile headers
+that ship with ROCm (``ck_ref.cpp``).  Both are built by ``oracle/Makefile``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+DT_F32, DT_BF16, DT_E4M3, DT_I8 = 0, 1, 2, 3
+_NP_OF_DT = {DT_F32: np.float32, DT_BF16: np.uint16, DT_E4M3: np.uint8, DT_I8: np.int8}
+
+
+def build(force: bool = False) -> None:
+    """Compile the oracle libraries (gcc, and hipcc for the ck_tile reference)."""
+    args = ["make", "-C", _HERE]
+    if force:
+        args.append("-B")
+    subprocess.run(args, check=True, stdout=subprocess.DEVNULL)
+
+
+def _load(path: str):
+    return C.CDLL(path) if os.path.exists(path) else None
+
+
+_lib = None
+_ref = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        p = os.path.join(_HERE, "libmoe_oracle.so")
+        if not os.path.exists(p):
+            build()
+        _lib = C.CDLL(p)
+        _lib.moe_oracle_bf16_to_f32.restype = C.c_float
+        _lib.moe_oracle_bf16_to_f32.argtypes = [C.c_uint16]
+        _lib.moe_oracle_f32_to_bf16.restype = C.c_uint16
+        _lib.moe_oracle_f32_to_bf16.argtypes = [C.c_float]
+        _lib.moe_oracle_e4m3_to_f32.restype = C.c_float
+        _lib.moe_oracle_e4m3_to_f32.argtypes = [C.c_uint8]
+        _lib.moe_oracle_f32_to_e4m3.restype = C.c_uint8
+        _lib.moe_oracle_f32_to_e4m3.argtypes = [C.c_float]
+        _lib.moe_oracle_silu.restype = C.c_float
+        _lib.moe_oracle_silu.argtypes = [C.c_float]
+        _lib.moe_oracle_num_threads.restype = C.c_int
+        _lib.moe_oracle_set_num_threads.argtypes = [C.c_int]
+    return _lib
+
+
+def ck_ref():
+    """ck_tile's own reference, or None when oracle/_ref has not been built."""
+    global _ref
+    if _ref is None:
+        _ref = _load(os.path.join(_HERE, "_ref", "libck_ref.so"))
+        if _ref is not None:
+            _ref.ck_ref_f32_to_bf16.restype = C.c_uint16
+            _ref.ck_ref_f32_to_bf16.argtypes = [C.c_float]
+            _ref.ck_ref_f32_to_fp8.restype = C.c_uint8
+            _ref.ck_ref_f32_to_fp8.argtypes = [C.c_float]
+            _ref.ck_ref_fp8_to_f32.restype = C.c_float
+            _ref.ck_ref_fp8_to_f32.argtypes = [C.c_uint8]
+            _ref.ck_ref_silu.restype = C.c_float
+            _ref.ck_ref_silu.argtypes = [C.c_float]
+    return _ref
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dtype):
+    return None if a is None else np.ascontiguousarray(a, dtype=dtype)
+
+
+def max_num_tokens_padded(tokens: int, topk: int, experts: int, unit: int) -> int:
+    return topk * tokens + experts * unit - topk
+
+
+# --------------------------------------------------------------------------- conversions
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    """Vectorised RNE float32 -> bf16 bit pattern (same rule as moe_oracle_f32_to_bf16)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u + (0x7FFF + ((u >> 16) & 1))) >> 16).astype(np.uint16)
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r
+
+
+def bf16_to_f32(h: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(h, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+_E4M3_TABLE = None
+
+
+def e4m3_table() -> np.ndarray:
+    """256-entry decode table produced by the C oracle."""
+    global _E4M3_TABLE
+    if _E4M3_TABLE is None:
+        l = lib()
+        _E4M3_TABLE = np.array([l.moe_oracle_e4m3_to_f32(i) for i in range(256)], dtype=np.float32)
+    return _E4M3_TABLE
+
+
+def e4m3_to_f32(q: np.ndarray) -> np.ndarray:
+    return e4m3_table()[np.ascontiguousarray(q, dtype=np.uint8)]
+
+
+def to_f32(x: np.ndarray, dt: int) -> np.ndarray:
+    if dt == DT_F32:
+        return np.asarray(x, dtype=np.float32)
+    if dt == DT_BF16:
+        return bf16_to_f32(x)
+    if dt == DT_E4M3:
+        return e4m3_to_f32(x)
+    return np.asarray(x, dtype=np.int8).astype(np.float32)
+
+
+def rowwise_quant(x: np.ndarray, dt: int):
+    """Per-row dynamic quantisation of a float32 [M,N] matrix -> (q, scale[M])."""
+    x = _c(x, np.float32)
+    M, N = x.shape
+    q = np.empty((M, N), dtype=_NP_OF_DT[dt])
+    s = np.empty((M,), dtype=np.float32)
+    rc = lib().moe_oracle_rowwise_quant(_p(x), C.c_int64(M), C.c_int64(N), C.c_int(dt), _p(q), _p(s))
+    if rc != 0:
+        raise ValueError("rowwise_quant: unsupported dtype")
+    return q, s
+
+
+# ------------------------------------------------------------------------------- sorting
+def moe_sorting(topk_ids, weights, experts, unit, local_expert_mask=None, skip_empty=True,
+                fill_id=-1, fill_w=-1.0, fill_eid=-1):
+    """Returns (sorted_ids[max_pad], sorted_w[max_pad], sorted_eid[tiles_max], post_pad).
+    Cells past the written prefix keep the fill values."""
+    topk_ids = _c(topk_ids, np.int32)
+    weights = _c(weights, np.float32)
+    T, K = topk_ids.shape
+    mp = max_num_tokens_padded(T, K, experts, unit)
+    ids = np.full((mp,), fill_id, dtype=np.int32)
+    w = np.full((mp,), fill_w, dtype=np.float32)
+    eid = np.full(((mp + unit - 1) // unit,), fill_eid, dtype=np.int32)
+    pp = C.c_int32(0)
+    mask = _c(local_expert_mask, np.int32)
+    rc = lib().moe_oracle_sorting(_p(topk_ids), _p(weights), _p(mask), T, K, experts, unit,
+                                  int(bool(skip_empty)), _p(ids), _p(w), _p(eid), C.byref(pp))
+    if rc < 0:
+        raise ValueError(f"moe_oracle_sorting failed ({rc})")
+    return ids, w, eid, int(pp.value)
+
+
+def ck_moe_sorting(topk_ids, weights, experts, unit, local_expert_mask=None, skip_empty=True,
+                   fill_id=-1, fill_w=-1.0, fill_eid=-1):
+    """Same contract as moe_sorting, computed by ck_tile::reference_moe_sorting."""
+    r = ck_ref()
+    if r is None:
+        raise RuntimeError("oracle/_ref is not built")
+    topk_ids = _c(topk_ids, np.int32)
+    weights = _c(weights, np.float32)
+    T, K = topk_ids.shape
+    mp = max_num_tokens_padded(T, K, experts, unit)
+    ids = np.full((mp,), fill_id, dtype=np.int32)
+    w = np.full((mp,), fill_w, dtype=np.float32)
+    eid = np.full(((mp + unit - 1) // unit,), fill_eid, dtype=np.int32)
+    mask = _c(local_expert_mask, np.int32)
+    pp = r.ck_ref_moe_sorting(_p(topk_ids), _p(weights), _p(mask), T, K, experts, unit,
+                              int(mask is not None), int(bool(skip_empty)), _p(ids), _p(w), _p(eid))
+    return ids, w, eid, int(pp)
+
+
+# ----------------------------------------------------------------------------- fused MoE
+def fused_moe(a, a_dt, g, g_dt, d, d_dt, sorted_ids, sorted_w, sorted_eid, post_pad, block_m,
+              tokens, experts, hidden, inter, topk, a_scale=None, g_scale=None, d_scale=None,
+              gate_only=False, out_dt=DT_BF16, strict=False, want_partials=False):
+    """Oracle forward.  Operands are numpy arrays holding the raw storage type of their dtype
+    code (uint16 for bf16, uint8 for e4m3, int8, float32).  Returns o[tokens, hidden] (uint16 bf16
+    bits or float32) and, if asked, the fp32 per-slot partials [tokens, topk, hidden]."""
+    a = _c(a, _NP_OF_DT[a_dt])
+    g = _c(g, _NP_OF_DT[g_dt])
+    d = _c(d, _NP_OF_DT[d_dt])
+    n0 = inter * (1 if gate_only else 2)
+    assert a.size == tokens * hidden and g.size == experts * n0 * hidden and d.size == experts * hidden * inter
+    a_scale, g_scale, d_scale = _c(a_scale, np.float32), _c(g_scale, np.float32), _c(d_scale, np.float32)
+    o = np.empty((tokens, hidden), dtype=_NP_OF_DT[out_dt])
+    part = np.empty((tokens, topk, hidden), dtype=np.float32) if want_partials else None
+    ids, w, eid = _c(sorted_ids, np.int32), _c(sorted_w, np.float32), _c(sorted_eid, np.int32)
+    rc = lib().moe_oracle_fused_moe(_p(a), a_dt, _p(a_scale), _p(g), g_dt, _p(g_scale), _p(d), d_dt,
+                                    _p(d_scale), _p(o), out_dt, _p(ids), _p(w), _p(eid),
+                                    int(post_pad), block_m, tokens, experts, hidden, inter, topk,
+                                    int(bool(gate_only)), int(bool(strict)), _p(part))
+    if rc != 0:
+        raise MemoryError("moe_oracle_fused_moe failed")
+    return (o, part) if want_partials else o
+
+
+def ck_fused_moe(a, g, d, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, tokens, experts,
+                 hidden, inter, topk, gate_only=False, f32_inputs=False):
+    """ck_tile::reference_fused_moe on bf16 (uint16 bits) or float32 operands -> bf16 bits."""
+    r = ck_ref()
+    if r is None:
+        raise RuntimeError("oracle/_ref is not built")
+    dt = np.float32 if f32_inputs else np.uint16
+    a, g, d = _c(a, dt), _c(g, dt), _c(d, dt)
+    o = np.empty((tokens, hidden), dtype=np.uint16)
+    fn = r.ck_ref_fused_moe_f32 if f32_inputs else r.ck_ref_fused_moe_bf16
+    ids, w, eid = _c(sorted_ids, np.int32), _c(sorted_w, np.float32), _c(sorted_eid, np.int32)
+    fn(_p(a), _p(g), _p(d), _p(o), _p(ids), _p(w), _p(eid), int(post_pad), block_m, tokens, experts,
+       hidden, inter, topk, int(bool(gate_only)))
+    return o
+
+
+def num_threads() -> int:
+    return int(lib().moe_oracle_num_threads())
