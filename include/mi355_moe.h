@@ -1,0 +1,188 @@
+/*
+ * mi355_moe.h - C ABI of the MI355X-native fused-MoE path (libmi355_moe.so).
+ *
+ * Every entry point takes plain pointers and sizes; all data pointers are DEVICE pointers owned by
+ * the caller, launches are asynchronous on the given HIP stream (passed as void*, NULL = default
+ * stream) and nothing is allocated behind the caller's back.  The structs mirror, field for
+ * field, the host argument blocks of Composable Kernel's ck_tile fused-MoE (ck_tile 1.2.0, paths
+ * relative to /opt/rocm/include/ck_tile):
+ *
+ *   mi355_moe_sorting_args   <- MoeSortingHostArgs    ops/fused_moe/kernel/moe_sorting_kernel.hpp:188-222
+ *   mi355_fused_moegemm_args <- FusedMoeGemmHostArgs  ops/fused_moe/kernel/fused_moegemm_kernel.hpp:97-120
+ *   mi355_fused_moe_args     <- fused_moe_args  of CK's example/ck_tile/15_fused_moe/fused_moe.hpp
+ *   mi355_fused_moe_traits   <- fused_moe_traits of the same example, with enums for its strings
+ *
+ * Return value of every int function: 0 on success, negative on failure (MI355_MOE_E_*);
+ * mi355_moe_last_error() returns a human-readable description for the calling thread.
+ */
+#ifndef MI355_MOE_H
+#define MI355_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_MOE_VERSION 100
+
+enum mi355_moe_status
+{
+    MI355_MOE_OK            = 0,
+    MI355_MOE_E_UNSUPPORTED = -1, /* no kernel for these traits (ck_tile's fused_moe() returns -1 too) */
+    MI355_MOE_E_INVALID     = -2, /* null pointer, size out of range, misaligned stride ... */
+    MI355_MOE_E_HIP         = -3, /* a HIP runtime call failed */
+    MI355_MOE_E_WORKSPACE   = -4  /* workspace missing or too small */
+};
+
+/* element types; the strings are the spellings of ck_tile's traits ("bf16", "fp8", "int8", ...) */
+enum mi355_moe_dtype
+{
+    MI355_MOE_BF16 = 0,
+    MI355_MOE_FP8  = 1, /* OCP e4m3 */
+    MI355_MOE_INT8 = 2,
+    MI355_MOE_FP32 = 3,
+    MI355_MOE_INT32 = 4,
+    MI355_MOE_FP16 = 5
+};
+
+/* ------------------------------------------------------------------------------ moe_sorting
+ * Replaces ck_tile::MoeSortingKernel / MoeSortingMultiPhaseKernel_* behind MoeSortingHostArgs
+ * (moe_sorting_kernel.hpp:188-222) and the example's moe_sorting(trait, args, stream).
+ * Output contract = ck_tile::reference_moe_sorting (host/reference/reference_moe_sorting.hpp:14-117)
+ * with skip_experts_with_zero_token = true: cells past the written prefix are left untouched. */
+typedef struct mi355_moe_sorting_args
+{
+    const void* p_topk_ids;          /* [tokens, topk] int32, distinct experts per token */
+    const void* p_weights;           /* [tokens, topk] fp32 */
+    const void* p_local_expert_mask; /* [num_experts] int32 or NULL; 0 = expert not on this rank */
+    const void* p_local_tokens;      /* [1] int32 or NULL; if set, the token count is read on device */
+    void* p_sorted_token_ids;        /* [max_num_tokens_padded] int32: token | topk_slot << 24 */
+    void* p_sorted_weights;          /* [max_num_tokens_padded] fp32 */
+    void* p_sorted_expert_ids;       /* [ceil(max_num_tokens_padded / unit_size)] int32 */
+    void* p_total_tokens_post_pad;   /* [2] int32: [0] tokens after padding, [1] actual tokens */
+    void* p_moe_buf;                 /* buffer to zero alongside the sort, or NULL */
+    void* p_ws;                      /* mi355_moe_sorting_workspace_size() bytes (may be NULL if 0);
+                                        unlike ck_tile it need not be cleared */
+    int32_t tokens;                  /* token count, or its upper bound when p_local_tokens is set */
+    int32_t unit_size;               /* block_m of the GEMM that consumes the result */
+    int32_t num_experts;
+    int32_t topk;
+    int32_t moe_buf_interm_dim;      /* p_moe_buf is [tokens, moe_buf_interm_dim] elements ... */
+    int32_t moe_buf_elem_bytes;      /* ... of this many bytes; a row must be a multiple of 16 B */
+} mi355_moe_sorting_args;
+
+/* max_num_tokens_padded = topk*tokens + num_experts*unit_size - topk (moe_sorting_kernel.hpp:64) */
+int64_t mi355_moe_max_num_tokens_padded(int32_t tokens, int32_t num_experts, int32_t topk, int32_t unit_size);
+
+/* replaces moe_sorting_get_workspace_size() (moe_sorting_kernel.hpp:1394-1438) */
+size_t mi355_moe_sorting_workspace_size(int32_t tokens, int32_t num_experts, int32_t topk);
+
+/* replaces moe_sorting(moe_sorting_trait, moe_sorting_args, stream_config) of CK's
+ * example/ck_tile/13_moe_sorting; index type int32 and weight type fp32 are the only ones CK has */
+int mi355_moe_sorting(const mi355_moe_sorting_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------- fused MoE */
+typedef struct mi355_fused_moe_traits
+{
+    int32_t prec_i;  /* activation dtype  (mi355_moe_dtype): BF16 | FP8 | INT8 */
+    int32_t prec_w;  /* weight dtype: same as prec_i */
+    int32_t prec_o;  /* output dtype: BF16 */
+    int32_t prec_st; /* per-token activation scale dtype: FP32 */
+    int32_t prec_sw; /* per-channel weight scale dtype: FP32 */
+    int32_t prec_sq; /* smooth-quant scale dtype: FP32 (unused) */
+    int32_t prec_kw; /* top-k weight dtype: FP32 */
+    int32_t block_m; /* rows per sorted tile = unit_size of the sort: 16, 32, 64 or 128 */
+    int32_t activation;  /* 0 = gelu (unsupported), 1 = silu */
+    int32_t gate_only;   /* 0 = gate and up ([e, 2*inter, hidden]), 1 = gate only (unsupported) */
+    int32_t fused_quant; /* 0 = none; quantised dtypes always take a_scale/g_scale/d_scale */
+    int32_t local_expert_masking; /* 1 = apply local_expert_mask_ptr in the sort */
+} mi355_fused_moe_traits;
+
+/* FusedMoeGemmHostArgs (fused_moegemm_kernel.hpp:97-120) plus the workspace this build needs for
+ * the intermediate activations.  Weights are plain row-major, K contiguous (what ck_tile's host
+ * reference takes; FusedMoeGemmWeightPermuteEnum::no_permute, fused_moegemm_traits.hpp:10-17). */
+typedef struct mi355_fused_moegemm_args
+{
+    const void* a_ptr;              /* [tokens, stride_token] activations */
+    const void* a_scale_ptr;        /* [tokens] fp32 per-token scale (quantised dtypes) or NULL */
+    const void* g_ptr;              /* [experts, 2*inter, hidden] gate rows then up rows */
+    const void* d_ptr;              /* [experts, hidden, inter] */
+    const void* g_scale_ptr;        /* [experts, 2*inter] fp32 or NULL */
+    const void* d_scale_ptr;        /* [experts, hidden] fp32 or NULL */
+    const void* y_smooth_scale_ptr; /* [experts, inter]; accepted, must be NULL */
+    void* o_ptr;                    /* [tokens, stride_token] output, written (not accumulated) */
+    const void* sorted_token_ids_ptr;  /* as written by mi355_moe_sorting */
+    const void* sorted_weight_ptr;
+    const void* sorted_expert_ids_ptr;
+    const void* num_sorted_tiles_ptr;  /* [>=1] int32: [0] holds tokens_post_pad (:243-246) */
+    void* ws_ptr;                   /* mi355_fused_moe_workspace_size() bytes */
+    size_t ws_bytes;
+    int32_t hidden_size;
+    int32_t intermediate_size;
+    int32_t num_tokens;
+    int32_t num_experts;
+    int32_t topk;
+    int32_t stride_token;           /* elements between rows of a and of o (>= hidden_size) */
+} mi355_fused_moegemm_args;
+
+/* fused_moe_args of CK's example: the GEMM arguments plus routing inputs and sort outputs */
+typedef struct mi355_fused_moe_args
+{
+    const void* a_ptr;
+    const void* a_scale_ptr;
+    const void* g_ptr;
+    const void* d_ptr;
+    const void* g_scale_ptr;
+    const void* d_scale_ptr;
+    const void* y_smooth_scale_ptr;
+    const void* local_expert_mask_ptr; /* [experts] int32, used when traits.local_expert_masking */
+    void* o_ptr;
+    void* ws_ptr;                      /* mi355_fused_moe_workspace_size() bytes */
+    size_t ws_bytes;
+    const void* topk_ids_ptr;          /* [tokens, topk] int32 */
+    const void* topk_weight_ptr;       /* [tokens, topk] fp32 */
+    void* sorted_token_ids_ptr;        /* outputs of the sort, sized as for mi355_moe_sorting */
+    void* sorted_weight_ptr;
+    void* sorted_expert_ids_ptr;
+    void* num_sorted_tiles_ptr;        /* [2] int32 */
+    int32_t block_m;
+    int32_t hidden_size;
+    int32_t intermediate_size;
+    int32_t num_tokens;
+    int32_t num_experts;
+    int32_t topk;
+    int32_t stride_token;
+} mi355_fused_moe_args;
+
+/* 1 if a kernel exists for these traits, else 0 (ck_tile's dispatcher returns -1 from fused_moe) */
+int mi355_fused_moe_supported(const mi355_fused_moe_traits* traits);
+
+/* bytes of ws_ptr for mi355_fused_moe / mi355_fused_moegemm (includes the sort's own workspace) */
+size_t mi355_fused_moe_workspace_size(const mi355_fused_moe_traits* traits, int32_t tokens,
+                                      int32_t num_experts, int32_t topk, int32_t hidden_size,
+                                      int32_t intermediate_size);
+
+/* replaces fused_moegemm(traits, args, stream): FusedMoeGemmKernel (fused_moegemm_kernel.hpp:238-259).
+ * Gate+up GEMM with SiLU*up, down GEMM, top-k weighted combine into o. */
+int mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_moegemm_args* args,
+                        void* stream);
+
+/* replaces fused_moe(traits, args, stream) of CK's example: mi355_moe_sorting then
+ * mi355_fused_moegemm on one stream */
+int mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* args, void* stream);
+
+/* per-row dynamic quantisation of bf16 activations, the step in front of the quantised path:
+ * scale[m] = amax(row)/qmax, q = saturate(x/scale) (host/reference/reference_rowwise_quantization2d.hpp:12-31).
+ * x [rows, stride_x] bf16 -> q [rows, cols] (FP8 or INT8), scale [rows] fp32. */
+int mi355_moe_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype,
+                            void* q, void* scale, void* stream);
+
+const char* mi355_moe_last_error(void);
+int mi355_moe_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_MOE_H */

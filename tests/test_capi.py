@@ -1,0 +1,72 @@
+"""The C ABI without a GPU: libmi355_moe.so loads, exports every function include/mi355_moe.h
+declares, the ctypes mirrors have the C structs' layout, and host-only entry points answer."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+
+from therock_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mi355_moe.h")
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_\w+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = declared_functions()
+    assert len(names) >= 10
+    lib = _lib.load()
+    for n in names:
+        assert n in _lib.PROTOTYPES, f"{n} has no ctypes prototype"
+        assert getattr(lib, n) is not None
+    assert sorted(_lib.PROTOTYPES) == names
+
+
+def test_struct_layouts_match_the_header(tmp_path):
+    structs = {"mi355_moe_sorting_args": _lib.SortingArgs, "mi355_fused_moe_traits": _lib.FusedMoeTraits,
+               "mi355_fused_moegemm_args": _lib.FusedMoeGemmArgs, "mi355_fused_moe_args": _lib.FusedMoeArgs}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void){"]
+    for cname, ct in structs.items():
+        lines.append(f'printf("{cname} %zu\\n", sizeof({cname}));')
+        for fname, _ in ct._fields_:
+            lines.append(f'printf("{cname}.{fname} %zu\\n", offsetof({cname}, {fname}));')
+    lines.append("return 0;}")
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", str(src), "-o", str(exe)], check=True)
+    out = dict(l.split() for l in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for cname, ct in structs.items():
+        assert int(out[cname]) == C.sizeof(ct), cname
+        for fname, _ in ct._fields_:
+            assert int(out[f"{cname}.{fname}"]) == getattr(ct, fname).offset, f"{cname}.{fname}"
+
+
+def test_host_only_entry_points():
+    lib = _lib.load()
+    assert lib.mi355_moe_version() == 100
+    assert lib.mi355_moe_max_num_tokens_padded(128, 8, 2, 32) == 2 * 128 + 8 * 32 - 2
+    assert lib.mi355_moe_sorting_workspace_size(64, 128, 8) == 0          # one workgroup, no workspace
+    assert lib.mi355_moe_sorting_workspace_size(32768, 64, 6) >= 384 * 64 * 4
+    t = _lib.FusedMoeTraits(0, 0, 0, 3, 3, 3, 3, 32, 1, 0, 0, 0)
+    assert lib.mi355_fused_moe_supported(C.byref(t)) == 1
+    ws = lib.mi355_fused_moe_workspace_size(C.byref(t), 128, 8, 2, 1024, 1024)
+    assert ws >= 510 * 1024 * 2 + 256 * 1024 * 2
+    bad = _lib.FusedMoeTraits(5, 5, 0, 3, 3, 3, 3, 32, 1, 0, 0, 0)
+    assert lib.mi355_fused_moe_supported(C.byref(bad)) == 0
+    assert lib.mi355_fused_moe_workspace_size(C.byref(bad), 128, 8, 2, 1024, 1024) == 0
+    assert lib.mi355_moe_sorting(None, None) == _lib.E_INVALID and b"null" in lib.mi355_moe_last_error()
+    assert lib.mi355_fused_moe(None, None, None) == _lib.E_INVALID
+
+
+def test_python_mirror_rejects_unknown_traits_without_touching_the_gpu():
+    import therock_amd as ta
+    assert ta.fused_moe(ta.fused_moe_traits(prec_i="fp16", prec_w="fp16"), ta.fused_moe_args()) == -1.0
+    with pytest.raises(ValueError):
+        ta.fused_moe_traits(prec_i="fp4").pod()

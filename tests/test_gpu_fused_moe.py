@@ -1,0 +1,128 @@
+"""GPU parity of mi355_fused_moe / mi355_fused_moegemm against the oracle.
+
+Tolerances are the ones the build targets: rel-L2 <= 1e-2 for bf16, <= 3e-2 for fp8 and int8
+(fp32 accumulation in both GEMMs; the intermediate activations are stored in bf16, or block-scaled
+e4m3 on the fp8 path, which the oracle keeps in fp32)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from therock_amd import inputs as mi
+
+pytestmark = pytest.mark.gpu
+
+DT = {"bf16": oracle.DT_BF16, "fp8": oracle.DT_E4M3, "int8": oracle.DT_I8}
+TOL = {"bf16": 1e-2, "fp8": 3e-2, "int8": 3e-2}
+
+
+def oracle_out(cfg, inp, mask=None):
+    s = oracle.moe_sorting(inp["topk_ids"], inp["topk_weight"], cfg.experts, cfg.unit, local_expert_mask=mask)
+    dt = DT[cfg.dtype]
+    o = oracle.fused_moe(inp["a"], dt, inp["g"], dt, inp["d"], dt, *s, cfg.unit, cfg.tokens, inp["g"].shape[0],
+                         cfg.hidden, cfg.inter, cfg.topk, a_scale=inp["a_scale"], g_scale=inp["g_scale"],
+                         d_scale=inp["d_scale"])
+    return oracle.bf16_to_f32(o), s
+
+
+def check(cfg, seed=0, mask=None, **kw):
+    from tests.gpu_util import rel_l2, run_fused_moe
+    inp = mi.make_inputs_np(cfg, seed)
+    if mask is not None:  # weights of the local experts only, indexed by local id
+        nloc = int(mask.sum())
+        for k in ("g", "d", "g_scale", "d_scale"):
+            if inp[k] is not None:
+                inp[k] = inp[k][:nloc]
+    print(f"fused_moe {cfg} seed={seed} mask={mask is not None} {kw}", flush=True)
+    got, buf = run_fused_moe(cfg, inp, mask=mask, **kw)
+    ref, s = oracle_out(cfg, inp, mask)
+    pp = s[3]
+    assert int(buf.total[0]) == pp
+    assert np.array_equal(buf.sorted_ids[:pp].cpu().numpy(), s[0][:pp])
+    assert np.array_equal(buf.sorted_eid[:pp // cfg.unit].cpu().numpy(), s[2][:pp // cfg.unit])
+    err = rel_l2(oracle.bf16_to_f32(got), ref)
+    print(f"  rel-L2 = {err:.3e} (tolerance {TOL[cfg.dtype]:.0e})", flush=True)
+    assert np.all(np.isfinite(oracle.bf16_to_f32(got)))
+    assert err <= TOL[cfg.dtype]
+    return err
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "int8", "fp8"])
+def test_small_single_tile(dtype):
+    # one expert tile, one K tile pair: the smallest problem that touches every code path
+    check(mi.MoeConfig("s", 8, 128, 128, 4, 2, dtype, "softmax_renorm"))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "int8", "fp8"])
+def test_medium_multi_tile(dtype):
+    check(mi.MoeConfig("m", 300, 512, 384, 8, 2, dtype, "softmax_renorm"))
+    check(mi.MoeConfig("m", 48, 512, 256, 16, 4, dtype, "sigmoid_renorm"))
+
+
+def test_cfg1_against_oracle_and_ck_golden(golden_dir):
+    from tests.gpu_util import rel_l2, run_fused_moe
+    cfg = mi.CONFIGS["cfg1_cpu_ref_bf16"]
+    check(cfg)
+    g = np.load(os.path.join(golden_dir, "cfg1_ck_reference.npz"))
+    got, buf = run_fused_moe(cfg, mi.make_inputs_np(cfg, 0))
+    pp = int(g["post_pad"])
+    assert np.array_equal(buf.sorted_ids[:pp].cpu().numpy(), g["sorted_ids"])
+    assert np.array_equal(buf.sorted_w[:pp].cpu().numpy(), g["sorted_w"])
+    assert rel_l2(oracle.bf16_to_f32(got), oracle.bf16_to_f32(g["out_bf16"])) <= 1e-2
+
+
+@pytest.mark.parametrize("key", ["fp8", "int8"])
+def test_small_quantised_against_ck_golden(key, golden_dir):
+    from tests.golden.make_golden import SMALL_QUANT
+    from tests.gpu_util import rel_l2, run_fused_moe
+    g = np.load(os.path.join(golden_dir, "small_quant_ck_reference.npz"))
+    cfg = SMALL_QUANT[key]
+    got, _ = run_fused_moe(cfg, mi.make_inputs_np(cfg, 0))
+    assert rel_l2(oracle.bf16_to_f32(got), oracle.bf16_to_f32(g[f"{key}_out_bf16"])) <= 3e-2
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
+def test_ragged_shapes_and_units(dtype):
+    # intermediate not a multiple of the 128-column tile, hidden not a multiple of 256, odd counts
+    inter = 384 if dtype == "fp8" else 416
+    check(mi.MoeConfig("r", 77, 320, inter, 12, 3, dtype, "softmax_renorm", unit=32), seed=3)
+    check(mi.MoeConfig("r", 130, 1152, 256, 6, 2, dtype, "softmax_renorm", unit=64), seed=4)
+    check(mi.MoeConfig("r", 200, 256, 128, 3, 1, dtype, "softmax_renorm", unit=128), seed=5)
+    check(mi.MoeConfig("r", 50, 256, 128, 16, 4, dtype, "softmax", unit=16), seed=6)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
+def test_local_expert_mask_and_unfused_entry(dtype):
+    cfg = mi.MoeConfig("e", 96, 256, 256, 10, 3, dtype, "softmax_renorm")
+    mask = (np.arange(cfg.experts) % 3 != 1).astype(np.int32)
+    check(cfg, seed=7, mask=mask)
+    check(cfg, seed=7, unfused=True)
+    check(cfg, seed=8, stride_pad=64)
+
+
+def test_skewed_routing_with_empty_experts():
+    check(mi.MoeConfig("z", 3000, 256, 128, 64, 6, "bf16", "zipf"), seed=2)
+
+
+def test_decode_shapes_int8():
+    for T in (16, 64):
+        check(mi.CONFIGS["cfg4_decode_int8_t64"].scaled(tokens=T, hidden=1024, inter=512))
+
+
+def test_traits_without_kernel_return_minus_one():
+    import torch
+    import therock_amd as ta
+    for kw in (dict(prec_i="fp16", prec_w="fp16"), dict(activation=0), dict(gate_only=1), dict(prec_o="fp32")):
+        assert ta.fused_moe(ta.fused_moe_traits(**kw), ta.fused_moe_args()) == -1.0
+    t = ta.fused_moe_traits()
+    buf = ta.MoeBuffers(t, 4, 4, 2, 128, 128, "cuda")
+    a = torch.zeros((4, 128), dtype=torch.bfloat16, device="cuda")
+    g = torch.zeros((4, 256, 128), dtype=torch.bfloat16, device="cuda")
+    d = torch.zeros((4, 128, 128), dtype=torch.bfloat16, device="cuda")
+    ids = torch.zeros((4, 2), dtype=torch.int32, device="cuda")
+    w = torch.zeros((4, 2), dtype=torch.float32, device="cuda")
+    args = ta.make_args(t, buf, a, g, d, ids, w)
+    args.ws_ptr = None
+    with pytest.raises(RuntimeError, match="workspace"):
+        ta.fused_moe(t, args)

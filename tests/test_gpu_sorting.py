@@ -1,0 +1,94 @@
+"""GPU parity of mi355_moe_sorting against the oracle (bit-exact on the written prefix, untouched
+cells beyond it), through the C ABI."""
+import hashlib
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from therock_amd import inputs as mi
+
+pytestmark = pytest.mark.gpu
+
+
+def routing(cfg, seed=1000):
+    rng = np.random.Generator(np.random.Philox(seed))
+    return mi.route_np(rng.standard_normal((cfg.tokens, cfg.experts), dtype=np.float32), cfg.topk, cfg.router)
+
+
+def check(ids, w, experts, unit, mask=None, local_tokens=None):
+    from tests.gpu_util import run_sorting
+    got = run_sorting(ids, w, experts, unit, mask=mask, local_tokens=local_tokens)
+    T = ids.shape[0] if local_tokens is None else local_tokens
+    ref = oracle.moe_sorting(ids[:T], w[:T], experts, unit, local_expert_mask=mask)
+    pp = ref[3]
+    print(f"sorting T={T} K={ids.shape[1]} E={experts} U={unit} post_pad={pp}", flush=True)
+    assert got[3][0] == pp and got[3][1] == T
+    assert np.array_equal(got[0][:pp], ref[0][:pp])
+    assert np.array_equal(got[1][:pp], ref[1][:pp])
+    assert np.array_equal(got[2][:pp // unit], ref[2][:pp // unit])
+    assert np.all(got[0][pp:] == -1) and np.all(got[1][pp:] == -1.0) and np.all(got[2][pp // unit:] == -1)
+    return got
+
+
+def test_header_examples(golden_dir):
+    g = np.load(os.path.join(golden_dir, "sorting_header_examples.npz"))
+    got = check(g["topk_ids"], g["topk_weight"], 6, 4)
+    assert np.array_equal(got[0][:24], g["skip_ids"]) and np.array_equal(got[2][:6], g["skip_eid"])
+    got = check(g["topk_ids"], g["topk_weight"], 6, 4, mask=np.array([1, 0, 1, 1, 0, 1]))
+    assert np.array_equal(got[0][:20], g["mask_ids"]) and np.array_equal(got[2][:5], g["mask_eid"])
+
+
+@pytest.mark.parametrize("name", list(mi.CONFIGS))
+@pytest.mark.parametrize("unit", [32, 64, 128])
+def test_benchmark_routings_match_oracle_and_golden(name, unit, golden_dir):
+    cfg = mi.CONFIGS[name]
+    ids, w = routing(cfg)
+    got = check(ids, w, cfg.experts, unit)
+    h = json.load(open(os.path.join(golden_dir, "sorting_hashes.json")))[f"{name}/u{unit}"]
+    pp = h["post_pad"]
+    sha = lambda a: hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+    assert (sha(got[0][:pp]), sha(got[1][:pp]), sha(got[2][:pp // unit])) == (h["ids"], h["w"], h["eid"])
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_shapes_masks_and_local_tokens(seed):
+    rng = np.random.default_rng(seed)
+    E = int(rng.choice([1, 2, 7, 64, 100, 256, 257, 1024]))
+    K = int(rng.integers(1, min(E, 8) + 1))
+    T = int(rng.choice([1, 3, 65, 513, 3000, 9000]))
+    U = int(rng.choice([1, 16, 32, 48]))
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
+    w = rng.random((T, K), dtype=np.float32)
+    check(ids, w, E, U)
+    check(ids, w, E, U, mask=(rng.random(E) < 0.5).astype(np.int32))
+    check(ids, w, E, U, local_tokens=int(rng.integers(0, T + 1)))
+
+
+def test_empty_and_skew():
+    check(np.zeros((0, 2), np.int32), np.zeros((0, 2), np.float32), 8, 32)
+    # every token picks the same experts: one giant bucket, the rest empty
+    T = 20000
+    ids = np.tile(np.array([[5, 2]], dtype=np.int32), (T, 1))
+    check(ids, np.ones((T, 2), np.float32), 64, 32)
+
+
+def test_moe_buf_is_zeroed():
+    from tests.gpu_util import run_sorting
+    for T, E, K in ((64, 128, 8), (8192, 256, 8)):
+        cfg = mi.MoeConfig("z", T, 0, 0, E, K, "bf16", "softmax")
+        ids, w = routing(cfg, 5)
+        buf = torch.full((T + 3, 1032), 7.0, dtype=torch.bfloat16, device="cuda")
+        run_sorting(ids, w, E, 32, moe_buf=buf[:T])
+        assert torch.all(buf[:T] == 0) and torch.all(buf[T:] == 7.0)
+
+
+def test_invalid_arguments_are_rejected():
+    import therock_amd as ta
+    a = ta.moe_sorting_args(tokens=4, unit_size=32, num_experts=8, topk=2)
+    with pytest.raises(RuntimeError, match="null"):
+        ta.moe_sorting(ta.moe_sorting_trait(), a)
+    assert ta.moe_sorting(ta.moe_sorting_trait(index_type="int64"), a) == -1.0

@@ -1,0 +1,93 @@
+"""Loader and ctypes prototypes of libmi355_moe.so (the C ABI declared in include/mi355_moe.h).
+
+The library is built in-tree by ``therock_amd.build`` (hipcc, gfx950).  There is no fallback: if
+it is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi355_moe.so")
+
+OK, E_UNSUPPORTED, E_INVALID, E_HIP, E_WORKSPACE = 0, -1, -2, -3, -4
+DTYPES = {"bf16": 0, "fp8": 1, "int8": 2, "fp32": 3, "int32": 4, "fp16": 5}
+
+
+class SortingArgs(C.Structure):
+    _fields_ = [
+        ("p_topk_ids", C.c_void_p), ("p_weights", C.c_void_p), ("p_local_expert_mask", C.c_void_p),
+        ("p_local_tokens", C.c_void_p), ("p_sorted_token_ids", C.c_void_p), ("p_sorted_weights", C.c_void_p),
+        ("p_sorted_expert_ids", C.c_void_p), ("p_total_tokens_post_pad", C.c_void_p), ("p_moe_buf", C.c_void_p),
+        ("p_ws", C.c_void_p), ("tokens", C.c_int32), ("unit_size", C.c_int32), ("num_experts", C.c_int32),
+        ("topk", C.c_int32), ("moe_buf_interm_dim", C.c_int32), ("moe_buf_elem_bytes", C.c_int32),
+    ]
+
+
+class FusedMoeTraits(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "prec_i", "prec_w", "prec_o", "prec_st", "prec_sw", "prec_sq", "prec_kw", "block_m", "activation",
+        "gate_only", "fused_quant", "local_expert_masking")]
+
+
+class FusedMoeGemmArgs(C.Structure):
+    _fields_ = [
+        ("a_ptr", C.c_void_p), ("a_scale_ptr", C.c_void_p), ("g_ptr", C.c_void_p), ("d_ptr", C.c_void_p),
+        ("g_scale_ptr", C.c_void_p), ("d_scale_ptr", C.c_void_p), ("y_smooth_scale_ptr", C.c_void_p),
+        ("o_ptr", C.c_void_p), ("sorted_token_ids_ptr", C.c_void_p), ("sorted_weight_ptr", C.c_void_p),
+        ("sorted_expert_ids_ptr", C.c_void_p), ("num_sorted_tiles_ptr", C.c_void_p), ("ws_ptr", C.c_void_p),
+        ("ws_bytes", C.c_size_t), ("hidden_size", C.c_int32), ("intermediate_size", C.c_int32),
+        ("num_tokens", C.c_int32), ("num_experts", C.c_int32), ("topk", C.c_int32), ("stride_token", C.c_int32),
+    ]
+
+
+class FusedMoeArgs(C.Structure):
+    _fields_ = [
+        ("a_ptr", C.c_void_p), ("a_scale_ptr", C.c_void_p), ("g_ptr", C.c_void_p), ("d_ptr", C.c_void_p),
+        ("g_scale_ptr", C.c_void_p), ("d_scale_ptr", C.c_void_p), ("y_smooth_scale_ptr", C.c_void_p),
+        ("local_expert_mask_ptr", C.c_void_p), ("o_ptr", C.c_void_p), ("ws_ptr", C.c_void_p),
+        ("ws_bytes", C.c_size_t), ("topk_ids_ptr", C.c_void_p), ("topk_weight_ptr", C.c_void_p),
+        ("sorted_token_ids_ptr", C.c_void_p), ("sorted_weight_ptr", C.c_void_p),
+        ("sorted_expert_ids_ptr", C.c_void_p), ("num_sorted_tiles_ptr", C.c_void_p), ("block_m", C.c_int32),
+        ("hidden_size", C.c_int32), ("intermediate_size", C.c_int32), ("num_tokens", C.c_int32),
+        ("num_experts", C.c_int32), ("topk", C.c_int32), ("stride_token", C.c_int32),
+    ]
+
+
+# every symbol include/mi355_moe.h declares: name -> (restype, argtypes)
+PROTOTYPES = {
+    "mi355_moe_max_num_tokens_padded": (C.c_int64, [C.c_int32] * 4),
+    "mi355_moe_sorting_workspace_size": (C.c_size_t, [C.c_int32] * 3),
+    "mi355_moe_sorting": (C.c_int, [C.POINTER(SortingArgs), C.c_void_p]),
+    "mi355_fused_moe_supported": (C.c_int, [C.POINTER(FusedMoeTraits)]),
+    "mi355_fused_moe_workspace_size": (C.c_size_t, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
+    "mi355_fused_moegemm": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeGemmArgs), C.c_void_p]),
+    "mi355_fused_moe": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.c_void_p]),
+    "mi355_moe_rowwise_quant": (C.c_int, [C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_int32, C.c_void_p,
+                                          C.c_void_p, C.c_void_p]),
+    "mi355_moe_last_error": (C.c_char_p, []),
+    "mi355_moe_version": (C.c_int, []),
+}
+
+_lib = None
+
+
+def load():
+    """dlopen the HIP library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m therock_amd.build` (needs hipcc); "
+                "there is no CPU fallback")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().mi355_moe_last_error().decode()

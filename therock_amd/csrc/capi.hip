@@ -1,0 +1,162 @@
+// extern "C" surface of libmi355_moe.so: argument checking, workspace carving, launches.
+#include "common.hpp"
+#include "moe_gemm.hpp"
+
+#include <cstring>
+#include <mutex>
+
+namespace mi355 {
+
+char* error_buffer()
+{
+    static thread_local char buf[512] = {0};
+    return buf;
+}
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(error_buffer(), 512, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+const DeviceInfo& device_info()
+{
+    constexpr int kMaxDev = 64;
+    static DeviceInfo info[kMaxDev];
+    static std::once_flag once[kMaxDev];
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if(dev < 0 || dev >= kMaxDev)
+        dev = 0;
+    std::call_once(once[dev], [dev] {
+        int v = 0;
+        info[dev].num_cu = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0 ? v : 256;
+        info[dev].max_lds = hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && v > 0 ? v : 65536;
+    });
+    return info[dev];
+}
+
+} // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+__attribute__((visibility("default"))) const char* mi355_moe_last_error(void) { return error_buffer(); }
+
+__attribute__((visibility("default"))) int mi355_moe_version(void) { return MI355_MOE_VERSION; }
+
+__attribute__((visibility("default"))) int64_t
+mi355_moe_max_num_tokens_padded(int32_t tokens, int32_t num_experts, int32_t topk, int32_t unit_size)
+{
+    return (int64_t)topk * tokens + (int64_t)num_experts * unit_size - topk;
+}
+
+__attribute__((visibility("default"))) size_t
+mi355_moe_sorting_workspace_size(int32_t tokens, int32_t num_experts, int32_t topk)
+{
+    return sorting_workspace_bytes(tokens, num_experts, topk);
+}
+
+__attribute__((visibility("default"))) int mi355_moe_sorting(const mi355_moe_sorting_args* args, void* stream)
+{
+    if(args == nullptr)
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: args is null");
+    return launch_moe_sorting(*args, static_cast<hipStream_t>(stream));
+}
+
+__attribute__((visibility("default"))) int mi355_fused_moe_supported(const mi355_fused_moe_traits* t)
+{
+    return t != nullptr && check_traits(*t) == MI355_MOE_OK ? 1 : 0;
+}
+
+__attribute__((visibility("default"))) size_t
+mi355_fused_moe_workspace_size(const mi355_fused_moe_traits* traits, int32_t tokens, int32_t num_experts,
+                               int32_t topk, int32_t hidden_size, int32_t intermediate_size)
+{
+    if(traits == nullptr || check_traits(*traits) != MI355_MOE_OK)
+        return 0;
+    return workspace_layout(*traits, tokens, num_experts, topk, hidden_size, intermediate_size).total;
+}
+
+__attribute__((visibility("default"))) int
+mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_moegemm_args* args, void* stream)
+{
+    if(traits == nullptr || args == nullptr)
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: traits or args is null");
+    return launch_fused_moegemm(*traits, *args, static_cast<hipStream_t>(stream));
+}
+
+__attribute__((visibility("default"))) int
+mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* a, void* stream)
+{
+    if(traits == nullptr || a == nullptr)
+        return fail(MI355_MOE_E_INVALID, "fused_moe: traits or args is null");
+    int rc = check_traits(*traits);
+    if(rc != MI355_MOE_OK)
+        return rc;
+    if(a->block_m != traits->block_m)
+        return fail(MI355_MOE_E_INVALID, "fused_moe: args.block_m=%d differs from traits.block_m=%d",
+                    a->block_m, traits->block_m);
+    const WorkspaceLayout ws = workspace_layout(*traits, a->num_tokens, a->num_experts, a->topk,
+                                                a->hidden_size, a->intermediate_size);
+    if(a->ws_ptr == nullptr || a->ws_bytes < ws.total)
+        return fail(MI355_MOE_E_WORKSPACE, "fused_moe: workspace of %zu bytes needed, %zu given", ws.total,
+                    a->ws_ptr ? a->ws_bytes : (size_t)0);
+
+    // the combine writes every element of o, so the sort does not need to zero it
+    mi355_moe_sorting_args s{};
+    s.p_topk_ids              = a->topk_ids_ptr;
+    s.p_weights               = a->topk_weight_ptr;
+    s.p_local_expert_mask     = traits->local_expert_masking ? a->local_expert_mask_ptr : nullptr;
+    s.p_local_tokens          = nullptr;
+    s.p_sorted_token_ids      = a->sorted_token_ids_ptr;
+    s.p_sorted_weights        = a->sorted_weight_ptr;
+    s.p_sorted_expert_ids     = a->sorted_expert_ids_ptr;
+    s.p_total_tokens_post_pad = a->num_sorted_tiles_ptr;
+    s.p_moe_buf               = nullptr;
+    s.p_ws                    = static_cast<char*>(a->ws_ptr) + ws.sort_off;
+    s.tokens                  = a->num_tokens;
+    s.unit_size               = a->block_m;
+    s.num_experts             = a->num_experts;
+    s.topk                    = a->topk;
+    if(traits->local_expert_masking && a->local_expert_mask_ptr == nullptr)
+        return fail(MI355_MOE_E_INVALID, "fused_moe: local_expert_masking set but mask pointer is null");
+    rc = launch_moe_sorting(s, static_cast<hipStream_t>(stream));
+    if(rc != MI355_MOE_OK)
+        return rc;
+
+    mi355_fused_moegemm_args g{};
+    g.a_ptr                 = a->a_ptr;
+    g.a_scale_ptr           = a->a_scale_ptr;
+    g.g_ptr                 = a->g_ptr;
+    g.d_ptr                 = a->d_ptr;
+    g.g_scale_ptr           = a->g_scale_ptr;
+    g.d_scale_ptr           = a->d_scale_ptr;
+    g.y_smooth_scale_ptr    = a->y_smooth_scale_ptr;
+    g.o_ptr                 = a->o_ptr;
+    g.sorted_token_ids_ptr  = a->sorted_token_ids_ptr;
+    g.sorted_weight_ptr     = a->sorted_weight_ptr;
+    g.sorted_expert_ids_ptr = a->sorted_expert_ids_ptr;
+    g.num_sorted_tiles_ptr  = a->num_sorted_tiles_ptr;
+    g.ws_ptr                = a->ws_ptr;
+    g.ws_bytes              = a->ws_bytes;
+    g.hidden_size           = a->hidden_size;
+    g.intermediate_size     = a->intermediate_size;
+    g.num_tokens            = a->num_tokens;
+    g.num_experts           = a->num_experts;
+    g.topk                  = a->topk;
+    g.stride_token          = a->stride_token;
+    return launch_fused_moegemm(*traits, g, static_cast<hipStream_t>(stream));
+}
+
+__attribute__((visibility("default"))) int
+mi355_moe_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype, void* q,
+                        void* scale, void* stream)
+{
+    return launch_rowwise_quant(x, rows, cols, stride_x, q_dtype, q, scale, static_cast<hipStream_t>(stream));
+}
+}

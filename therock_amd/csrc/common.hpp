@@ -1,0 +1,60 @@
+// Shared host/device helpers of libmi355_moe.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/mi355_moe.h"
+
+namespace mi355 {
+
+constexpr int kWave = 64;
+
+// thread-local error text behind mi355_moe_last_error()
+char* error_buffer();
+int fail(int code, const char* fmt, ...);
+
+#define MI355_HIP_TRY(expr)                                                                   \
+    do                                                                                        \
+    {                                                                                         \
+        hipError_t e_ = (expr);                                                               \
+        if(e_ != hipSuccess)                                                                  \
+            return ::mi355::fail(MI355_MOE_E_HIP, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+    } while(0)
+
+template <typename T>
+__host__ __device__ constexpr T ceil_div(T a, T b)
+{
+    return (a + b - 1) / b;
+}
+
+template <typename T>
+__host__ __device__ constexpr T round_up(T a, T b)
+{
+    return ceil_div(a, b) * b;
+}
+
+// token | slot << 24, the id format of ck_tile's moe_sorting (moe_sorting_kernel.hpp:78-80)
+__host__ __device__ inline int32_t mock_id(int32_t token, int32_t slot)
+{
+    return static_cast<int32_t>((static_cast<uint32_t>(token) & 0x00ffffffu) |
+                                ((static_cast<uint32_t>(slot) & 0xffu) << 24));
+}
+
+struct DeviceInfo
+{
+    int num_cu;
+    int max_lds;
+};
+// cached per device (ck_tile queries hipGetDeviceProperties on every call)
+const DeviceInfo& device_info();
+
+// ---- sorting launcher shared by the stand-alone and the fused entry points
+// tile_* (optional, may be null): work list for the grouped GEMMs, built by the sort's scan
+int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream);
+
+size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk);
+
+} // namespace mi355

@@ -1,0 +1,74 @@
+// Device-side helpers shared by the sorting and GEMM kernels (gfx950, wave64).
+#pragma once
+
+#include "common.hpp"
+
+namespace mi355 {
+
+__device__ inline void wave_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Exclusive scan of one int per thread over a block of NWAVES*64 threads.  s_wave needs
+// NWAVES+1 ints of LDS.  Every thread of the block must call it; `total` gets the block sum.
+template <int NWAVES>
+__device__ inline int block_exclusive_scan(int v, int* s_wave, int& total)
+{
+    static_assert(NWAVES <= kWave, "one wave scans the wave totals");
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    int x          = v;
+#pragma unroll
+    for(int d = 1; d < kWave; d <<= 1)
+    {
+        const int y = __shfl_up(x, d);
+        if(lane >= d)
+            x += y;
+    }
+    if(lane == kWave - 1)
+        s_wave[wave] = x;
+    __syncthreads();
+    if(wave == 0)
+    {
+        const int w = lane < NWAVES ? s_wave[lane] : 0;
+        int xx      = w;
+#pragma unroll
+        for(int d = 1; d < NWAVES; d <<= 1)
+        {
+            const int y = __shfl_up(xx, d);
+            if(lane >= d)
+                xx += y;
+        }
+        if(lane < NWAVES)
+            s_wave[lane] = xx - w;
+        if(lane == NWAVES - 1)
+            s_wave[NWAVES] = xx;
+    }
+    __syncthreads();
+    const int r = s_wave[wave] + x - v;
+    total       = s_wave[NWAVES];
+    __syncthreads();
+    return r;
+}
+
+__device__ inline float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
+
+// round-to-nearest-even float -> bf16 bits (NaN stays NaN)
+__device__ inline uint32_t float_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if((u & 0x7fffffffu) > 0x7f800000u)
+        return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+__device__ inline uint32_t pack_bf16x2(float lo, float hi)
+{
+    return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
+}
+
+} // namespace mi355

@@ -1,0 +1,860 @@
+// Grouped GEMMs of the fused-MoE path for gfx950 (CDNA4, wave64, MFMA 32x32).
+//
+// Replaces ck_tile's FusedMoeGemmKernel + FusedMoeGemmPipeline_FlatmmUk
+// (ops/fused_moe/kernel/fused_moegemm_kernel.hpp:238-259,
+//  ops/fused_moe/pipeline/fused_moegemm_pipeline_flatmm_uk.hpp:169-416); numerics follow
+// ck_tile::reference_fused_moe (host/reference/reference_fused_moe.hpp:42-204).
+//
+// Instead of ck_tile's single kernel (32 sorted rows x 512 intermediate columns per workgroup,
+// bf16 atomics into the output) the path is three launches over a tile list built from the sort:
+//   gemm0  Y[row, n]   = silu(x . Wgate[n]) * (x . Wup[n])      (gather rows by sorted token id)
+//   gemm1  P[t*K+k, h] = (Y[row] . Wdown[h]) * topk_weight      (bf16 partial per (token, slot))
+//   combine O[t, h]    = sum_k P[t*K+k, h]  in slot order, fp32, one rounding to bf16
+// A workgroup (4 waves) owns up to MBLK*32 sorted rows of ONE expert and 256 weight rows
+// (gemm0: 128 gate + 128 up rows = 128 Y columns).  The MFMA's M side is the weight rows and its
+// N side the tokens, so every lane ends up with 16 consecutive output channels of one token and
+// the SiLU*up, the scales and the packing all happen in registers.  All four waves share the
+// token tile and split the weight rows, which keeps the waves balanced for any number of rows.
+// Operand tiles are staged through LDS (16-byte padded rows, conflict-free ds_read_b128) with the
+// next K tile prefetched into registers while the current one feeds the MFMAs.
+#include "moe_gemm.hpp"
+#include "device_utils.hpp"
+
+#include <algorithm>
+
+namespace mi355 {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(16))) int i32x16_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+
+enum Mode
+{
+    kBf16   = 0, // x bf16, w bf16, bf16 MFMA
+    kFp8    = 1, // x e4m3, w e4m3, block-scaled f8f6f4 MFMA
+    kI8     = 2, // x int8, w int8, i8 MFMA (gemm0 only)
+    kBf16W8 = 3  // x bf16, w int8 converted to bf16 after the LDS read (gemm1 of the int8 path)
+};
+
+constexpr int kBlock   = 256;
+constexpr int kWRows   = 256; // weight rows per workgroup tile
+constexpr int kTileKB  = 128; // bytes of K per row of the x tile
+constexpr int kPadB    = 16;
+constexpr int kMapHdr  = 4;   // ints in front of the tile entries
+constexpr int kMapEnt  = 8;   // ints per tile entry: expert,row0,nrows,first,ntiles,0,0,0
+
+struct GemmParams
+{
+    const unsigned char* x;  // gemm0: activations [tokens, x_row_bytes]; gemm1: Y [rows, x_row_bytes]
+    const unsigned char* w;  // [experts, n_total, k] K contiguous
+    const float* x_scale;    // gemm0: per-token scale or null
+    const float* w_scale;    // [experts, n_total] or null
+    const int* sorted_ids;
+    const float* sorted_w;
+    const int* tile_map;
+    unsigned char* out;      // gemm0: Y; gemm1: P
+    unsigned char* y_scale;  // e8m0 block scales of Y (fp8 path): written by gemm0, read by gemm1
+    int* valid;              // gemm1: flags per (token, slot)
+    int64_t x_row_bytes;
+    int64_t w_row_bytes;
+    int64_t w_expert_bytes;
+    int64_t out_row_bytes;
+    int64_t ys_row_bytes;
+    int k_bytes_x;           // bytes of K in a row of x
+    int k_bytes_w;           // bytes of K in a row of w
+    int n_out;               // gemm0: inter; gemm1: hidden
+    int n_total;             // weight rows per expert (gemm0: 2*inter, gemm1: hidden)
+    int n_ntiles;            // tiles along n
+    int tokens;
+    int topk;
+};
+
+template <int MODE>
+struct ModeTraits;
+template <>
+struct ModeTraits<kBf16>
+{
+    using Acc                  = f32x16_t;
+    static constexpr int kOpB  = 16; // operand bytes per lane per MFMA
+    static constexpr int kWKB  = 128;
+};
+template <>
+struct ModeTraits<kFp8>
+{
+    using Acc                  = f32x16_t;
+    static constexpr int kOpB  = 32;
+    static constexpr int kWKB  = 128;
+};
+template <>
+struct ModeTraits<kI8>
+{
+    using Acc                  = i32x16_t;
+    static constexpr int kOpB  = 16;
+    static constexpr int kWKB  = 128;
+};
+template <>
+struct ModeTraits<kBf16W8>
+{
+    using Acc                  = f32x16_t;
+    static constexpr int kOpB  = 16;
+    static constexpr int kWKB  = 64; // int8 weights: 64 K elements per tile row
+};
+
+// MFMA row m of a 32-row weight block holds weight channel chan_of_row(m); with the 32x32
+// accumulator layout (register v = 4j+i of lane l is row 8j + 4(l/32) + i) lane l then owns the 16
+// consecutive channels 16*(l/32) .. +15 of its token in registers 0..15.
+__device__ __host__ constexpr int chan_of_row(int m) { return 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3); }
+
+__device__ inline float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+
+// 8 int8 (two dwords) -> 8 bf16 (exact: |v| <= 128 fits bf16's 8 significant bits)
+__device__ inline uint4 int8x8_to_bf16x8(uint2 v)
+{
+    uint4 r;
+    uint32_t d[2] = {v.x, v.y};
+    uint32_t o[4];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+    {
+        const int s = static_cast<int>(d[h]);
+        const uint32_t f0 = __float_as_uint(static_cast<float>((s << 24) >> 24));
+        const uint32_t f1 = __float_as_uint(static_cast<float>((s << 16) >> 24));
+        const uint32_t f2 = __float_as_uint(static_cast<float>((s << 8) >> 24));
+        const uint32_t f3 = __float_as_uint(static_cast<float>(s >> 24));
+        o[2 * h]     = (f1 & 0xffff0000u) | (f0 >> 16);
+        o[2 * h + 1] = (f3 & 0xffff0000u) | (f2 >> 16);
+    }
+    r.x = o[0];
+    r.y = o[1];
+    r.z = o[2];
+    r.w = o[3];
+    return r;
+}
+
+template <typename To, typename From>
+__device__ inline To bit_cast_dev(const From& f)
+{
+    static_assert(sizeof(To) == sizeof(From), "size mismatch");
+    To t;
+    __builtin_memcpy(&t, &f, sizeof(To));
+    return t;
+}
+
+struct Frag
+{
+    uint4 lo, hi; // hi only used by 32-byte operands
+};
+
+template <int MODE>
+__device__ inline typename ModeTraits<MODE>::Acc mfma(const Frag& w, const Frag& x, uint32_t x_scale,
+                                                      typename ModeTraits<MODE>::Acc c)
+{
+    if constexpr(MODE == kBf16 || MODE == kBf16W8)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(bit_cast_dev<bf16x8_t>(w.lo), bit_cast_dev<bf16x8_t>(x.lo), c,
+                                                       0, 0, 0);
+    }
+    else if constexpr(MODE == kI8)
+    {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(bit_cast_dev<i32x4_t>(w.lo), bit_cast_dev<i32x4_t>(x.lo), c, 0,
+                                                     0, 0);
+    }
+    else
+    {
+        i32x8_t a, b;
+        a[0] = w.lo.x; a[1] = w.lo.y; a[2] = w.lo.z; a[3] = w.lo.w;
+        a[4] = w.hi.x; a[5] = w.hi.y; a[6] = w.hi.z; a[7] = w.hi.w;
+        b[0] = x.lo.x; b[1] = x.lo.y; b[2] = x.lo.z; b[3] = x.lo.w;
+        b[4] = x.hi.x; b[5] = x.hi.y; b[6] = x.hi.z; b[7] = x.hi.w;
+        // cbsz = blgp = 0: both operands e4m3; weights carry the unit block scale 2^0 (e8m0 127),
+        // the token operand its per-32 block scale in byte 0 (op_sel 0)
+        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 127, 0, static_cast<int>(x_scale));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// GEMM0 : MODE in {kBf16, kFp8, kI8};  GEMM1 : MODE in {kBf16, kFp8, kBf16W8}
+template <int MODE, bool GEMM0, int MBLK>
+__global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
+{
+    using MT  = ModeTraits<MODE>;
+    using Acc = typename MT::Acc;
+    constexpr int kOpB     = MT::kOpB;
+    constexpr int kWKB     = MT::kWKB;
+    constexpr int kXStride = kTileKB + kPadB;
+    constexpr int kWStride = kWKB + kPadB;
+    constexpr int kSteps   = kTileKB / (2 * kOpB); // MFMAs along K per tile
+    constexpr int kWChunks = kWKB / 16;            // 16-byte chunks per weight tile row
+    constexpr int kWLoads  = kWRows * kWChunks / kBlock;
+    constexpr int kWRowsPerPass = kBlock / kWChunks;
+    constexpr bool kMx     = MODE == kFp8 && !GEMM0; // token operand carries e8m0 block scales
+
+    extern __shared__ __align__(16) unsigned char lds[];
+    unsigned char* lds_w = lds;
+    unsigned char* lds_x = lds + kWRows * kWStride;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int r32  = lane & 31;
+    const int kg   = lane >> 5;
+
+    // ---- work item: XCD x gets a contiguous range of the work list (workgroup ids are dealt
+    // round-robin to the 8 XCDs), and inside an expert the M tiles of one weight tile are adjacent
+    const int live_tiles = p.tile_map[0];
+    const int total      = live_tiles * p.n_ntiles;
+    const int per_xcd    = ceil_div(total, 8);
+    const int slot       = blockIdx.x >> 3;
+    const int work       = (blockIdx.x & 7) * per_xcd + slot;
+    if(slot >= per_xcd || work >= total)
+        return;
+    int mt, nt;
+    {
+        const int t0     = work / p.n_ntiles;
+        const int* ent0  = p.tile_map + kMapHdr + t0 * kMapEnt;
+        const int first  = ent0[3];
+        const int ntiles = ent0[4];
+        const int rel    = work - first * p.n_ntiles;
+        nt               = rel / ntiles;
+        mt               = first + (rel - nt * ntiles);
+    }
+    const int* ent   = p.tile_map + kMapHdr + mt * kMapEnt;
+    const int expert = ent[0];
+    const int row0   = ent[1];
+    const int nrows  = ent[2];
+    const int nmb    = ceil_div(nrows, 32);
+
+    // ---- global -> register staging assignments
+    const int xchunk = tid & 7;
+    const int xrow   = tid >> 3; // + 32*j
+    const unsigned char* xptr[MBLK];
+    bool xvalid[MBLK];
+#pragma unroll
+    for(int j = 0; j < MBLK; j++)
+    {
+        const int r = xrow + 32 * j;
+        if constexpr(GEMM0)
+        {
+            int tok = p.tokens;
+            if(r < nrows)
+                tok = p.sorted_ids[row0 + r] & 0xffffff;
+            xvalid[j] = tok < p.tokens;
+            xptr[j]   = p.x + (int64_t)(xvalid[j] ? tok : 0) * p.x_row_bytes + xchunk * 16;
+        }
+        else
+        {
+            xvalid[j] = r < nrows;
+            xptr[j]   = p.x + (int64_t)(row0 + (xvalid[j] ? r : 0)) * p.x_row_bytes + xchunk * 16;
+        }
+    }
+
+    const int wchunk = tid % kWChunks;
+    const int wrow   = tid / kWChunks; // + kWRowsPerPass*j  (row of the LDS weight tile)
+    const int n_base = nt * (GEMM0 ? 128 : 256);
+    const unsigned char* wbase = p.w + (int64_t)expert * p.w_expert_bytes + wchunk * 16;
+    int64_t woff[kWLoads];
+#pragma unroll
+    for(int j = 0; j < kWLoads; j++)
+    {
+        const int lrow = wrow + kWRowsPerPass * j;
+        const int blk  = lrow >> 5;
+        const int c    = chan_of_row(lrow & 31);
+        int grow;
+        if constexpr(GEMM0)
+        {
+            const int col = min(n_base + (blk >> 1) * 32 + c, p.n_out - 1);
+            grow          = (blk & 1) * p.n_out + col;
+        }
+        else
+        {
+            grow = min(n_base + blk * 32 + c, p.n_total - 1);
+        }
+        woff[j] = (int64_t)grow * p.w_row_bytes;
+    }
+
+    uint4 xv[MBLK];
+    uint4 wv[kWLoads];
+    uint32_t ys_next[MBLK], ys_cur[MBLK];
+    const uint4 zero4 = {0u, 0u, 0u, 0u};
+
+    auto load_tiles = [&](int kt) {
+        const int kx = kt * kTileKB + xchunk * 16;
+#pragma unroll
+        for(int j = 0; j < MBLK; j++)
+        {
+            xv[j] = zero4;
+            if(j < nmb && xvalid[j] && kx < p.k_bytes_x)
+                xv[j] = *reinterpret_cast<const uint4*>(xptr[j] + kt * kTileKB);
+        }
+        const int kw = kt * kWKB + wchunk * 16;
+#pragma unroll
+        for(int j = 0; j < kWLoads; j++)
+        {
+            wv[j] = zero4;
+            if(kw < p.k_bytes_w)
+                wv[j] = *reinterpret_cast<const uint4*>(wbase + woff[j] + kt * kWKB);
+        }
+        if constexpr(kMx)
+        {
+#pragma unroll
+            for(int j = 0; j < MBLK; j++)
+            {
+                ys_next[j] = 0x7f7f7f7fu;
+                const int r = j * 32 + r32;
+                if(r < nrows)
+                    ys_next[j] = *reinterpret_cast<const uint32_t*>(p.y_scale + (int64_t)(row0 + r) * p.ys_row_bytes + kt * 4);
+            }
+        }
+    };
+
+    Acc acc[MBLK][2];
+#pragma unroll
+    for(int j = 0; j < MBLK; j++)
+#pragma unroll
+        for(int b = 0; b < 2; b++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                acc[j][b][v] = 0;
+
+    const int kt_count = ceil_div(p.k_bytes_x, kTileKB);
+    load_tiles(0);
+    for(int kt = 0; kt < kt_count; kt++)
+    {
+        // registers -> LDS
+#pragma unroll
+        for(int j = 0; j < MBLK; j++)
+            if(j < nmb)
+                *reinterpret_cast<uint4*>(lds_x + (xrow + 32 * j) * kXStride + xchunk * 16) = xv[j];
+#pragma unroll
+        for(int j = 0; j < kWLoads; j++)
+            *reinterpret_cast<uint4*>(lds_w + (wrow + kWRowsPerPass * j) * kWStride + wchunk * 16) = wv[j];
+        if constexpr(kMx)
+        {
+#pragma unroll
+            for(int j = 0; j < MBLK; j++)
+                ys_cur[j] = ys_next[j];
+        }
+        __syncthreads();
+        if(kt + 1 < kt_count)
+            load_tiles(kt + 1);
+
+        // MFMAs from LDS
+#pragma unroll
+        for(int s = 0; s < kSteps; s++)
+        {
+            Frag wf[2];
+#pragma unroll
+            for(int b = 0; b < 2; b++)
+            {
+                const unsigned char* wp = lds_w + ((wave * 2 + b) * 32 + r32) * kWStride;
+                if constexpr(MODE == kBf16W8)
+                    wf[b].lo = int8x8_to_bf16x8(*reinterpret_cast<const uint2*>(wp + (2 * s + kg) * 8));
+                else if constexpr(kOpB == 16)
+                    wf[b].lo = *reinterpret_cast<const uint4*>(wp + (2 * s + kg) * 16);
+                else
+                {
+                    // f8f6f4 operands: the low 16 bytes of lanes r and r+32 form one 32-element
+                    // scale block, the high 16 bytes the next one
+                    wf[b].lo = *reinterpret_cast<const uint4*>(wp + (4 * s + kg) * 16);
+                    wf[b].hi = *reinterpret_cast<const uint4*>(wp + (4 * s + 2 + kg) * 16);
+                }
+            }
+#pragma unroll
+            for(int j = 0; j < MBLK; j++)
+            {
+                if(j < nmb)
+                {
+                    Frag xf;
+                    const unsigned char* xp = lds_x + (j * 32 + r32) * kXStride;
+                    uint32_t xs             = 127;
+                    if constexpr(kOpB == 16)
+                        xf.lo = *reinterpret_cast<const uint4*>(xp + (2 * s + kg) * 16);
+                    else
+                    {
+                        xf.lo = *reinterpret_cast<const uint4*>(xp + (4 * s + kg) * 16);
+                        xf.hi = *reinterpret_cast<const uint4*>(xp + (4 * s + 2 + kg) * 16);
+                        // lane r carries the scale of block 2s, lane r+32 that of block 2s+1
+                        if constexpr(kMx)
+                            xs = (ys_cur[j] >> (8 * (2 * s + kg))) & 0xffu;
+                    }
+                    acc[j][0] = mfma<MODE>(wf[0], xf, xs, acc[j][0]);
+                    acc[j][1] = mfma<MODE>(wf[1], xf, xs, acc[j][1]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane owns token row (j*32 + r32) and 16 consecutive channels per block
+#pragma unroll
+    for(int j = 0; j < MBLK; j++)
+    {
+        if(j >= nmb)
+            continue;
+        const int r = j * 32 + r32;
+        if(r >= nrows)
+            continue;
+        const int sid   = p.sorted_ids[row0 + r];
+        const int tok   = sid & 0xffffff;
+        const bool real = tok < p.tokens;
+        if constexpr(GEMM0)
+        {
+            const int col0 = n_base + wave * 32 + 16 * kg; // first Y column of this lane
+            if(n_base + wave * 32 >= p.n_out)
+                continue;
+            float y[16];
+            float sa = 1.0f;
+            if(p.x_scale != nullptr)
+                sa = real ? p.x_scale[tok] : 0.0f;
+            const float* gs = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total + col0 : nullptr;
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+            {
+                float g = static_cast<float>(acc[j][0][v]);
+                float u = static_cast<float>(acc[j][1][v]);
+                if(gs != nullptr)
+                {
+                    g *= sa * gs[v];
+                    u *= sa * gs[p.n_out + v];
+                }
+                y[v] = silu(g) * u;
+            }
+            unsigned char* dst = p.out + (int64_t)(row0 + r) * p.out_row_bytes;
+            if constexpr(MODE == kFp8)
+            {
+                // e4m3 with one power-of-two scale per 32 columns (this lane's 16 + lane^32's 16)
+                float amax = 0.f;
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    amax = fmaxf(amax, fabsf(y[v]));
+                amax = fmaxf(amax, __shfl_xor(amax, 32));
+                const uint32_t ab = __float_as_uint(amax);
+                int sb            = static_cast<int>(ab >> 23) - 8 + ((ab & 0x7fffffu) > 0x600000u ? 1 : 0);
+                sb                = amax == 0.f ? 0 : max(0, min(254, sb));
+                const float inv   = __uint_as_float(static_cast<uint32_t>(254 - sb) << 23);
+                uint32_t q[4];
+#pragma unroll
+                for(int v = 0; v < 4; v++)
+                {
+                    float a0 = fminf(fmaxf(y[4 * v] * inv, -448.f), 448.f);
+                    float a1 = fminf(fmaxf(y[4 * v + 1] * inv, -448.f), 448.f);
+                    float a2 = fminf(fmaxf(y[4 * v + 2] * inv, -448.f), 448.f);
+                    float a3 = fminf(fmaxf(y[4 * v + 3] * inv, -448.f), 448.f);
+                    int pk   = __builtin_amdgcn_cvt_pk_fp8_f32(a0, a1, 0, false);
+                    pk       = __builtin_amdgcn_cvt_pk_fp8_f32(a2, a3, pk, true);
+                    q[v]     = static_cast<uint32_t>(pk);
+                }
+                *reinterpret_cast<uint4*>(dst + col0) = make_uint4(q[0], q[1], q[2], q[3]);
+                if(kg == 0)
+                    p.y_scale[(int64_t)(row0 + r) * p.ys_row_bytes + (col0 >> 5)] = static_cast<unsigned char>(sb);
+            }
+            else
+            {
+                uint4 o0, o1;
+                o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
+                o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
+                o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
+                o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
+                uint4* d4 = reinterpret_cast<uint4*>(dst + (int64_t)col0 * 2);
+                d4[0] = o0;
+                d4[1] = o1;
+            }
+        }
+        else
+        {
+            if(!real)
+                continue;
+            const int slot_k  = static_cast<int>(static_cast<uint32_t>(sid) >> 24);
+            const int64_t prow = (int64_t)tok * p.topk + slot_k;
+            const float tw    = p.sorted_w[row0 + r];
+            if(nt == 0 && wave == 0 && kg == 0)
+                p.valid[prow] = 1;
+            unsigned char* dst = p.out + prow * p.out_row_bytes;
+#pragma unroll
+            for(int b = 0; b < 2; b++)
+            {
+                const int col0 = n_base + (wave * 2 + b) * 32 + 16 * kg;
+                if(n_base + (wave * 2 + b) * 32 >= p.n_out)
+                    continue;
+                const float* ds = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total + col0 : nullptr;
+                float y[16];
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                {
+                    float o = static_cast<float>(acc[j][b][v]);
+                    if(ds != nullptr)
+                        o *= ds[v];
+                    y[v] = o * tw;
+                }
+                uint4 o0, o1;
+                o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
+                o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
+                o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
+                o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
+                uint4* d4 = reinterpret_cast<uint4*>(dst + (int64_t)col0 * 2);
+                d4[0] = o0;
+                d4[1] = o1;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tile list: one entry per (expert, group of <= rows_per_tile sorted rows), rows split evenly.
+// Block 0 builds the list from sorted_expert_ids; every block helps clear the valid flags.
+constexpr int kPrepBlock = 1024;
+constexpr int kPrepWaves = kPrepBlock / kWave;
+
+__device__ inline int lower_bound_dev(const int* a, int n, int key)
+{
+    int lo = 0, hi = n;
+    while(lo < hi)
+    {
+        const int mid = (lo + hi) >> 1;
+        if(a[mid] < key)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+__global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restrict__ sorted_eid,
+                                                               const int* __restrict__ post_pad_ptr, int unit,
+                                                               int experts, int rows_per_tile, int max_units,
+                                                               int max_tiles, int* __restrict__ tile_map,
+                                                               int* __restrict__ valid, int n_valid)
+{
+    for(int i = blockIdx.x * kPrepBlock + threadIdx.x; i < n_valid; i += gridDim.x * kPrepBlock)
+        valid[i] = 0;
+    if(blockIdx.x != 0)
+        return;
+    __shared__ int s_wave[kPrepWaves + 1];
+    const int post_pad = post_pad_ptr[0];
+    int nunits         = post_pad / unit;
+    nunits             = max(0, min(nunits, max_units));
+    int total          = 0;
+    for(int e0 = 0; e0 < experts; e0 += kPrepBlock) // experts <= 1024: one pass
+    {
+        const int e = e0 + threadIdx.x;
+        int lo = 0, hi = 0;
+        if(e < experts)
+        {
+            lo = lower_bound_dev(sorted_eid, nunits, e);
+            hi = lower_bound_dev(sorted_eid, nunits, e + 1);
+        }
+        const int rows = (hi - lo) * unit;
+        const int nt   = ceil_div(rows, rows_per_tile);
+        int sum;
+        const int tb   = total + block_exclusive_scan<kPrepWaves>(nt, s_wave, sum);
+        total += sum;
+        if(nt > 0)
+        {
+            const int per = round_up(ceil_div(rows, nt), 32);
+            for(int j = 0; j < nt; j++)
+            {
+                if(tb + j >= max_tiles)
+                    break;
+                int* ent = tile_map + kMapHdr + (tb + j) * kMapEnt;
+                ent[0]   = e;
+                ent[1]   = lo * unit + j * per;
+                ent[2]   = min(per, rows - j * per);
+                ent[3]   = tb;
+                ent[4]   = nt;
+            }
+        }
+    }
+    if(threadIdx.x == 0)
+        tile_map[0] = min(total, max_tiles);
+}
+
+// O[t, h] = sum over slots (in slot order) of the bf16 partials, fp32 accumulate, one rounding
+__global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* __restrict__ part,
+                                                           const int* __restrict__ valid,
+                                                           unsigned char* __restrict__ out, int topk, int hidden,
+                                                           int64_t out_row_bytes)
+{
+    const int t  = blockIdx.x;
+    const int h0 = (blockIdx.y * 256 + threadIdx.x) * 8;
+    if(h0 >= hidden)
+        return;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for(int k = 0; k < topk; k++)
+    {
+        const int64_t prow = (int64_t)t * topk + k;
+        if(valid[prow] == 0)
+            continue;
+        const uint4 v = *reinterpret_cast<const uint4*>(part + (prow * hidden + h0) * 2);
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            acc[2 * i] += __uint_as_float(d[i] << 16);
+            acc[2 * i + 1] += __uint_as_float(d[i] & 0xffff0000u);
+        }
+    }
+    uint4 o;
+    o.x = pack_bf16x2(acc[0], acc[1]);
+    o.y = pack_bf16x2(acc[2], acc[3]);
+    o.z = pack_bf16x2(acc[4], acc[5]);
+    o.w = pack_bf16x2(acc[6], acc[7]);
+    *reinterpret_cast<uint4*>(out + (int64_t)t * out_row_bytes + (int64_t)h0 * 2) = o;
+}
+
+// per-row dynamic quantisation bf16 -> e4m3 / int8
+template <bool FP8>
+__global__ __launch_bounds__(256) void rowwise_quant_kernel(const uint16_t* __restrict__ x, int cols,
+                                                             int64_t stride_x, unsigned char* __restrict__ q,
+                                                             float* __restrict__ scale)
+{
+    __shared__ float s_red[4];
+    const int64_t row  = blockIdx.x;
+    const uint16_t* xr = x + row * stride_x;
+    float amax         = 0.f;
+    for(int c = threadIdx.x; c < cols; c += 256)
+        amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c])));
+#pragma unroll
+    for(int d = 32; d > 0; d >>= 1)
+        amax = fmaxf(amax, __shfl_xor(amax, d));
+    if((threadIdx.x & 63) == 0)
+        s_red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax            = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    const float qmx = FP8 ? 448.0f : 127.0f;
+    const float s   = amax > 0.f ? amax / qmx : 1.0f;
+    if(threadIdx.x == 0)
+        scale[row] = s;
+    for(int c = threadIdx.x; c < cols; c += 256)
+    {
+        const float v = bf16_bits_to_float(xr[c]) / s;
+        if constexpr(FP8)
+        {
+            const float cl = fminf(fmaxf(v, -448.f), 448.f);
+            q[row * cols + c] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
+        }
+        else
+        {
+            const float cl = fminf(fmaxf(v, -128.f), 127.f);
+            q[row * cols + c] = static_cast<unsigned char>(static_cast<signed char>(__float2int_rn(cl)));
+        }
+    }
+}
+
+inline int pick_mblk(int64_t tokens, int topk, int experts)
+{
+    const int64_t avg = tokens * topk / experts;
+    if(avg <= 32)
+        return 1;
+    if(avg <= 64)
+        return 2;
+    return 4;
+}
+
+template <int MODE, bool GEMM0>
+int launch_gemm(int mblk, const GemmParams& p, int max_tiles, hipStream_t stream)
+{
+    using MT = ModeTraits<MODE>;
+    const int grid = round_up(max_tiles * p.n_ntiles, 8);
+    if(grid <= 0)
+        return MI355_MOE_OK;
+#define MI355_LAUNCH(MB)                                                                               \
+    {                                                                                                  \
+        const size_t lds = kWRows * (MT::kWKB + kPadB) + (MB)*32 * (kTileKB + kPadB);                  \
+        hipLaunchKernelGGL((moe_gemm_kernel<MODE, GEMM0, MB>), dim3(grid), dim3(kBlock), lds, stream, p); \
+    }
+    if(mblk == 1)
+        MI355_LAUNCH(1)
+    else if(mblk == 2)
+        MI355_LAUNCH(2)
+    else
+        MI355_LAUNCH(4)
+#undef MI355_LAUNCH
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+} // namespace
+
+int check_traits(const mi355_fused_moe_traits& t)
+{
+    const bool prec_ok = (t.prec_i == MI355_MOE_BF16 || t.prec_i == MI355_MOE_FP8 || t.prec_i == MI355_MOE_INT8) &&
+                         t.prec_w == t.prec_i && t.prec_o == MI355_MOE_BF16;
+    if(!prec_ok)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: unsupported precision (i=%d w=%d o=%d)", t.prec_i, t.prec_w,
+                    t.prec_o);
+    if(t.prec_st != MI355_MOE_FP32 || t.prec_sw != MI355_MOE_FP32 || t.prec_kw != MI355_MOE_FP32)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: scales and top-k weights must be fp32");
+    if(t.activation != 1)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: only activation=1 (silu) is implemented");
+    if(t.gate_only != 0)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: gate_only is not implemented");
+    if(t.fused_quant != 0)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: fused_quant=%d is not implemented", t.fused_quant);
+    if(t.block_m < 1 || t.block_m > 1024)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: block_m=%d", t.block_m);
+    return MI355_MOE_OK;
+}
+
+WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk,
+                                 int32_t hidden, int32_t inter)
+{
+    WorkspaceLayout w{};
+    auto bump = [&](size_t bytes) {
+        const size_t off = w.total;
+        w.total += round_up<size_t>(bytes, 256);
+        return off;
+    };
+    const int mblk   = pick_mblk(tokens, topk, experts);
+    w.max_pad        = (int64_t)topk * tokens + (int64_t)experts * t.block_m - topk;
+    w.max_tiles      = (int32_t)(experts + w.max_pad / (mblk * 32) + 1);
+    const int y_b    = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
+    w.sort_off       = bump(sorting_workspace_bytes(tokens, experts, topk));
+    w.map_off        = bump(sizeof(int) * (kMapHdr + (size_t)kMapEnt * w.max_tiles));
+    w.valid_off      = bump(sizeof(int) * (size_t)tokens * topk);
+    w.y_off          = bump((size_t)w.max_pad * inter * y_b);
+    w.ys_off         = bump(t.prec_i == MI355_MOE_FP8 ? (size_t)w.max_pad * (inter / 32) : 0);
+    w.p_off          = bump((size_t)tokens * topk * hidden * 2);
+    return w;
+}
+
+int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a, hipStream_t stream)
+{
+    int rc = check_traits(t);
+    if(rc != MI355_MOE_OK)
+        return rc;
+    if(!a.a_ptr || !a.g_ptr || !a.d_ptr || !a.o_ptr || !a.sorted_token_ids_ptr || !a.sorted_weight_ptr ||
+       !a.sorted_expert_ids_ptr || !a.num_sorted_tiles_ptr)
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: null tensor pointer");
+    if(a.y_smooth_scale_ptr != nullptr)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: y_smooth_scale is not implemented");
+    const bool quant = t.prec_i != MI355_MOE_BF16;
+    if(quant && (!a.a_scale_ptr || !a.g_scale_ptr || !a.d_scale_ptr))
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: quantised dtypes need a_scale, g_scale and d_scale");
+    const int H = a.hidden_size, I = a.intermediate_size, T = a.num_tokens, E = a.num_experts, K = a.topk;
+    if(H <= 0 || I <= 0 || T < 0 || E <= 0 || E > 1024 || K <= 0 || K > 255 || a.stride_token < H)
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: bad sizes (H=%d I=%d T=%d E=%d K=%d stride=%d)", H, I, T, E,
+                    K, a.stride_token);
+    const int eb = quant ? 1 : 2; // bytes per activation / weight element
+    if(H % 32 != 0 || I % 32 != 0 || (t.prec_i == MI355_MOE_FP8 && I % 128 != 0) ||
+       ((int64_t)a.stride_token * eb) % 16 != 0 || ((int64_t)a.stride_token * 2) % 16 != 0)
+        return fail(MI355_MOE_E_UNSUPPORTED,
+                    "fused_moegemm: hidden and intermediate must be multiples of 32 (128 for fp8 intermediate) and "
+                    "token rows 16-byte aligned (H=%d I=%d stride=%d)", H, I, a.stride_token);
+    for(const void* ptr : {a.a_ptr, a.g_ptr, a.d_ptr, static_cast<const void*>(a.o_ptr)})
+        if(reinterpret_cast<uintptr_t>(ptr) % 16 != 0)
+            return fail(MI355_MOE_E_INVALID, "fused_moegemm: a, g, d and o must be 16-byte aligned");
+    if(T == 0)
+        return MI355_MOE_OK;
+
+    const WorkspaceLayout ws = workspace_layout(t, T, E, K, H, I);
+    if(a.ws_ptr == nullptr || a.ws_bytes < ws.total)
+        return fail(MI355_MOE_E_WORKSPACE, "fused_moegemm: workspace of %zu bytes needed, %zu given", ws.total,
+                    a.ws_ptr ? a.ws_bytes : (size_t)0);
+    if(reinterpret_cast<uintptr_t>(a.ws_ptr) % 256 != 0)
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: workspace must be 256-byte aligned");
+    unsigned char* wsb = static_cast<unsigned char*>(a.ws_ptr);
+    int* tile_map      = reinterpret_cast<int*>(wsb + ws.map_off);
+    int* valid         = reinterpret_cast<int*>(wsb + ws.valid_off);
+    const int mblk     = pick_mblk(T, K, E);
+    const int max_units = (int)ceil_div<int64_t>(ws.max_pad, t.block_m);
+
+    const int n_valid    = T * K;
+    const int prep_grid  = 1 + std::min(ceil_div(n_valid, kPrepBlock * 4), 64);
+    hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
+                       static_cast<const int*>(a.sorted_expert_ids_ptr), static_cast<const int*>(a.num_sorted_tiles_ptr),
+                       t.block_m, E, mblk * 32, max_units, ws.max_tiles, tile_map, valid, n_valid);
+    MI355_HIP_TRY(hipGetLastError());
+
+    GemmParams p{};
+    p.sorted_ids = static_cast<const int*>(a.sorted_token_ids_ptr);
+    p.sorted_w   = static_cast<const float*>(a.sorted_weight_ptr);
+    p.tile_map   = tile_map;
+    p.valid      = valid;
+    p.tokens     = T;
+    p.topk       = K;
+    p.y_scale    = wsb + ws.ys_off;
+    p.ys_row_bytes = I / 32;
+
+    // ---- gemm0: gate+up, SiLU*up
+    const int y_b     = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
+    p.x               = static_cast<const unsigned char*>(a.a_ptr);
+    p.x_row_bytes     = (int64_t)a.stride_token * eb;
+    p.x_scale         = quant ? static_cast<const float*>(a.a_scale_ptr) : nullptr;
+    p.w               = static_cast<const unsigned char*>(a.g_ptr);
+    p.w_row_bytes     = (int64_t)H * eb;
+    p.w_expert_bytes  = (int64_t)2 * I * H * eb;
+    p.w_scale         = quant ? static_cast<const float*>(a.g_scale_ptr) : nullptr;
+    p.out             = wsb + ws.y_off;
+    p.out_row_bytes   = (int64_t)I * y_b;
+    p.k_bytes_x       = H * eb;
+    p.k_bytes_w       = H * eb;
+    p.n_out           = I;
+    p.n_total         = 2 * I;
+    p.n_ntiles        = ceil_div(I, 128);
+    if(t.prec_i == MI355_MOE_BF16)
+        rc = launch_gemm<kBf16, true>(mblk, p, ws.max_tiles, stream);
+    else if(t.prec_i == MI355_MOE_FP8)
+        rc = launch_gemm<kFp8, true>(mblk, p, ws.max_tiles, stream);
+    else
+        rc = launch_gemm<kI8, true>(mblk, p, ws.max_tiles, stream);
+    if(rc != MI355_MOE_OK)
+        return rc;
+
+    // ---- gemm1: down, * top-k weight, bf16 partial per (token, slot)
+    p.x              = wsb + ws.y_off;
+    p.x_row_bytes    = (int64_t)I * y_b;
+    p.x_scale        = nullptr;
+    p.w              = static_cast<const unsigned char*>(a.d_ptr);
+    p.w_row_bytes    = (int64_t)I * eb;
+    p.w_expert_bytes = (int64_t)H * I * eb;
+    p.w_scale        = quant ? static_cast<const float*>(a.d_scale_ptr) : nullptr;
+    p.out            = wsb + ws.p_off;
+    p.out_row_bytes  = (int64_t)H * 2;
+    p.k_bytes_x      = I * y_b;
+    p.k_bytes_w      = I * eb;
+    p.n_out          = H;
+    p.n_total        = H;
+    p.n_ntiles       = ceil_div(H, 256);
+    if(t.prec_i == MI355_MOE_BF16)
+        rc = launch_gemm<kBf16, false>(mblk, p, ws.max_tiles, stream);
+    else if(t.prec_i == MI355_MOE_FP8)
+        rc = launch_gemm<kFp8, false>(mblk, p, ws.max_tiles, stream);
+    else
+        rc = launch_gemm<kBf16W8, false>(mblk, p, ws.max_tiles, stream);
+    if(rc != MI355_MOE_OK)
+        return rc;
+
+    // ---- combine
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, valid,
+                       static_cast<unsigned char*>(a.o_ptr), K, H, (int64_t)a.stride_token * 2);
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype, void* q,
+                         void* scale, hipStream_t stream)
+{
+    if(!x || !q || !scale || rows < 0 || cols <= 0 || stride_x < cols)
+        return fail(MI355_MOE_E_INVALID, "rowwise_quant: bad arguments");
+    if(q_dtype != MI355_MOE_FP8 && q_dtype != MI355_MOE_INT8)
+        return fail(MI355_MOE_E_UNSUPPORTED, "rowwise_quant: q_dtype must be fp8 or int8");
+    if(rows == 0)
+        return MI355_MOE_OK;
+    if(rows > 0x7fffffff)
+        return fail(MI355_MOE_E_INVALID, "rowwise_quant: too many rows");
+    if(q_dtype == MI355_MOE_FP8)
+        hipLaunchKernelGGL(rowwise_quant_kernel<true>, dim3((unsigned)rows), dim3(256), 0, stream,
+                           static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),
+                           static_cast<float*>(scale));
+    else
+        hipLaunchKernelGGL(rowwise_quant_kernel<false>, dim3((unsigned)rows), dim3(256), 0, stream,
+                           static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),
+                           static_cast<float*>(scale));
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+} // namespace mi355

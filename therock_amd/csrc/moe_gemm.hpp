@@ -1,0 +1,33 @@
+// Host-side declarations of the grouped-GEMM half of libmi355_moe.so.
+#pragma once
+
+#include "common.hpp"
+
+namespace mi355 {
+
+// Carving of the caller's workspace (all offsets 256-byte aligned).
+struct WorkspaceLayout
+{
+    size_t sort_off;   // moe_sorting segment counters
+    size_t map_off;    // int32 [4 + 8 * max_tiles]: live tile count, then one entry per M tile
+    size_t valid_off;  // int32 [tokens * topk]: 1 where the (token, slot) partial was produced
+    size_t y_off;      // intermediate activations Y [max_pad, inter] (bf16 or e4m3)
+    size_t ys_off;     // e8m0 block scales of Y [max_pad, inter / 32] (fp8 path only)
+    size_t p_off;      // per-slot partial outputs [tokens * topk, hidden] bf16
+    size_t total;
+    int64_t max_pad;
+    int32_t max_tiles; // upper bound of M tiles
+};
+
+int check_traits(const mi355_fused_moe_traits& t);
+
+WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts,
+                                 int32_t topk, int32_t hidden, int32_t inter);
+
+int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a,
+                         hipStream_t stream);
+
+int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype,
+                         void* q, void* scale, hipStream_t stream);
+
+} // namespace mi355

@@ -1,0 +1,405 @@
+// moe_sorting for gfx950: stable token -> expert bucketing with padding to unit_size.
+//
+// Replaces ck_tile's MoeSortingKernel / MoeSortingMultiPhaseKernel_P0..P3
+// (ops/fused_moe/kernel/moe_sorting_kernel.hpp:224-1152, :1576-3229) and produces exactly what
+// ck_tile::reference_moe_sorting (host/reference/reference_moe_sorting.hpp:14-117) produces.
+//
+// Design (not ck_tile's mesh): the flat routing list ids[t*K+k] is cut into segments, one per
+// wavefront.  Pass 1 counts experts per segment (wave ballot match + per-wave LDS histogram),
+// pass 2 turns the [segment][expert] counts into output offsets (per-expert prefix over segments,
+// padded prefix over experts), pass 3 walks every segment again and scatters: the rank of an
+// entry inside its expert is segment offset + entries of that expert seen earlier in the wave
+// walk + popcount of lower lanes holding the same expert.  The sort is stable by construction
+// (no atomics decide an order), so the result is bit-exact with the host reference.  Small
+// problems run all three passes in one workgroup; large ones in three launches.  Traffic is
+// O(T*K) read twice plus O(segments*E) counters instead of ck_tile's O(E*T) mesh.
+#include "common.hpp"
+#include "device_utils.hpp"
+
+#include <algorithm>
+
+namespace mi355 {
+namespace {
+
+constexpr int kSeg               = 512;  // routing entries per wave segment (multi-launch path)
+constexpr int kWalkBlock         = 256;  // 4 waves = 4 segments per workgroup
+constexpr int kScanBlock         = 1024;
+constexpr int kScanWaves         = kScanBlock / kWave;
+constexpr int kMaxExperts        = 1024;
+constexpr int kOneShotMaxEntries = 16384;
+constexpr int kOneShotMaxExperts = 256;
+
+// lanes of this wave whose expert id equals mine
+__device__ inline uint64_t match_expert(int e, int nbits)
+{
+    uint64_t m = ~0ull;
+    for(int b = 0; b < nbits; b++)
+    {
+        const bool bit     = (e >> b) & 1;
+        const uint64_t bal = __ballot(bit);
+        m &= bit ? bal : ~bal;
+    }
+    return m;
+}
+
+__device__ inline int real_tokens(const int* local_tokens, int tokens)
+{
+    if(local_tokens == nullptr)
+        return tokens;
+    int t = *local_tokens;
+    return t < 0 ? 0 : (t > tokens ? tokens : t);
+}
+
+// One wave walks routing entries [begin, end) in order, 64 at a time.
+// cnt[e] holds (COUNT) the number of entries of expert e seen so far, or (SCATTER) the output
+// position of the next entry of expert e (negative: expert masked out, entries dropped).
+template <bool SCATTER>
+__device__ inline void walk_segment(const int* __restrict__ ids, const float* __restrict__ weights,
+                                    int begin, int end, int K, int E, int nbits, int* cnt,
+                                    int* __restrict__ out_ids, float* __restrict__ out_w)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    for(int i0 = begin; i0 < end; i0 += kWave)
+    {
+        const int i = i0 + lane;
+        int e       = i < end ? ids[i] : -1;
+        const bool valid = e >= 0 && e < E;
+        if(!valid)
+            e = 0;
+        const uint64_t same = match_expert(e, nbits) & __ballot(valid);
+        const int before    = __popcll(same & ((1ull << lane) - 1ull));
+        int base            = 0;
+        if(valid)
+            base = cnt[e];
+        wave_sync(); // every lane has read cnt[] before a leader updates it
+        if(valid)
+        {
+            if constexpr(SCATTER)
+            {
+                if(base >= 0)
+                {
+                    const int t        = i / K;
+                    const int k        = i - t * K;
+                    out_ids[base + before] = mock_id(t, k);
+                    out_w[base + before]   = weights[i];
+                }
+            }
+            if(before == 0 && base >= 0)
+                cnt[e] = base + __popcll(same);
+        }
+        wave_sync();
+    }
+}
+
+struct ScanShared
+{
+    int part[kScanBlock];  // [parts][Ep] partial sums over groups of segments
+    int cnt[kMaxExperts];  // entries per expert
+    int tiles[kMaxExperts];
+    int tbase[kMaxExperts]; // first output tile of the expert
+    int oeid[kMaxExperts];  // expert id written to sorted_expert_ids
+    int wave[kScanWaves + 1];
+};
+
+// Pass 2, run by one 1024-thread block.  counts is [nseg][E] (global or LDS): on entry the
+// per-segment histogram, on exit the output position of each segment's first entry per expert
+// (-1 for experts that produce no output).
+__device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, int Ep, int U,
+                                  const int* __restrict__ mask, int T, int K,
+                                  int* __restrict__ sorted_ids, float* __restrict__ sorted_w,
+                                  int* __restrict__ sorted_eid, int* __restrict__ total)
+{
+    const int tid   = threadIdx.x;
+    const int e     = tid & (Ep - 1);
+    const int part  = tid / Ep;
+    const int parts = kScanBlock / Ep;
+    const int spp   = ceil_div(nseg, parts);
+    const int s0    = part * spp;
+    const int s1    = min(s0 + spp, nseg);
+
+    int sum = 0;
+    if(e < E)
+        for(int sg = s0; sg < s1; sg++)
+            sum += counts[sg * E + e];
+    s.part[part * Ep + e] = sum;
+    __syncthreads();
+    if(tid < Ep)
+    {
+        int run = 0;
+        for(int p = 0; p < parts; p++)
+        {
+            const int v          = s.part[p * Ep + tid];
+            s.part[p * Ep + tid] = run;
+            run += v;
+        }
+        s.cnt[tid] = run;
+    }
+    if(tid >= Ep && tid < kMaxExperts)
+        s.cnt[tid] = 0;
+    __syncthreads();
+
+    // an expert that is masked out is skipped without consuming an output expert id; an expert
+    // with no token is skipped but does consume one (reference_moe_sorting.hpp:84-98)
+    const bool on_rank = tid < E && (mask == nullptr || mask[tid] != 0);
+    const int my_cnt   = tid < E ? s.cnt[tid] : 0;
+    const int my_tiles = on_rank ? ceil_div(my_cnt, U) : 0;
+    int total_tiles, total_ids;
+    const int tbase = block_exclusive_scan<kScanWaves>(my_tiles, s.wave, total_tiles);
+    const int oeid  = block_exclusive_scan<kScanWaves>(on_rank ? 1 : 0, s.wave, total_ids);
+    (void)total_ids;
+    if(tid < kMaxExperts)
+    {
+        s.tiles[tid] = my_tiles;
+        s.tbase[tid] = tbase;
+        s.oeid[tid]  = oeid;
+    }
+    __syncthreads();
+
+    if(e < E)
+    {
+        int base = s.tiles[e] > 0 ? s.tbase[e] * U + s.part[part * Ep + e] : -1;
+        for(int sg = s0; sg < s1; sg++)
+        {
+            const int c          = counts[sg * E + e];
+            counts[sg * E + e]   = base;
+            if(base >= 0)
+                base += c;
+        }
+    }
+
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int pad  = mock_id(T, K);
+    for(int ex = wave; ex < E; ex += kScanWaves)
+    {
+        const int tl = s.tiles[ex];
+        if(tl == 0)
+            continue;
+        const int tb = s.tbase[ex];
+        const int oe = s.oeid[ex];
+        for(int j = lane; j < tl; j += kWave)
+            sorted_eid[tb + j] = oe;
+        for(int p = s.cnt[ex] + lane; p < tl * U; p += kWave)
+        {
+            sorted_ids[tb * U + p] = pad;
+            sorted_w[tb * U + p]   = 0.f;
+        }
+    }
+    if(tid == 0)
+    {
+        total[0] = total_tiles * U;
+        total[1] = T;
+    }
+}
+
+__device__ inline void zero_buffer(uint4* buf, int64_t nvec, int64_t first, int64_t stride)
+{
+    const uint4 z = {0u, 0u, 0u, 0u};
+    for(int64_t i = first; i < nvec; i += stride)
+        buf[i] = z;
+}
+
+struct SortParams
+{
+    const int* ids;
+    const float* weights;
+    const int* mask;
+    const int* local_tokens;
+    int* sorted_ids;
+    float* sorted_w;
+    int* sorted_eid;
+    int* total;
+    uint4* moe_buf;
+    int64_t moe_row_vec16; // 16-byte vectors per token row of moe_buf
+    int* counts;           // workspace [nseg][E]
+    int tokens, K, E, Ep, nbits, U, nseg, work_blocks;
+};
+
+// ---- whole sort in one workgroup (block 0); the other blocks zero moe_buf
+__global__ __launch_bounds__(kScanBlock) void moe_sorting_oneshot_kernel(SortParams p)
+{
+    extern __shared__ int dyn_lds[]; // [kScanWaves][E]
+    __shared__ ScanShared sh;
+    const int T = real_tokens(p.local_tokens, p.tokens);
+    if(blockIdx.x > 0)
+    {
+        zero_buffer(p.moe_buf, p.moe_row_vec16 * T,
+                    (int64_t)(blockIdx.x - 1) * kScanBlock + threadIdx.x,
+                    (int64_t)(gridDim.x - 1) * kScanBlock);
+        return;
+    }
+    const int N      = T * p.K;
+    const int lane   = threadIdx.x & (kWave - 1);
+    const int wave   = threadIdx.x / kWave;
+    const int seglen = round_up(ceil_div(N, kScanWaves), kWave);
+    const int begin  = min(wave * seglen, N);
+    const int end    = min(begin + seglen, N);
+    int* cnt         = dyn_lds + wave * p.E;
+    for(int e = lane; e < p.E; e += kWave)
+        cnt[e] = 0;
+    wave_sync();
+    walk_segment<false>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, nullptr, nullptr);
+    __syncthreads();
+    scan_phase(sh, dyn_lds, kScanWaves, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
+               p.sorted_eid, p.total);
+    __syncthreads();
+    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w);
+}
+
+// ---- pass 1: per-segment expert histogram; trailing blocks zero moe_buf
+__global__ __launch_bounds__(kWalkBlock) void moe_sorting_count_kernel(SortParams p)
+{
+    extern __shared__ int dyn_lds[]; // [4][E]
+    const int T = real_tokens(p.local_tokens, p.tokens);
+    if((int)blockIdx.x >= p.work_blocks)
+    {
+        zero_buffer(p.moe_buf, p.moe_row_vec16 * T,
+                    (int64_t)(blockIdx.x - p.work_blocks) * kWalkBlock + threadIdx.x,
+                    (int64_t)(gridDim.x - p.work_blocks) * kWalkBlock);
+        return;
+    }
+    const int N    = T * p.K;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int seg  = blockIdx.x * (kWalkBlock / kWave) + wave;
+    if(seg >= p.nseg)
+        return;
+    int* cnt = dyn_lds + wave * p.E;
+    for(int e = lane; e < p.E; e += kWave)
+        cnt[e] = 0;
+    wave_sync();
+    const int begin = min(seg * kSeg, N);
+    const int end   = min(begin + kSeg, N);
+    walk_segment<false>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, nullptr, nullptr);
+    for(int e = lane; e < p.E; e += kWave)
+        p.counts[seg * p.E + e] = cnt[e];
+}
+
+// ---- pass 2
+__global__ __launch_bounds__(kScanBlock) void moe_sorting_scan_kernel(SortParams p)
+{
+    __shared__ ScanShared sh;
+    const int T = real_tokens(p.local_tokens, p.tokens);
+    scan_phase(sh, p.counts, p.nseg, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
+               p.sorted_eid, p.total);
+}
+
+// ---- pass 3
+__global__ __launch_bounds__(kWalkBlock) void moe_sorting_scatter_kernel(SortParams p)
+{
+    extern __shared__ int dyn_lds[]; // [4][E]
+    const int T    = real_tokens(p.local_tokens, p.tokens);
+    const int N    = T * p.K;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int seg  = blockIdx.x * (kWalkBlock / kWave) + wave;
+    if(seg >= p.nseg)
+        return;
+    int* cnt = dyn_lds + wave * p.E;
+    for(int e = lane; e < p.E; e += kWave)
+        cnt[e] = p.counts[seg * p.E + e];
+    wave_sync();
+    const int begin = min(seg * kSeg, N);
+    const int end   = min(begin + kSeg, N);
+    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w);
+}
+
+inline bool use_oneshot(int64_t entries, int experts)
+{
+    return entries <= kOneShotMaxEntries && experts <= kOneShotMaxExperts;
+}
+
+} // namespace
+
+size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk)
+{
+    if(tokens < 0 || experts <= 0 || topk <= 0)
+        return 0;
+    const int64_t n = (int64_t)tokens * topk;
+    if(use_oneshot(n, experts))
+        return 0;
+    return round_up<size_t>((size_t)ceil_div<int64_t>(n, kSeg) * experts * sizeof(int), 256);
+}
+
+int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream)
+{
+    if((a.tokens > 0 && (!a.p_topk_ids || !a.p_weights)) || !a.p_sorted_token_ids || !a.p_sorted_weights ||
+       !a.p_sorted_expert_ids || !a.p_total_tokens_post_pad)
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: null input or output pointer");
+    if(a.tokens < 0 || a.tokens >= (1 << 24))
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: tokens=%d outside [0, 2^24)", a.tokens);
+    if(a.topk < 1 || a.topk > 255)
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: topk=%d outside [1, 255]", a.topk);
+    if(a.num_experts < 1 || a.num_experts > kMaxExperts)
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: num_experts=%d outside [1, %d]", a.num_experts,
+                    kMaxExperts);
+    if(a.unit_size < 1)
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: unit_size=%d", a.unit_size);
+    const int64_t n = (int64_t)a.tokens * a.topk;
+    if(n + (int64_t)a.num_experts * a.unit_size >= (1ll << 31))
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: tokens*topk too large for int32 positions");
+
+    SortParams p{};
+    p.ids          = static_cast<const int*>(a.p_topk_ids);
+    p.weights      = static_cast<const float*>(a.p_weights);
+    p.mask         = static_cast<const int*>(a.p_local_expert_mask);
+    p.local_tokens = static_cast<const int*>(a.p_local_tokens);
+    p.sorted_ids   = static_cast<int*>(a.p_sorted_token_ids);
+    p.sorted_w     = static_cast<float*>(a.p_sorted_weights);
+    p.sorted_eid   = static_cast<int*>(a.p_sorted_expert_ids);
+    p.total        = static_cast<int*>(a.p_total_tokens_post_pad);
+    p.tokens       = a.tokens;
+    p.K            = a.topk;
+    p.E            = a.num_experts;
+    p.U            = a.unit_size;
+    p.Ep           = 1;
+    while(p.Ep < p.E)
+        p.Ep <<= 1;
+    p.nbits = 0;
+    while((1 << p.nbits) < p.E)
+        p.nbits++;
+
+    int zero_blocks = 0;
+    if(a.p_moe_buf != nullptr)
+    {
+        const int64_t row_bytes = (int64_t)a.moe_buf_interm_dim * a.moe_buf_elem_bytes;
+        if(row_bytes <= 0 || row_bytes % 16 != 0)
+            return fail(MI355_MOE_E_INVALID,
+                        "moe_sorting: moe_buf row of %lld bytes is not a positive multiple of 16",
+                        (long long)row_bytes);
+        if(reinterpret_cast<uintptr_t>(a.p_moe_buf) % 16 != 0)
+            return fail(MI355_MOE_E_INVALID, "moe_sorting: p_moe_buf is not 16-byte aligned");
+        p.moe_buf       = static_cast<uint4*>(a.p_moe_buf);
+        p.moe_row_vec16 = row_bytes / 16;
+        const int64_t nvec = p.moe_row_vec16 * a.tokens;
+        zero_blocks = (int)std::min<int64_t>(ceil_div<int64_t>(nvec, 4 * kScanBlock), (int64_t)device_info().num_cu * 4);
+        if(nvec > 0 && zero_blocks < 1)
+            zero_blocks = 1;
+    }
+
+    if(use_oneshot(n, p.E))
+    {
+        p.nseg = kScanWaves;
+        hipLaunchKernelGGL(moe_sorting_oneshot_kernel, dim3(1 + zero_blocks), dim3(kScanBlock),
+                           kScanWaves * p.E * sizeof(int), stream, p);
+        MI355_HIP_TRY(hipGetLastError());
+        return MI355_MOE_OK;
+    }
+    if(a.p_ws == nullptr)
+        return fail(MI355_MOE_E_WORKSPACE, "moe_sorting: p_ws is null but %zu bytes are needed",
+                    sorting_workspace_bytes(a.tokens, a.num_experts, a.topk));
+    p.counts      = static_cast<int*>(a.p_ws);
+    p.nseg        = (int)ceil_div<int64_t>(n, kSeg);
+    p.work_blocks = ceil_div(p.nseg, kWalkBlock / kWave);
+    const size_t lds = (kWalkBlock / kWave) * p.E * sizeof(int);
+    hipLaunchKernelGGL(moe_sorting_count_kernel, dim3(p.work_blocks + zero_blocks), dim3(kWalkBlock), lds,
+                       stream, p);
+    MI355_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(moe_sorting_scan_kernel, dim3(1), dim3(kScanBlock), 0, stream, p);
+    MI355_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(moe_sorting_scatter_kernel, dim3(p.work_blocks), dim3(kWalkBlock), lds, stream, p);
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+} // namespace mi355

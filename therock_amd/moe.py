@@ -1,0 +1,237 @@
+"""Host-side mirror of Composable Kernel's fused-MoE example API on top of the C ABI.
+
+Same names, argument meaning and error behaviour as CK's example/ck_tile/15_fused_moe and
+13_moe_sorting (``fused_moe_traits`` / ``fused_moe_args`` / ``fused_moe()``, ``moe_sorting_trait`` /
+``moe_sorting_args`` / ``moe_sorting()``): tensors are caller-owned device tensors, the calls are
+asynchronous on a stream, ``fused_moe`` returns a float (0 when not timing, -1 when no kernel
+matches the traits) and HIP / argument errors raise ``RuntimeError``.  torch is used only to hold
+device memory and streams; all compute happens in libmi355_moe.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional
+
+from . import _lib
+
+
+@dataclass
+class fused_moe_traits:
+    prec_i: str = "bf16"   # input (activation) precision
+    prec_w: str = "bf16"   # weight precision
+    prec_o: str = "bf16"   # output precision
+    prec_st: str = "fp32"  # token scale
+    prec_sw: str = "fp32"  # weight scale
+    prec_sq: str = "fp32"  # smooth-quant scale
+    prec_kw: str = "fp32"  # top-k weight
+    block_m: int = 32
+    activation: int = 1    # 0 gelu, 1 silu
+    gate_only: int = 0
+    fused_quant: int = 0
+    local_expert_masking: bool = False
+
+    def pod(self) -> _lib.FusedMoeTraits:
+        d = _lib.DTYPES
+        for k in ("prec_i", "prec_w", "prec_o", "prec_st", "prec_sw", "prec_sq", "prec_kw"):
+            if getattr(self, k) not in d:
+                raise ValueError(f"unknown precision {getattr(self, k)!r} for {k}")
+        return _lib.FusedMoeTraits(d[self.prec_i], d[self.prec_w], d[self.prec_o], d[self.prec_st], d[self.prec_sw],
+                                   d[self.prec_sq], d[self.prec_kw], self.block_m, self.activation, self.gate_only,
+                                   self.fused_quant, int(self.local_expert_masking))
+
+
+@dataclass
+class moe_sorting_trait:
+    index_type: str = "int32"
+    weight_type: str = "fp32"
+    local_expert_masking: bool = False
+
+
+def _ptr(t) -> Optional[int]:
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    if not t.is_cuda:
+        raise ValueError("tensors handed to the MoE path must live on the GPU")
+    if not t.is_contiguous():
+        raise ValueError("tensors handed to the MoE path must be contiguous")
+    return t.data_ptr()
+
+
+def _stream(stream) -> Optional[int]:
+    import torch
+
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return stream.cuda_stream if hasattr(stream, "cuda_stream") else int(stream)
+
+
+@dataclass
+class moe_sorting_args:
+    p_topk_ids: object = None
+    p_weights: object = None
+    p_local_expert_mask: object = None
+    p_local_tokens: object = None
+    p_sorted_token_ids: object = None
+    p_sorted_weights: object = None
+    p_sorted_expert_ids: object = None
+    p_total_tokens_post_pad: object = None
+    p_moe_buf: object = None
+    p_ws: object = None
+    tokens: int = 0
+    unit_size: int = 32
+    num_experts: int = 0
+    topk: int = 0
+    moe_buf_interm_dim: int = 0
+    moe_buf_elem_bytes: int = 0
+
+
+@dataclass
+class fused_moe_args:
+    a_ptr: object = None
+    a_scale_ptr: object = None
+    g_ptr: object = None
+    d_ptr: object = None
+    g_scale_ptr: object = None
+    d_scale_ptr: object = None
+    y_smooth_scale_ptr: object = None
+    local_expert_mask_ptr: object = None
+    o_ptr: object = None
+    ws_ptr: object = None
+    topk_ids_ptr: object = None
+    topk_weight_ptr: object = None
+    sorted_token_ids_ptr: object = None
+    sorted_weight_ptr: object = None
+    sorted_expert_ids_ptr: object = None
+    num_sorted_tiles_ptr: object = None
+    block_m: int = 32
+    hidden_size: int = 0
+    intermediate_size: int = 0
+    num_tokens: int = 0
+    num_experts: int = 0
+    topk: int = 0
+    stride_token: int = 0
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != _lib.OK:
+        raise RuntimeError(f"{what} failed ({rc}): {_lib.last_error()}")
+
+
+def moe_max_num_tokens_padded(tokens: int, num_experts: int, topk: int, unit_size: int) -> int:
+    return int(_lib.load().mi355_moe_max_num_tokens_padded(tokens, num_experts, topk, unit_size))
+
+
+def moe_sorting_get_workspace_size(tokens: int, num_experts: int, topk: int, dispatch_policy: int = 0) -> int:
+    return int(_lib.load().mi355_moe_sorting_workspace_size(tokens, num_experts, topk))
+
+
+def moe_sorting(trait: moe_sorting_trait, a: moe_sorting_args, stream=None) -> float:
+    """Returns 0.0 on success, -1.0 when the trait has no kernel (as CK's dispatcher does)."""
+    if trait.index_type != "int32" or trait.weight_type != "fp32":
+        return -1.0
+    mask = a.p_local_expert_mask if trait.local_expert_masking else None
+    s = _lib.SortingArgs(_ptr(a.p_topk_ids), _ptr(a.p_weights), _ptr(mask), _ptr(a.p_local_tokens),
+                         _ptr(a.p_sorted_token_ids), _ptr(a.p_sorted_weights), _ptr(a.p_sorted_expert_ids),
+                         _ptr(a.p_total_tokens_post_pad), _ptr(a.p_moe_buf), _ptr(a.p_ws), a.tokens, a.unit_size,
+                         a.num_experts, a.topk, a.moe_buf_interm_dim, a.moe_buf_elem_bytes)
+    _check(_lib.load().mi355_moe_sorting(C.byref(s), _stream(stream)), "moe_sorting")
+    return 0.0
+
+
+def fused_moe_get_workspace_size(traits: fused_moe_traits, tokens, num_experts, topk, hidden_size,
+                                 intermediate_size) -> int:
+    t = traits.pod()
+    return int(_lib.load().mi355_fused_moe_workspace_size(C.byref(t), tokens, num_experts, topk, hidden_size,
+                                                          intermediate_size))
+
+
+def _ws_bytes(ws) -> int:
+    return 0 if ws is None else ws.numel() * ws.element_size()
+
+
+def fused_moe(traits: fused_moe_traits, a: fused_moe_args, stream=None) -> float:
+    """Sort + gate/up GEMM + SiLU*up + down GEMM + top-k combine.  0.0 on success, -1.0 when no
+    kernel matches the traits."""
+    lib = _lib.load()
+    t = traits.pod()
+    if not lib.mi355_fused_moe_supported(C.byref(t)):
+        return -1.0
+    f = _lib.FusedMoeArgs(_ptr(a.a_ptr), _ptr(a.a_scale_ptr), _ptr(a.g_ptr), _ptr(a.d_ptr), _ptr(a.g_scale_ptr),
+                          _ptr(a.d_scale_ptr), _ptr(a.y_smooth_scale_ptr), _ptr(a.local_expert_mask_ptr),
+                          _ptr(a.o_ptr), _ptr(a.ws_ptr), _ws_bytes(a.ws_ptr), _ptr(a.topk_ids_ptr),
+                          _ptr(a.topk_weight_ptr), _ptr(a.sorted_token_ids_ptr), _ptr(a.sorted_weight_ptr),
+                          _ptr(a.sorted_expert_ids_ptr), _ptr(a.num_sorted_tiles_ptr), a.block_m, a.hidden_size,
+                          a.intermediate_size, a.num_tokens, a.num_experts, a.topk, a.stride_token)
+    rc = lib.mi355_fused_moe(C.byref(t), C.byref(f), _stream(stream))
+    if rc == _lib.E_UNSUPPORTED:
+        return -1.0
+    _check(rc, "fused_moe")
+    return 0.0
+
+
+def fused_moegemm(traits: fused_moe_traits, a: fused_moe_args, stream=None) -> float:
+    """GEMM half only: consumes sorted_* / num_sorted_tiles already written by moe_sorting."""
+    lib = _lib.load()
+    t = traits.pod()
+    if not lib.mi355_fused_moe_supported(C.byref(t)):
+        return -1.0
+    g = _lib.FusedMoeGemmArgs(_ptr(a.a_ptr), _ptr(a.a_scale_ptr), _ptr(a.g_ptr), _ptr(a.d_ptr), _ptr(a.g_scale_ptr),
+                              _ptr(a.d_scale_ptr), _ptr(a.y_smooth_scale_ptr), _ptr(a.o_ptr),
+                              _ptr(a.sorted_token_ids_ptr), _ptr(a.sorted_weight_ptr), _ptr(a.sorted_expert_ids_ptr),
+                              _ptr(a.num_sorted_tiles_ptr), _ptr(a.ws_ptr), _ws_bytes(a.ws_ptr), a.hidden_size,
+                              a.intermediate_size, a.num_tokens, a.num_experts, a.topk, a.stride_token)
+    rc = lib.mi355_fused_moegemm(C.byref(t), C.byref(g), _stream(stream))
+    if rc == _lib.E_UNSUPPORTED:
+        return -1.0
+    _check(rc, "fused_moegemm")
+    return 0.0
+
+
+def rowwise_quant(x, q_dtype: str, stream=None):
+    """Per-token dynamic quantisation of a bf16 [rows, cols] tensor -> (q, scale[rows] fp32)."""
+    import torch
+
+    rows, cols = x.shape
+    st = {"fp8": torch.float8_e4m3fn, "int8": torch.int8}[q_dtype]
+    q = torch.empty((rows, cols), dtype=st, device=x.device)
+    scale = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    _check(_lib.load().mi355_moe_rowwise_quant(_ptr(x), rows, cols, x.stride(0), _lib.DTYPES[q_dtype], _ptr(q),
+                                               _ptr(scale), _stream(stream)), "rowwise_quant")
+    return q, scale
+
+
+# ------------------------------------------------------------------ convenience for harnesses
+class MoeBuffers:
+    """Caller-side allocation of everything fused_moe needs (what CK's example main does with
+    DeviceMem): sort outputs, workspace and the output tensor."""
+
+    def __init__(self, traits: fused_moe_traits, tokens, experts, topk, hidden, inter, device):
+        import torch
+
+        self.max_pad = moe_max_num_tokens_padded(tokens, experts, topk, traits.block_m)
+        self.max_tiles = (self.max_pad + traits.block_m - 1) // traits.block_m
+        self.sorted_ids = torch.empty((self.max_pad,), dtype=torch.int32, device=device)
+        self.sorted_w = torch.empty((self.max_pad,), dtype=torch.float32, device=device)
+        self.sorted_eid = torch.empty((self.max_tiles,), dtype=torch.int32, device=device)
+        self.total = torch.zeros((2,), dtype=torch.int32, device=device)
+        ws = fused_moe_get_workspace_size(traits, tokens, experts, topk, hidden, inter)
+        self.ws = torch.empty((max(ws, 256),), dtype=torch.uint8, device=device)
+        self.out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=device)
+
+
+def make_args(traits: fused_moe_traits, buf: MoeBuffers, a, g, d, topk_ids, topk_weight, a_scale=None,
+              g_scale=None, d_scale=None, local_expert_mask=None, num_experts=None) -> fused_moe_args:
+    T, H = a.shape
+    E, n0, _ = g.shape
+    if num_experts is not None:  # with a local expert mask g/d hold the local experts only
+        E = num_experts
+    return fused_moe_args(
+        a_ptr=a, a_scale_ptr=a_scale, g_ptr=g, d_ptr=d, g_scale_ptr=g_scale, d_scale_ptr=d_scale,
+        local_expert_mask_ptr=local_expert_mask, o_ptr=buf.out, ws_ptr=buf.ws, topk_ids_ptr=topk_ids,
+        topk_weight_ptr=topk_weight, sorted_token_ids_ptr=buf.sorted_ids, sorted_weight_ptr=buf.sorted_w,
+        sorted_expert_ids_ptr=buf.sorted_eid, num_sorted_tiles_ptr=buf.total, block_m=traits.block_m,
+        hidden_size=H, intermediate_size=n0 // 2, num_tokens=T, num_experts=E, topk=topk_ids.shape[1],
+        stride_token=a.stride(0))
