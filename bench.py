@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-MoE path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--headline-only] [--no-cpu-baseline]
+
+One "step" is one pass of the whole path (moe_sorting + gate/up GEMM with SiLU*up + down GEMM +
+top-k combine) over one batch of synthetic, already-quantised inputs resident in HBM.  The headline
+workload is the DeepSeek-V3-shaped fp8 layer at 8192 tokens (the configuration the target of the
+metric is quoted on); the other benchmark configurations are reported under "workloads" in the
+same JSON line.  Prints exactly one JSON line on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "fused-MoE TFLOP/s (prefill) + HBM GB/s (decode), % of MI355X roofline, 1 GPU"
+HEADLINE = "cfg3_dsv3_fp8"
+# published MI355X peaks: dense MFMA TFLOP/s (TOP/s for int8) and HBM GB/s
+PEAK_MFMA = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
+PEAK_HBM = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def run_workload(cfg, steps, warmup, seed=0):
+    """Times `steps` passes of the path; per-kernel durations come from HIP events recorded by
+    the library on the launch stream inside the same timed region."""
+    import torch
+
+    import therock_amd as ta
+    from therock_amd import _lib
+    from therock_amd import inputs as mi
+
+    dev = torch.device("cuda:0")
+    inp = mi.make_inputs_torch(cfg, dev, seed)
+    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit)
+    buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, dev)
+    args = ta.make_args(traits, buf, inp["a"], inp["g"], inp["d"], inp["topk_ids"], inp["topk_weight"],
+                        a_scale=inp["a_scale"], g_scale=inp["g_scale"], d_scale=inp["d_scale"])
+    for _ in range(warmup):
+        assert ta.fused_moe(traits, args) == 0.0
+    torch.cuda.synchronize()
+    _lib.profile_start()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ta.fused_moe(traits, args)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kern = _lib.profile_stop()
+    ms = (t1 - t0) * 1e3 / steps
+    post_pad = int(buf.total[0])
+    active = int(torch.unique(inp["topk_ids"]).numel())
+    kavg = {k: v[0] / max(v[1], 1) for k, v in kern.items()}
+    T, K, H, I = cfg.tokens, cfg.topk, cfg.hidden, cfg.inter
+    flops0, flops1 = 4.0 * T * K * H * I, 2.0 * T * K * H * I
+    byt = mi.decode_bytes(cfg, active, post_pad)
+    gemm_ms = kavg.get("moe_gemm0_gate_up_silu", 0) + kavg.get("moe_gemm1_down", 0) + kavg.get("moe_combine", 0) + kavg.get("moe_prep", 0)
+    res = {
+        "workload": cfg.name, "dtype": cfg.dtype, "tokens": T, "hidden": H, "inter": I, "experts": cfg.experts,
+        "topk": K, "block_m": cfg.unit, "ms_per_step": ms, "tflops": cfg.flops / ms / 1e9,
+        "tokens_per_s": T / ms * 1e3, "algorithmic_GB": byt / 1e9, "hbm_GBps": byt / ms / 1e6,
+        "frac_mfma_peak": cfg.flops / ms / 1e9 / PEAK_MFMA[cfg.dtype], "frac_hbm_peak": byt / ms / 1e6 / PEAK_HBM,
+        "gemm_only_ms": gemm_ms, "post_pad": post_pad, "active_experts": active,
+        "kernel_avg_ms": {k: round(v, 5) for k, v in kavg.items()},
+        "gemm0_tflops": flops0 / kavg["moe_gemm0_gate_up_silu"] / 1e9 if "moe_gemm0_gate_up_silu" in kavg else None,
+        "gemm1_tflops": flops1 / kavg["moe_gemm1_down"] / 1e9 if "moe_gemm1_down" in kavg else None,
+    }
+    return res, inp, buf
+
+
+def roofline_of(cfg, res):
+    """Roofline entry for the dominant kernel of a workload."""
+    k0, k1 = res["kernel_avg_ms"].get("moe_gemm0_gate_up_silu"), res["kernel_avg_ms"].get("moe_gemm1_down")
+    T, K, H, I = cfg.tokens, cfg.topk, cfg.hidden, cfg.inter
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(cfg.name, {}).get("gemm0_hbm_bytes_per_launch")
+    if cfg.flops / (res["algorithmic_GB"] * 1e9) > PEAK_MFMA[cfg.dtype] * 1e12 / (PEAK_HBM * 1e9):
+        ach = 4.0 * T * K * H * I / k0 / 1e9  # gate+up GEMM: 2/3 of the FLOPs
+        return {"kernel": "moe_gemm_kernel (gemm0: gate+up, SiLU*up)", "bound": "mfma", "achieved": ach,
+                "peak": PEAK_MFMA[cfg.dtype], "unit": "TFLOP/s", "frac": ach / PEAK_MFMA[cfg.dtype],
+                "avg_launch_ms": k0, "traffic": traffic}
+    b = {"bf16": 2, "fp8": 1, "int8": 1}[cfg.dtype]
+    byt0 = res["active_experts"] * 2 * I * H * b + res["active_experts"] * 2 * I * 4 + T * H * b + res["post_pad"] * I * 2
+    ach = byt0 / k0 / 1e6
+    return {"kernel": "moe_gemm_kernel (gemm0: gate+up, SiLU*up)", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM,
+            "unit": "GB/s", "frac": ach / PEAK_HBM, "avg_launch_ms": k0, "traffic": traffic}
+
+
+def cpu_baseline(cfg, inp, max_rows=256):
+    """ck_tile's own host reference (oracle/_ref) timed on this machine's cores on a bounded
+    sample of the workload: every row routed to one expert (T'=rows, E'=1, K'=1), operands
+    de-quantised to fp32 because the reference ignores scale tensors.  Falls back to the C
+    restatement when oracle/_ref is not built."""
+    import numpy as np
+    import torch
+
+    import oracle
+
+    e0 = int(inp["topk_ids"][0, 0])
+    t_idx, k_idx = torch.nonzero(inp["topk_ids"] == e0, as_tuple=True)
+    t_idx, k_idx = t_idx[:max_rows], k_idx[:max_rows]
+    n = int(t_idx.numel())
+    H, I = cfg.hidden, cfg.inter
+
+    def deq(x, scale):
+        x = x.float()
+        return (x * scale[..., None]) if scale is not None else x
+
+    def rows(x, idx):  # row gather that also works for 8-bit float storage
+        return x.view(torch.uint8)[idx].view(x.dtype) if x.element_size() == 1 else x[idx]
+
+    a = deq(rows(inp["a"], t_idx), None if inp["a_scale"] is None else inp["a_scale"][t_idx]).cpu().numpy()
+    g = deq(inp["g"][e0], None if inp["g_scale"] is None else inp["g_scale"][e0]).cpu().numpy()[None]
+    d = deq(inp["d"][e0], None if inp["d_scale"] is None else inp["d_scale"][e0]).cpu().numpy()[None]
+    ids = np.zeros((n, 1), dtype=np.int32)
+    w = inp["topk_weight"][t_idx, k_idx].cpu().numpy().reshape(n, 1)
+    flops = 6.0 * n * H * I
+    sample = (f"the {n} rows routed to expert {e0} of {cfg.name} as a T'={n}, E'=1, K'=1 problem "
+              f"(same H={H}, I={I}), de-quantised fp32 operands")
+    if oracle.ck_ref() is not None:
+        t0 = time.perf_counter()
+        s = oracle.ck_moe_sorting(ids, w, 1, cfg.unit)
+        oracle.ck_fused_moe(a, g, d, *s, cfg.unit, n, 1, H, I, 1, f32_inputs=True)
+        dt = time.perf_counter() - t0
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "reference", "seconds": dt,
+                "sample": sample + "; ck_tile::reference_moe_sorting + reference_fused_moe (GEMM phase is "
+                "single-threaded by construction, the final top-k reduce uses all cores)"}
+    t0 = time.perf_counter()
+    s = oracle.moe_sorting(ids, w, 1, cfg.unit)
+    oracle.fused_moe(a, oracle.DT_F32, g, oracle.DT_F32, d, oracle.DT_F32, *s, cfg.unit, n, 1, H, I, 1)
+    dt = time.perf_counter() - t0
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+            "seconds": dt, "sample": sample + "; C restatement of the ck_tile reference (oracle/moe_oracle.c)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default=HEADLINE)
+    ap.add_argument("--headline-only", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build measures one GPU only; run with --gpus 1 (the path is single-GPU, "
+                 "how it would shard across GPUs is described in DESIGN.md)")
+    import torch
+
+    from therock_amd import inputs as mi
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    cfg = mi.CONFIGS[a.workload]
+    log(f"[bench] {cfg}")
+    res, inp, buf = run_workload(cfg, a.steps, a.warmup)
+    log(f"[bench] {cfg.name}: {res['ms_per_step']:.3f} ms/step, {res['tflops']:.1f} TFLOP/s, kernels {res['kernel_avg_ms']}")
+    roof = roofline_of(cfg, res)
+    cpu = None
+    if not a.no_cpu_baseline:
+        try:
+            cpu = cpu_baseline(cfg, inp)
+            log(f"[bench] cpu baseline: {cpu}")
+        except Exception as e:  # the baseline is a report, never a reason to lose the measurement
+            log(f"[bench] cpu baseline failed: {e!r}")
+    del inp, buf
+    torch.cuda.empty_cache()
+
+    others = {}
+    if not a.headline_only:
+        for name, c in mi.CONFIGS.items():
+            if name == cfg.name:
+                continue
+            try:
+                steps = max(5, a.steps // 2)
+                r, i2, b2 = run_workload(c, steps, a.warmup)
+                r["roofline"] = roofline_of(c, r)
+                others[name] = r
+                log(f"[bench] {name}: {r['ms_per_step']:.3f} ms/step, {r['tflops']:.1f} TFLOP/s, "
+                    f"{r['hbm_GBps']:.0f} GB/s, kernels {r['kernel_avg_ms']}")
+                del i2, b2
+                torch.cuda.empty_cache()
+            except Exception as e:
+                log(f"[bench] {name} failed: {e!r}")
+                others[name] = {"error": repr(e)}
+
+    line = {
+        "metric": METRIC, "value": res["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": {"bf16": "bf16", "fp8": "fp8_e4m3", "int8": "int8"}[cfg.dtype],
+        "data": "synthetic (seeded N(0,1) activations, N(0,0.02) weights, pre-quantised, resident in HBM)",
+        "config": {"workload": f"{cfg.name}: tokens={cfg.tokens} hidden={cfg.hidden} inter={cfg.inter} "
+                               f"experts={cfg.experts} topk={cfg.topk} block_m={cfg.unit} router={cfg.router}",
+                   "path": "moe_sorting + gemm0(gate,up,SiLU*up) + gemm1(down) + combine, one stream"},
+        "frac_of_mfma_peak": res["frac_mfma_peak"], "tokens_per_s": res["tokens_per_s"],
+        "hbm_GBps": res["hbm_GBps"], "kernel_avg_ms": res["kernel_avg_ms"], "gemm0_tflops": res["gemm0_tflops"],
+        "gemm1_tflops": res["gemm1_tflops"], "roofline": roof, "cpu_baseline": cpu, "workloads": others,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -179,6 +179,29 @@ int mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_
 int mi355_moe_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype,
                             void* q, void* scale, void* stream);
 
+/* ------------------------------------------------------------------------------ kernel timing
+ * Counterpart of ck_tile::stream_config::time_kernel_ (host/stream_config.hpp:29-39,
+ * host/kernel_launch.hpp:106-143): between _start and _stop every kernel the library launches is
+ * bracketed by HIP events on its own stream.  _stop waits for the events, adds the elapsed
+ * milliseconds and launch counts per kernel kind into ms[] / launches[] (MI355_MOE_NUM_KERNELS
+ * entries each) and switches timing off.  Process-wide, not re-entrant; for benchmarks only. */
+enum mi355_moe_kernel_kind
+{
+    MI355_MOE_K_SORT_ONESHOT = 0,
+    MI355_MOE_K_SORT_COUNT   = 1,
+    MI355_MOE_K_SORT_SCAN    = 2,
+    MI355_MOE_K_SORT_SCATTER = 3,
+    MI355_MOE_K_PREP         = 4,
+    MI355_MOE_K_GEMM0        = 5,
+    MI355_MOE_K_GEMM1        = 6,
+    MI355_MOE_K_COMBINE      = 7,
+    MI355_MOE_K_QUANT        = 8,
+    MI355_MOE_NUM_KERNELS    = 9
+};
+int mi355_moe_profile_start(void);
+int mi355_moe_profile_stop(double* ms, int32_t* launches);
+const char* mi355_moe_kernel_name(int32_t kind);
+
 const char* mi355_moe_last_error(void);
 int mi355_moe_version(void);
 

@@ -66,6 +66,9 @@ PROTOTYPES = {
     "mi355_fused_moe": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.c_void_p]),
     "mi355_moe_rowwise_quant": (C.c_int, [C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_int32, C.c_void_p,
                                           C.c_void_p, C.c_void_p]),
+    "mi355_moe_profile_start": (C.c_int, []),
+    "mi355_moe_profile_stop": (C.c_int, [C.POINTER(C.c_double), C.POINTER(C.c_int32)]),
+    "mi355_moe_kernel_name": (C.c_char_p, [C.c_int32]),
     "mi355_moe_last_error": (C.c_char_p, []),
     "mi355_moe_version": (C.c_int, []),
 }
@@ -87,6 +90,24 @@ def load():
             fn.restype, fn.argtypes = res, args
         _lib = lib
     return _lib
+
+
+NUM_KERNELS = 9
+
+
+def profile_start() -> None:
+    load().mi355_moe_profile_start()
+
+
+def profile_stop() -> dict:
+    """{kernel name: (total ms, launches)} for the kernels launched since profile_start()."""
+    lib = load()
+    ms = (C.c_double * NUM_KERNELS)()
+    n = (C.c_int32 * NUM_KERNELS)()
+    rc = lib.mi355_moe_profile_stop(ms, n)
+    if rc != OK:
+        raise RuntimeError(f"profile_stop failed ({rc}): {last_error()}")
+    return {lib.mi355_moe_kernel_name(k).decode(): (ms[k], n[k]) for k in range(NUM_KERNELS) if n[k] > 0}
 
 
 def last_error() -> str:

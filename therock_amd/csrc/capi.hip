@@ -4,6 +4,7 @@
 
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 namespace mi355 {
 
@@ -39,6 +40,53 @@ const DeviceInfo& device_info()
     return info[dev];
 }
 
+namespace {
+struct ProfileState
+{
+    bool enabled = false;
+    std::vector<hipEvent_t> pool; // events created so far
+    size_t used = 0;
+    struct Rec
+    {
+        int kind;
+        hipEvent_t e0, e1;
+    };
+    std::vector<Rec> recs;
+    hipEvent_t pending[MI355_MOE_NUM_KERNELS] = {};
+    hipEvent_t get()
+    {
+        if(used == pool.size())
+        {
+            hipEvent_t e = nullptr;
+            if(hipEventCreate(&e) != hipSuccess)
+                return nullptr;
+            pool.push_back(e);
+        }
+        return pool[used++];
+    }
+};
+ProfileState g_prof;
+} // namespace
+
+bool profiling_enabled() { return g_prof.enabled; }
+
+void profile_mark(int kind, hipStream_t stream, bool begin)
+{
+    if(kind < 0 || kind >= MI355_MOE_NUM_KERNELS)
+        return;
+    hipEvent_t e = g_prof.get();
+    if(e == nullptr)
+        return;
+    (void)hipEventRecord(e, stream);
+    if(begin)
+        g_prof.pending[kind] = e;
+    else if(g_prof.pending[kind] != nullptr)
+    {
+        g_prof.recs.push_back({kind, g_prof.pending[kind], e});
+        g_prof.pending[kind] = nullptr;
+    }
+}
+
 } // namespace mi355
 
 using namespace mi355;
@@ -48,6 +96,47 @@ extern "C" {
 __attribute__((visibility("default"))) const char* mi355_moe_last_error(void) { return error_buffer(); }
 
 __attribute__((visibility("default"))) int mi355_moe_version(void) { return MI355_MOE_VERSION; }
+
+__attribute__((visibility("default"))) const char* mi355_moe_kernel_name(int32_t kind)
+{
+    static const char* names[MI355_MOE_NUM_KERNELS] = {
+        "moe_sorting_oneshot", "moe_sorting_count", "moe_sorting_scan", "moe_sorting_scatter", "moe_prep",
+        "moe_gemm0_gate_up_silu", "moe_gemm1_down", "moe_combine", "rowwise_quant"};
+    return kind >= 0 && kind < MI355_MOE_NUM_KERNELS ? names[kind] : "?";
+}
+
+__attribute__((visibility("default"))) int mi355_moe_profile_start(void)
+{
+    g_prof.used = 0;
+    g_prof.recs.clear();
+    for(auto& p : g_prof.pending)
+        p = nullptr;
+    g_prof.enabled = true;
+    return MI355_MOE_OK;
+}
+
+__attribute__((visibility("default"))) int mi355_moe_profile_stop(double* ms, int32_t* launches)
+{
+    g_prof.enabled = false;
+    if(ms == nullptr || launches == nullptr)
+        return fail(MI355_MOE_E_INVALID, "profile_stop: null output");
+    for(int k = 0; k < MI355_MOE_NUM_KERNELS; k++)
+    {
+        ms[k]       = 0.0;
+        launches[k] = 0;
+    }
+    for(const auto& r : g_prof.recs)
+    {
+        MI355_HIP_TRY(hipEventSynchronize(r.e1));
+        float t = 0.f;
+        MI355_HIP_TRY(hipEventElapsedTime(&t, r.e0, r.e1));
+        ms[r.kind] += t;
+        launches[r.kind] += 1;
+    }
+    g_prof.recs.clear();
+    g_prof.used = 0;
+    return MI355_MOE_OK;
+}
 
 __attribute__((visibility("default"))) int64_t
 mi355_moe_max_num_tokens_padded(int32_t tokens, int32_t num_experts, int32_t topk, int32_t unit_size)

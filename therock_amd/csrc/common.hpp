@@ -51,6 +51,28 @@ struct DeviceInfo
 // cached per device (ck_tile queries hipGetDeviceProperties on every call)
 const DeviceInfo& device_info();
 
+// ---- optional per-kernel event timing (mi355_moe_profile_start / _stop)
+bool profiling_enabled();
+void profile_mark(int kind, hipStream_t stream, bool begin);
+
+// brackets one kernel launch with events while profiling is on
+struct KernelTimer
+{
+    int kind;
+    hipStream_t stream;
+    bool on;
+    KernelTimer(int k, hipStream_t s) : kind(k), stream(s), on(profiling_enabled())
+    {
+        if(on)
+            profile_mark(kind, stream, true);
+    }
+    ~KernelTimer()
+    {
+        if(on)
+            profile_mark(kind, stream, false);
+    }
+};
+
 // ---- sorting launcher shared by the stand-alone and the fused entry points
 // tile_* (optional, may be null): work list for the grouped GEMMs, built by the sort's scan
 int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream);

@@ -657,6 +657,7 @@ template <int MODE, bool GEMM0>
 int launch_gemm(int mblk, const GemmParams& p, int max_tiles, hipStream_t stream)
 {
     using MT = ModeTraits<MODE>;
+    KernelTimer timer(GEMM0 ? MI355_MOE_K_GEMM0 : MI355_MOE_K_GEMM1, stream);
     const int grid = round_up(max_tiles * p.n_ntiles, 8);
     if(grid <= 0)
         return MI355_MOE_OK;
@@ -763,9 +764,12 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
 
     const int n_valid    = T * K;
     const int prep_grid  = 1 + std::min(ceil_div(n_valid, kPrepBlock * 4), 64);
+    {
+    KernelTimer timer(MI355_MOE_K_PREP, stream);
     hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
                        static_cast<const int*>(a.sorted_expert_ids_ptr), static_cast<const int*>(a.num_sorted_tiles_ptr),
                        t.block_m, E, mblk * 32, max_units, ws.max_tiles, tile_map, valid, n_valid);
+    }
     MI355_HIP_TRY(hipGetLastError());
 
     GemmParams p{};
@@ -828,8 +832,11 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
         return rc;
 
     // ---- combine
+    {
+    KernelTimer timer(MI355_MOE_K_COMBINE, stream);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, valid,
                        static_cast<unsigned char*>(a.o_ptr), K, H, (int64_t)a.stride_token * 2);
+    }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }
@@ -845,6 +852,7 @@ int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stri
         return MI355_MOE_OK;
     if(rows > 0x7fffffff)
         return fail(MI355_MOE_E_INVALID, "rowwise_quant: too many rows");
+    KernelTimer timer(MI355_MOE_K_QUANT, stream);
     if(q_dtype == MI355_MOE_FP8)
         hipLaunchKernelGGL(rowwise_quant_kernel<true>, dim3((unsigned)rows), dim3(256), 0, stream,
                            static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),

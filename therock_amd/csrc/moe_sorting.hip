@@ -380,6 +380,7 @@ int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream)
     if(use_oneshot(n, p.E))
     {
         p.nseg = kScanWaves;
+        KernelTimer timer(MI355_MOE_K_SORT_ONESHOT, stream);
         hipLaunchKernelGGL(moe_sorting_oneshot_kernel, dim3(1 + zero_blocks), dim3(kScanBlock),
                            kScanWaves * p.E * sizeof(int), stream, p);
         MI355_HIP_TRY(hipGetLastError());
@@ -392,12 +393,21 @@ int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream)
     p.nseg        = (int)ceil_div<int64_t>(n, kSeg);
     p.work_blocks = ceil_div(p.nseg, kWalkBlock / kWave);
     const size_t lds = (kWalkBlock / kWave) * p.E * sizeof(int);
-    hipLaunchKernelGGL(moe_sorting_count_kernel, dim3(p.work_blocks + zero_blocks), dim3(kWalkBlock), lds,
-                       stream, p);
+    {
+        KernelTimer timer(MI355_MOE_K_SORT_COUNT, stream);
+        hipLaunchKernelGGL(moe_sorting_count_kernel, dim3(p.work_blocks + zero_blocks), dim3(kWalkBlock), lds,
+                           stream, p);
+    }
     MI355_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(moe_sorting_scan_kernel, dim3(1), dim3(kScanBlock), 0, stream, p);
+    {
+        KernelTimer timer(MI355_MOE_K_SORT_SCAN, stream);
+        hipLaunchKernelGGL(moe_sorting_scan_kernel, dim3(1), dim3(kScanBlock), 0, stream, p);
+    }
     MI355_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(moe_sorting_scatter_kernel, dim3(p.work_blocks), dim3(kWalkBlock), lds, stream, p);
+    {
+        KernelTimer timer(MI355_MOE_K_SORT_SCATTER, stream);
+        hipLaunchKernelGGL(moe_sorting_scatter_kernel, dim3(p.work_blocks), dim3(kWalkBlock), lds, stream, p);
+    }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }
