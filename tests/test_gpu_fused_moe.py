@@ -126,3 +126,13 @@ def test_traits_without_kernel_return_minus_one():
     args.ws_ptr = None
     with pytest.raises(RuntimeError, match="workspace"):
         ta.fused_moe(t, args)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+def test_large_tile_kernel(dtype):
+    # >= 160 rows per expert selects the 256-row tile kernel (global->LDS DMA ring): full tiles,
+    # ragged tiles, padding ids, column tails and a K depth that is not a multiple of the ring
+    check(mi.MoeConfig("b", 1024, 512, 384, 8, 2, dtype, "softmax_renorm"), seed=1)
+    check(mi.MoeConfig("b", 700, 320, 128, 4, 1, dtype, "softmax_renorm", unit=64), seed=2)
+    check(mi.MoeConfig("b", 2000, 192, 256, 6, 3, dtype, "zipf"), seed=3)
+    check(mi.MoeConfig("b", 600, 64, 128, 2, 1, dtype, "softmax_renorm"), seed=4)

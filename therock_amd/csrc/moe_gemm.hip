@@ -17,163 +17,13 @@
 // token tile and split the weight rows, which keeps the waves balanced for any number of rows.
 // Operand tiles are staged through LDS (16-byte padded rows, conflict-free ds_read_b128) with the
 // next K tile prefetched into registers while the current one feeds the MFMAs.
-#include "moe_gemm.hpp"
-#include "device_utils.hpp"
+#include "moe_gemm_device.hpp"
 
 #include <algorithm>
 
 namespace mi355 {
+using namespace gemm;
 namespace {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(16))) float f32x16_t;
-typedef __attribute__((ext_vector_type(16))) int i32x16_t;
-typedef __attribute__((ext_vector_type(4))) int i32x4_t;
-typedef __attribute__((ext_vector_type(8))) int i32x8_t;
-
-enum Mode
-{
-    kBf16   = 0, // x bf16, w bf16, bf16 MFMA
-    kFp8    = 1, // x e4m3, w e4m3, block-scaled f8f6f4 MFMA
-    kI8     = 2, // x int8, w int8, i8 MFMA (gemm0 only)
-    kBf16W8 = 3  // x bf16, w int8 converted to bf16 after the LDS read (gemm1 of the int8 path)
-};
-
-constexpr int kBlock   = 256;
-constexpr int kWRows   = 256; // weight rows per workgroup tile
-constexpr int kTileKB  = 128; // bytes of K per row of the x tile
-constexpr int kPadB    = 16;
-constexpr int kMapHdr  = 4;   // ints in front of the tile entries
-constexpr int kMapEnt  = 8;   // ints per tile entry: expert,row0,nrows,first,ntiles,0,0,0
-
-struct GemmParams
-{
-    const unsigned char* x;  // gemm0: activations [tokens, x_row_bytes]; gemm1: Y [rows, x_row_bytes]
-    const unsigned char* w;  // [experts, n_total, k] K contiguous
-    const float* x_scale;    // gemm0: per-token scale or null
-    const float* w_scale;    // [experts, n_total] or null
-    const int* sorted_ids;
-    const float* sorted_w;
-    const int* tile_map;
-    unsigned char* out;      // gemm0: Y; gemm1: P
-    unsigned char* y_scale;  // e8m0 block scales of Y (fp8 path): written by gemm0, read by gemm1
-    int* valid;              // gemm1: flags per (token, slot)
-    int64_t x_row_bytes;
-    int64_t w_row_bytes;
-    int64_t w_expert_bytes;
-    int64_t out_row_bytes;
-    int64_t ys_row_bytes;
-    int k_bytes_x;           // bytes of K in a row of x
-    int k_bytes_w;           // bytes of K in a row of w
-    int n_out;               // gemm0: inter; gemm1: hidden
-    int n_total;             // weight rows per expert (gemm0: 2*inter, gemm1: hidden)
-    int n_ntiles;            // tiles along n
-    int tokens;
-    int topk;
-};
-
-template <int MODE>
-struct ModeTraits;
-template <>
-struct ModeTraits<kBf16>
-{
-    using Acc                  = f32x16_t;
-    static constexpr int kOpB  = 16; // operand bytes per lane per MFMA
-    static constexpr int kWKB  = 128;
-};
-template <>
-struct ModeTraits<kFp8>
-{
-    using Acc                  = f32x16_t;
-    static constexpr int kOpB  = 32;
-    static constexpr int kWKB  = 128;
-};
-template <>
-struct ModeTraits<kI8>
-{
-    using Acc                  = i32x16_t;
-    static constexpr int kOpB  = 16;
-    static constexpr int kWKB  = 128;
-};
-template <>
-struct ModeTraits<kBf16W8>
-{
-    using Acc                  = f32x16_t;
-    static constexpr int kOpB  = 16;
-    static constexpr int kWKB  = 64; // int8 weights: 64 K elements per tile row
-};
-
-// MFMA row m of a 32-row weight block holds weight channel chan_of_row(m); with the 32x32
-// accumulator layout (register v = 4j+i of lane l is row 8j + 4(l/32) + i) lane l then owns the 16
-// consecutive channels 16*(l/32) .. +15 of its token in registers 0..15.
-__device__ __host__ constexpr int chan_of_row(int m) { return 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3); }
-
-__device__ inline float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
-
-// 8 int8 (two dwords) -> 8 bf16 (exact: |v| <= 128 fits bf16's 8 significant bits)
-__device__ inline uint4 int8x8_to_bf16x8(uint2 v)
-{
-    uint4 r;
-    uint32_t d[2] = {v.x, v.y};
-    uint32_t o[4];
-#pragma unroll
-    for(int h = 0; h < 2; h++)
-    {
-        const int s = static_cast<int>(d[h]);
-        const uint32_t f0 = __float_as_uint(static_cast<float>((s << 24) >> 24));
-        const uint32_t f1 = __float_as_uint(static_cast<float>((s << 16) >> 24));
-        const uint32_t f2 = __float_as_uint(static_cast<float>((s << 8) >> 24));
-        const uint32_t f3 = __float_as_uint(static_cast<float>(s >> 24));
-        o[2 * h]     = (f1 & 0xffff0000u) | (f0 >> 16);
-        o[2 * h + 1] = (f3 & 0xffff0000u) | (f2 >> 16);
-    }
-    r.x = o[0];
-    r.y = o[1];
-    r.z = o[2];
-    r.w = o[3];
-    return r;
-}
-
-template <typename To, typename From>
-__device__ inline To bit_cast_dev(const From& f)
-{
-    static_assert(sizeof(To) == sizeof(From), "size mismatch");
-    To t;
-    __builtin_memcpy(&t, &f, sizeof(To));
-    return t;
-}
-
-struct Frag
-{
-    uint4 lo, hi; // hi only used by 32-byte operands
-};
-
-template <int MODE>
-__device__ inline typename ModeTraits<MODE>::Acc mfma(const Frag& w, const Frag& x, uint32_t x_scale,
-                                                      typename ModeTraits<MODE>::Acc c)
-{
-    if constexpr(MODE == kBf16 || MODE == kBf16W8)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(bit_cast_dev<bf16x8_t>(w.lo), bit_cast_dev<bf16x8_t>(x.lo), c,
-                                                       0, 0, 0);
-    }
-    else if constexpr(MODE == kI8)
-    {
-        return __builtin_amdgcn_mfma_i32_32x32x32_i8(bit_cast_dev<i32x4_t>(w.lo), bit_cast_dev<i32x4_t>(x.lo), c, 0,
-                                                     0, 0);
-    }
-    else
-    {
-        i32x8_t a, b;
-        a[0] = w.lo.x; a[1] = w.lo.y; a[2] = w.lo.z; a[3] = w.lo.w;
-        a[4] = w.hi.x; a[5] = w.hi.y; a[6] = w.hi.z; a[7] = w.hi.w;
-        b[0] = x.lo.x; b[1] = x.lo.y; b[2] = x.lo.z; b[3] = x.lo.w;
-        b[4] = x.hi.x; b[5] = x.hi.y; b[6] = x.hi.z; b[7] = x.hi.w;
-        // cbsz = blgp = 0: both operands e4m3; weights carry the unit block scale 2^0 (e8m0 127),
-        // the token operand its per-32 block scale in byte 0 (op_sel 0)
-        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 127, 0, static_cast<int>(x_scale));
-    }
-}
 
 // ---------------------------------------------------------------------------------------------
 // GEMM0 : MODE in {kBf16, kFp8, kI8};  GEMM1 : MODE in {kBf16, kFp8, kBf16W8}
@@ -305,7 +155,11 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
                 ys_next[j] = 0x7f7f7f7fu;
                 const int r = j * 32 + r32;
                 if(r < nrows)
-                    ys_next[j] = *reinterpret_cast<const uint32_t*>(p.y_scale + (int64_t)(row0 + r) * p.ys_row_bytes + kt * 4);
+                {
+                    const unsigned char* sp = p.y_scale + (int64_t)(kt * 4) * p.ys_kb_stride + row0 + r;
+                    ys_next[j] = sp[0] | (sp[p.ys_kb_stride] << 8) | (sp[2 * p.ys_kb_stride] << 16) |
+                                 (static_cast<uint32_t>(sp[3 * p.ys_kb_stride]) << 24);
+                }
             }
         }
     };
@@ -394,110 +248,28 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
     {
         if(j >= nmb)
             continue;
-        const int r = j * 32 + r32;
-        if(r >= nrows)
-            continue;
-        const int sid   = p.sorted_ids[row0 + r];
-        const int tok   = sid & 0xffffff;
-        const bool real = tok < p.tokens;
+        const int r        = j * 32 + r32;
+        const bool in_tile = r < nrows;
+        const int sid      = in_tile ? p.sorted_ids[row0 + r] : p.tokens;
+        const int tok      = sid & 0xffffff;
         if constexpr(GEMM0)
         {
-            const int col0 = n_base + wave * 32 + 16 * kg; // first Y column of this lane
-            if(n_base + wave * 32 >= p.n_out)
-                continue;
-            float y[16];
-            float sa = 1.0f;
-            if(p.x_scale != nullptr)
-                sa = real ? p.x_scale[tok] : 0.0f;
-            const float* gs = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total + col0 : nullptr;
-#pragma unroll
-            for(int v = 0; v < 16; v++)
-            {
-                float g = static_cast<float>(acc[j][0][v]);
-                float u = static_cast<float>(acc[j][1][v]);
-                if(gs != nullptr)
-                {
-                    g *= sa * gs[v];
-                    u *= sa * gs[p.n_out + v];
-                }
-                y[v] = silu(g) * u;
-            }
-            unsigned char* dst = p.out + (int64_t)(row0 + r) * p.out_row_bytes;
-            if constexpr(MODE == kFp8)
-            {
-                // e4m3 with one power-of-two scale per 32 columns (this lane's 16 + lane^32's 16)
-                float amax = 0.f;
-#pragma unroll
-                for(int v = 0; v < 16; v++)
-                    amax = fmaxf(amax, fabsf(y[v]));
-                amax = fmaxf(amax, __shfl_xor(amax, 32));
-                const uint32_t ab = __float_as_uint(amax);
-                int sb            = static_cast<int>(ab >> 23) - 8 + ((ab & 0x7fffffu) > 0x600000u ? 1 : 0);
-                sb                = amax == 0.f ? 0 : max(0, min(254, sb));
-                const float inv   = __uint_as_float(static_cast<uint32_t>(254 - sb) << 23);
-                uint32_t q[4];
-#pragma unroll
-                for(int v = 0; v < 4; v++)
-                {
-                    float a0 = fminf(fmaxf(y[4 * v] * inv, -448.f), 448.f);
-                    float a1 = fminf(fmaxf(y[4 * v + 1] * inv, -448.f), 448.f);
-                    float a2 = fminf(fmaxf(y[4 * v + 2] * inv, -448.f), 448.f);
-                    float a3 = fminf(fmaxf(y[4 * v + 3] * inv, -448.f), 448.f);
-                    int pk   = __builtin_amdgcn_cvt_pk_fp8_f32(a0, a1, 0, false);
-                    pk       = __builtin_amdgcn_cvt_pk_fp8_f32(a2, a3, pk, true);
-                    q[v]     = static_cast<uint32_t>(pk);
-                }
-                *reinterpret_cast<uint4*>(dst + col0) = make_uint4(q[0], q[1], q[2], q[3]);
-                if(kg == 0)
-                    p.y_scale[(int64_t)(row0 + r) * p.ys_row_bytes + (col0 >> 5)] = static_cast<unsigned char>(sb);
-            }
-            else
-            {
-                uint4 o0, o1;
-                o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
-                o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
-                o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
-                o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
-                uint4* d4 = reinterpret_cast<uint4*>(dst + (int64_t)col0 * 2);
-                d4[0] = o0;
-                d4[1] = o1;
-            }
+            if(n_base + wave * 32 < p.n_out)
+                epilogue_gemm0<MODE>(p, acc[j][0], acc[j][1], expert, row0 + r, tok, in_tile,
+                                     n_base + wave * 32 + 16 * kg, kg);
         }
         else
         {
-            if(!real)
+            if(!in_tile || tok >= p.tokens)
                 continue;
-            const int slot_k  = static_cast<int>(static_cast<uint32_t>(sid) >> 24);
-            const int64_t prow = (int64_t)tok * p.topk + slot_k;
-            const float tw    = p.sorted_w[row0 + r];
+            const int64_t prow = (int64_t)tok * p.topk + static_cast<int>(static_cast<uint32_t>(sid) >> 24);
+            const float tw     = p.sorted_w[row0 + r];
             if(nt == 0 && wave == 0 && kg == 0)
                 p.valid[prow] = 1;
-            unsigned char* dst = p.out + prow * p.out_row_bytes;
 #pragma unroll
             for(int b = 0; b < 2; b++)
-            {
-                const int col0 = n_base + (wave * 2 + b) * 32 + 16 * kg;
-                if(n_base + (wave * 2 + b) * 32 >= p.n_out)
-                    continue;
-                const float* ds = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total + col0 : nullptr;
-                float y[16];
-#pragma unroll
-                for(int v = 0; v < 16; v++)
-                {
-                    float o = static_cast<float>(acc[j][b][v]);
-                    if(ds != nullptr)
-                        o *= ds[v];
-                    y[v] = o * tw;
-                }
-                uint4 o0, o1;
-                o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
-                o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
-                o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
-                o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
-                uint4* d4 = reinterpret_cast<uint4*>(dst + (int64_t)col0 * 2);
-                d4[0] = o0;
-                d4[1] = o1;
-            }
+                if(n_base + (wave * 2 + b) * 32 < p.n_out)
+                    epilogue_gemm1<MODE>(p, acc[j][b], expert, prow, tw, n_base + (wave * 2 + b) * 32 + 16 * kg);
         }
     }
 }
@@ -526,12 +298,15 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
                                                                const int* __restrict__ post_pad_ptr, int unit,
                                                                int experts, int rows_per_tile, int max_units,
                                                                int max_tiles, int* __restrict__ tile_map,
-                                                               int* __restrict__ valid, int n_valid)
+                                                               int* __restrict__ valid, int n_valid,
+                                                               int* __restrict__ zero_page)
 {
     for(int i = blockIdx.x * kPrepBlock + threadIdx.x; i < n_valid; i += gridDim.x * kPrepBlock)
         valid[i] = 0;
     if(blockIdx.x != 0)
         return;
+    if(threadIdx.x < 64)
+        zero_page[threadIdx.x] = 0;
     __shared__ int s_wave[kPrepWaves + 1];
     const int post_pad = post_pad_ptr[0];
     int nunits         = post_pad / unit;
@@ -643,13 +418,19 @@ __global__ __launch_bounds__(256) void rowwise_quant_kernel(const uint16_t* __re
     }
 }
 
-inline int pick_mblk(int64_t tokens, int topk, int experts)
+// 32-row blocks per M tile, from the expected rows per expert; big_tile_rows()/32 selects the
+// large-tile kernel
+inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
 {
     const int64_t avg = tokens * topk / experts;
     if(avg <= 32)
         return 1;
     if(avg <= 64)
         return 2;
+    const int eb  = t.prec_i == MI355_MOE_BF16 ? 2 : 1;
+    const int y_b = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
+    if(avg >= 160 && t.block_m % 4 == 0 && big_tile_supported(t.prec_i, hidden * eb, inter * y_b))
+        return big_tile_rows() / 32;
     return 4;
 }
 
@@ -708,7 +489,7 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
         w.total += round_up<size_t>(bytes, 256);
         return off;
     };
-    const int mblk   = pick_mblk(tokens, topk, experts);
+    const int mblk   = pick_mblk(t, tokens, topk, experts, hidden, inter);
     w.max_pad        = (int64_t)topk * tokens + (int64_t)experts * t.block_m - topk;
     w.max_tiles      = (int32_t)(experts + w.max_pad / (mblk * 32) + 1);
     const int y_b    = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
@@ -716,7 +497,9 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
     w.map_off        = bump(sizeof(int) * (kMapHdr + (size_t)kMapEnt * w.max_tiles));
     w.valid_off      = bump(sizeof(int) * (size_t)tokens * topk);
     w.y_off          = bump((size_t)w.max_pad * inter * y_b);
-    w.ys_off         = bump(t.prec_i == MI355_MOE_FP8 ? (size_t)w.max_pad * (inter / 32) : 0);
+    w.ys_kb_stride   = round_up<int64_t>(w.max_pad, 256) + 512;
+    w.ys_off         = bump(t.prec_i == MI355_MOE_FP8 ? (size_t)w.ys_kb_stride * (inter / 32) : 0);
+    w.zero_off       = bump(256);
     w.p_off          = bump((size_t)tokens * topk * hidden * 2);
     return w;
 }
@@ -759,7 +542,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     unsigned char* wsb = static_cast<unsigned char*>(a.ws_ptr);
     int* tile_map      = reinterpret_cast<int*>(wsb + ws.map_off);
     int* valid         = reinterpret_cast<int*>(wsb + ws.valid_off);
-    const int mblk     = pick_mblk(T, K, E);
+    const int mblk     = pick_mblk(t, T, K, E, H, I);
     const int max_units = (int)ceil_div<int64_t>(ws.max_pad, t.block_m);
 
     const int n_valid    = T * K;
@@ -768,7 +551,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     KernelTimer timer(MI355_MOE_K_PREP, stream);
     hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
                        static_cast<const int*>(a.sorted_expert_ids_ptr), static_cast<const int*>(a.num_sorted_tiles_ptr),
-                       t.block_m, E, mblk * 32, max_units, ws.max_tiles, tile_map, valid, n_valid);
+                       t.block_m, E, mblk * 32, max_units, ws.max_tiles, tile_map, valid, n_valid,
+                       reinterpret_cast<int*>(wsb + ws.zero_off));
     }
     MI355_HIP_TRY(hipGetLastError());
 
@@ -780,7 +564,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.tokens     = T;
     p.topk       = K;
     p.y_scale    = wsb + ws.ys_off;
-    p.ys_row_bytes = I / 32;
+    p.ys_kb_stride = ws.ys_kb_stride;
+    p.zero_page    = wsb + ws.zero_off;
 
     // ---- gemm0: gate+up, SiLU*up
     const int y_b     = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
@@ -798,7 +583,9 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.n_out           = I;
     p.n_total         = 2 * I;
     p.n_ntiles        = ceil_div(I, 128);
-    if(t.prec_i == MI355_MOE_BF16)
+    if(mblk > 4)
+        rc = launch_gemm_big(t.prec_i, true, p, ws.max_tiles, stream);
+    else if(t.prec_i == MI355_MOE_BF16)
         rc = launch_gemm<kBf16, true>(mblk, p, ws.max_tiles, stream);
     else if(t.prec_i == MI355_MOE_FP8)
         rc = launch_gemm<kFp8, true>(mblk, p, ws.max_tiles, stream);
@@ -822,7 +609,9 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.n_out          = H;
     p.n_total        = H;
     p.n_ntiles       = ceil_div(H, 256);
-    if(t.prec_i == MI355_MOE_BF16)
+    if(mblk > 4)
+        rc = launch_gemm_big(t.prec_i, false, p, ws.max_tiles, stream);
+    else if(t.prec_i == MI355_MOE_BF16)
         rc = launch_gemm<kBf16, false>(mblk, p, ws.max_tiles, stream);
     else if(t.prec_i == MI355_MOE_FP8)
         rc = launch_gemm<kFp8, false>(mblk, p, ws.max_tiles, stream);

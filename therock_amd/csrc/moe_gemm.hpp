@@ -12,7 +12,9 @@ struct WorkspaceLayout
     size_t map_off;    // int32 [4 + 8 * max_tiles]: live tile count, then one entry per M tile
     size_t valid_off;  // int32 [tokens * topk]: 1 where the (token, slot) partial was produced
     size_t y_off;      // intermediate activations Y [max_pad, inter] (bf16 or e4m3)
-    size_t ys_off;     // e8m0 block scales of Y [max_pad, inter / 32] (fp8 path only)
+    size_t ys_off;     // e8m0 block scales of Y [inter / 32][ys_kb_stride] (fp8 path only)
+    size_t zero_off;   // 256 zero bytes
+    int64_t ys_kb_stride;
     size_t p_off;      // per-slot partial outputs [tokens * topk, hidden] bf16
     size_t total;
     int64_t max_pad;
@@ -26,6 +28,14 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
 
 int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a,
                          hipStream_t stream);
+
+namespace gemm {
+struct GemmParams;
+}
+// large-tile kernel (moe_gemm_big.hip)
+int big_tile_rows();
+bool big_tile_supported(int prec, int k_bytes0, int k_bytes1);
+int launch_gemm_big(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream);
 
 int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype,
                          void* q, void* scale, hipStream_t stream);

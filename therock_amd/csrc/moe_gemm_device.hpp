@@ -1,0 +1,276 @@
+// Device code shared by the grouped-GEMM kernels: operand types, MFMA wrappers, the per-lane
+// epilogues (scales, SiLU*up, packing) and the kernel parameter block.
+#pragma once
+
+#include "moe_gemm.hpp"
+#include "device_utils.hpp"
+
+namespace mi355 {
+namespace gemm {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(16))) int i32x16_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+
+enum Mode
+{
+    kBf16   = 0, // x bf16, w bf16, bf16 MFMA
+    kFp8    = 1, // x e4m3, w e4m3, block-scaled f8f6f4 MFMA
+    kI8     = 2, // x int8, w int8, i8 MFMA (gemm0 only)
+    kBf16W8 = 3  // x bf16, w int8 converted to bf16 after the LDS read (gemm1 of the int8 path)
+};
+
+constexpr int kBlock   = 256;
+constexpr int kWRows   = 256; // weight rows per workgroup tile
+constexpr int kTileKB  = 128; // bytes of K per row of the x tile
+constexpr int kPadB    = 16;
+constexpr int kMapHdr  = 4;   // ints in front of the tile entries
+constexpr int kMapEnt  = 8;   // ints per tile entry: expert,row0,nrows,first,ntiles,0,0,0
+
+struct GemmParams
+{
+    const unsigned char* x;  // gemm0: activations [tokens, x_row_bytes]; gemm1: Y [rows, x_row_bytes]
+    const unsigned char* w;  // [experts, n_total, k] K contiguous
+    const float* x_scale;    // gemm0: per-token scale or null
+    const float* w_scale;    // [experts, n_total] or null
+    const int* sorted_ids;
+    const float* sorted_w;
+    const int* tile_map;
+    unsigned char* out;      // gemm0: Y; gemm1: P
+    unsigned char* y_scale;  // e8m0 block scales of Y (fp8 path): written by gemm0, read by gemm1
+    int* valid;              // gemm1: flags per (token, slot)
+    int64_t x_row_bytes;
+    int64_t w_row_bytes;
+    int64_t w_expert_bytes;
+    int64_t out_row_bytes;
+    int64_t ys_kb_stride;    // bytes between consecutive 32-column blocks of y_scale ([inter/32][rows])
+    const unsigned char* zero_page; // >= 256 zero bytes (rows that must read as zero)
+    int k_bytes_x;           // bytes of K in a row of x
+    int k_bytes_w;           // bytes of K in a row of w
+    int n_out;               // gemm0: inter; gemm1: hidden
+    int n_total;             // weight rows per expert (gemm0: 2*inter, gemm1: hidden)
+    int n_ntiles;            // tiles along n
+    int tokens;
+    int topk;
+    int debug; // experiments only: bit0 = no DMA after the first stage, bit1 = no MFMA work
+};
+
+template <int MODE>
+struct ModeTraits;
+template <>
+struct ModeTraits<kBf16>
+{
+    using Acc                  = f32x16_t;
+    static constexpr int kOpB  = 16; // operand bytes per lane per MFMA
+    static constexpr int kWKB  = 128;
+};
+template <>
+struct ModeTraits<kFp8>
+{
+    using Acc                  = f32x16_t;
+    static constexpr int kOpB  = 32;
+    static constexpr int kWKB  = 128;
+};
+template <>
+struct ModeTraits<kI8>
+{
+    using Acc                  = i32x16_t;
+    static constexpr int kOpB  = 16;
+    static constexpr int kWKB  = 128;
+};
+template <>
+struct ModeTraits<kBf16W8>
+{
+    using Acc                  = f32x16_t;
+    static constexpr int kOpB  = 16;
+    static constexpr int kWKB  = 64; // int8 weights: 64 K elements per tile row
+};
+
+// MFMA row m of a 32-row weight block holds weight channel chan_of_row(m); with the 32x32
+// accumulator layout (register v = 4j+i of lane l is row 8j + 4(l/32) + i) lane l then owns the 16
+// consecutive channels 16*(l/32) .. +15 of its token in registers 0..15.
+__device__ __host__ constexpr int chan_of_row(int m) { return 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3); }
+
+__device__ inline float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+
+// 8 int8 (two dwords) -> 8 bf16 (exact: |v| <= 128 fits bf16's 8 significant bits)
+__device__ inline uint4 int8x8_to_bf16x8(uint2 v)
+{
+    uint4 r;
+    uint32_t d[2] = {v.x, v.y};
+    uint32_t o[4];
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+    {
+        const int s = static_cast<int>(d[h]);
+        const uint32_t f0 = __float_as_uint(static_cast<float>((s << 24) >> 24));
+        const uint32_t f1 = __float_as_uint(static_cast<float>((s << 16) >> 24));
+        const uint32_t f2 = __float_as_uint(static_cast<float>((s << 8) >> 24));
+        const uint32_t f3 = __float_as_uint(static_cast<float>(s >> 24));
+        o[2 * h]     = (f1 & 0xffff0000u) | (f0 >> 16);
+        o[2 * h + 1] = (f3 & 0xffff0000u) | (f2 >> 16);
+    }
+    r.x = o[0];
+    r.y = o[1];
+    r.z = o[2];
+    r.w = o[3];
+    return r;
+}
+
+template <typename To, typename From>
+__device__ inline To bit_cast_dev(const From& f)
+{
+    static_assert(sizeof(To) == sizeof(From), "size mismatch");
+    To t;
+    __builtin_memcpy(&t, &f, sizeof(To));
+    return t;
+}
+
+struct Frag
+{
+    uint4 lo, hi; // hi only used by 32-byte operands
+};
+
+template <int MODE>
+__device__ inline typename ModeTraits<MODE>::Acc mfma(const Frag& w, const Frag& x, uint32_t x_scale,
+                                                      typename ModeTraits<MODE>::Acc c)
+{
+    if constexpr(MODE == kBf16 || MODE == kBf16W8)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(bit_cast_dev<bf16x8_t>(w.lo), bit_cast_dev<bf16x8_t>(x.lo), c,
+                                                       0, 0, 0);
+    }
+    else if constexpr(MODE == kI8)
+    {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(bit_cast_dev<i32x4_t>(w.lo), bit_cast_dev<i32x4_t>(x.lo), c, 0,
+                                                     0, 0);
+    }
+    else
+    {
+        i32x8_t a, b;
+        a[0] = w.lo.x; a[1] = w.lo.y; a[2] = w.lo.z; a[3] = w.lo.w;
+        a[4] = w.hi.x; a[5] = w.hi.y; a[6] = w.hi.z; a[7] = w.hi.w;
+        b[0] = x.lo.x; b[1] = x.lo.y; b[2] = x.lo.z; b[3] = x.lo.w;
+        b[4] = x.hi.x; b[5] = x.hi.y; b[6] = x.hi.z; b[7] = x.hi.w;
+        // cbsz = blgp = 0: both operands e4m3; weights carry the unit block scale 2^0 (e8m0 127),
+        // the token operand its per-32 block scale in byte 0 (op_sel 0)
+        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 127, 0, static_cast<int>(x_scale));
+    }
+}
+
+
+// e4m3 x e4m3 without block scales (both scale operands literal 0 select the unscaled encoding,
+// which issues faster than the scaled one)
+__device__ inline f32x16_t mfma_fp8_unscaled(const Frag& w, const Frag& x, f32x16_t c)
+{
+    i32x8_t a, b;
+    a[0] = w.lo.x; a[1] = w.lo.y; a[2] = w.lo.z; a[3] = w.lo.w;
+    a[4] = w.hi.x; a[5] = w.hi.y; a[6] = w.hi.z; a[7] = w.hi.w;
+    b[0] = x.lo.x; b[1] = x.lo.y; b[2] = x.lo.z; b[3] = x.lo.w;
+    b[4] = x.hi.x; b[5] = x.hi.y; b[6] = x.hi.z; b[7] = x.hi.w;
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Epilogues.  With the weight rows on the MFMA's M side and chan_of_row(), a lane holds, for the
+// token in column (lane % 32), the 16 consecutive output channels col0 .. col0+15 in acc[0..15].
+
+// gemm0: y = silu(gate) * up with the per-token and per-channel scales folded in; stored as bf16
+// or (fp8 path) as e4m3 with one power-of-two scale per 32 columns.  Every lane of the wave must
+// call it (the fp8 path exchanges the block maximum with lane ^ 32); `store` masks the writes.
+template <int MODE>
+__device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc_gate,
+                                      const typename ModeTraits<MODE>::Acc& acc_up, int expert, int64_t grow,
+                                      int token, bool store, int col0, int kg)
+{
+    float y[16];
+    float sa = 1.0f;
+    if(p.x_scale != nullptr)
+        sa = (store && token < p.tokens) ? p.x_scale[token] : 0.0f;
+    const float* gs = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total + col0 : nullptr;
+#pragma unroll
+    for(int v = 0; v < 16; v++)
+    {
+        float g = static_cast<float>(acc_gate[v]);
+        float u = static_cast<float>(acc_up[v]);
+        if(gs != nullptr)
+        {
+            g *= sa * gs[v];
+            u *= sa * gs[p.n_out + v];
+        }
+        y[v] = silu(g) * u;
+    }
+    unsigned char* dst = p.out + grow * p.out_row_bytes;
+    if constexpr(MODE == kFp8)
+    {
+        float amax = 0.f;
+#pragma unroll
+        for(int v = 0; v < 16; v++)
+            amax = fmaxf(amax, fabsf(y[v]));
+        amax = fmaxf(amax, __shfl_xor(amax, 32));
+        // scale 2^s with amax / 2^s <= 448 = 1.75 * 2^8; stored as e8m0 (s + 127)
+        const uint32_t ab = __float_as_uint(amax);
+        int sb            = static_cast<int>(ab >> 23) - 8 + ((ab & 0x7fffffu) > 0x600000u ? 1 : 0);
+        sb                = amax == 0.f ? 0 : max(0, min(254, sb));
+        const float inv   = __uint_as_float(static_cast<uint32_t>(254 - sb) << 23);
+        uint32_t q[4];
+#pragma unroll
+        for(int v = 0; v < 4; v++)
+        {
+            const float a0 = fminf(fmaxf(y[4 * v] * inv, -448.f), 448.f);
+            const float a1 = fminf(fmaxf(y[4 * v + 1] * inv, -448.f), 448.f);
+            const float a2 = fminf(fmaxf(y[4 * v + 2] * inv, -448.f), 448.f);
+            const float a3 = fminf(fmaxf(y[4 * v + 3] * inv, -448.f), 448.f);
+            int pk         = __builtin_amdgcn_cvt_pk_fp8_f32(a0, a1, 0, false);
+            pk             = __builtin_amdgcn_cvt_pk_fp8_f32(a2, a3, pk, true);
+            q[v]           = static_cast<uint32_t>(pk);
+        }
+        if(store)
+        {
+            *reinterpret_cast<uint4*>(dst + col0) = make_uint4(q[0], q[1], q[2], q[3]);
+            if(kg == 0)
+                p.y_scale[(int64_t)(col0 >> 5) * p.ys_kb_stride + grow] = static_cast<unsigned char>(sb);
+        }
+    }
+    else if(store)
+    {
+        uint4 o0, o1;
+        o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
+        o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
+        o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
+        o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
+        uint4* d4 = reinterpret_cast<uint4*>(dst + (int64_t)col0 * 2);
+        d4[0]     = o0;
+        d4[1]     = o1;
+    }
+}
+
+// gemm1: * per-channel scale * top-k weight, bf16 partial row (token * topk + slot)
+template <int MODE>
+__device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc, int expert,
+                                      int64_t prow, float topk_weight, int col0)
+{
+    const float* ds = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total + col0 : nullptr;
+    float y[16];
+#pragma unroll
+    for(int v = 0; v < 16; v++)
+    {
+        float o = static_cast<float>(acc[v]);
+        if(ds != nullptr)
+            o *= ds[v];
+        y[v] = o * topk_weight;
+    }
+    uint4 o0, o1;
+    o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
+    o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
+    o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
+    o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
+    uint4* d4 = reinterpret_cast<uint4*>(p.out + prow * p.out_row_bytes + (int64_t)col0 * 2);
+    d4[0]     = o0;
+    d4[1]     = o1;
+}
+
+} // namespace gemm
+} // namespace mi355
