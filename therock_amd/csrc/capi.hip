@@ -214,7 +214,9 @@ mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args
     s.topk                    = a->topk;
     if(traits->local_expert_masking && a->local_expert_mask_ptr == nullptr)
         return fail(MI355_MOE_E_INVALID, "fused_moe: local_expert_masking set but mask pointer is null");
-    rc = launch_moe_sorting(s, static_cast<hipStream_t>(stream));
+    const GemmPlan plan = make_gemm_plan(*traits, a->ws_ptr, a->num_tokens, a->num_experts, a->topk, a->hidden_size,
+                                         a->intermediate_size);
+    rc = launch_moe_sorting(s, static_cast<hipStream_t>(stream), &plan);
     if(rc != MI355_MOE_OK)
         return rc;
 
@@ -239,7 +241,7 @@ mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args
     g.num_experts           = a->num_experts;
     g.topk                  = a->topk;
     g.stride_token          = a->stride_token;
-    return launch_fused_moegemm(*traits, g, static_cast<hipStream_t>(stream));
+    return launch_fused_moegemm(*traits, g, static_cast<hipStream_t>(stream), /*prep_done=*/true);
 }
 
 __attribute__((visibility("default"))) int

@@ -73,9 +73,24 @@ struct KernelTimer
     }
 };
 
+// ---- work list of the grouped GEMMs: int32 [kMapHdr + kMapEnt * max_tiles]; [0] = live tiles, then per
+// tile (local expert id, first sorted row, rows, first tile of the expert, tiles of the expert, 0, 0, 0)
+constexpr int kMapHdr = 4;
+constexpr int kMapEnt = 8;
+
+// what the sort can prepare for the GEMMs while it has the per-expert counts at hand
+struct GemmPlan
+{
+    int* tile_map;     // work list, see above
+    int rows_per_tile; // sorted rows per GEMM tile (multiple of 32)
+    int max_tiles;     // capacity of tile_map
+    int* valid;        // [n_valid] flags to clear
+    int n_valid;
+    int* zero_page;    // 64 ints to clear
+};
+
 // ---- sorting launcher shared by the stand-alone and the fused entry points
-// tile_* (optional, may be null): work list for the grouped GEMMs, built by the sort's scan
-int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream);
+int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, const GemmPlan* plan = nullptr);
 
 size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk);
 

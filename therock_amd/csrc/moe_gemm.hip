@@ -34,9 +34,13 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
     using Acc = typename MT::Acc;
     constexpr int kOpB     = MT::kOpB;
     constexpr int kWKB     = MT::kWKB;
-    constexpr int kXStride = kTileKB + kPadB;
+    constexpr int kXKB     = MT::kXKB; // bytes of K per row of the token tile
+    constexpr int kXStride = kXKB + kPadB;
     constexpr int kWStride = kWKB + kPadB;
-    constexpr int kSteps   = kTileKB / (2 * kOpB); // MFMAs along K per tile
+    constexpr int kSteps   = kXKB / (2 * kOpB); // MFMAs along K per tile
+    constexpr int kXChunks = kXKB / 16;
+    constexpr int kXRowsPerPass = kBlock / kXChunks;
+    constexpr int kXLoads  = MBLK * 32 / kXRowsPerPass;
     constexpr int kWChunks = kWKB / 16;            // 16-byte chunks per weight tile row
     constexpr int kWLoads  = kWRows * kWChunks / kBlock;
     constexpr int kWRowsPerPass = kBlock / kWChunks;
@@ -78,14 +82,14 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
     const int nmb    = ceil_div(nrows, 32);
 
     // ---- global -> register staging assignments
-    const int xchunk = tid & 7;
-    const int xrow   = tid >> 3; // + 32*j
-    const unsigned char* xptr[MBLK];
-    bool xvalid[MBLK];
+    const int xchunk = tid % kXChunks;
+    const int xrow   = tid / kXChunks; // + kXRowsPerPass*j
+    const unsigned char* xptr[kXLoads];
+    bool xvalid[kXLoads];
 #pragma unroll
-    for(int j = 0; j < MBLK; j++)
+    for(int j = 0; j < kXLoads; j++)
     {
-        const int r = xrow + 32 * j;
+        const int r = xrow + kXRowsPerPass * j;
         if constexpr(GEMM0)
         {
             int tok = p.tokens;
@@ -125,19 +129,19 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
         woff[j] = (int64_t)grow * p.w_row_bytes;
     }
 
-    uint4 xv[MBLK];
+    uint4 xv[kXLoads];
     uint4 wv[kWLoads];
     uint32_t ys_next[MBLK], ys_cur[MBLK];
     const uint4 zero4 = {0u, 0u, 0u, 0u};
 
     auto load_tiles = [&](int kt) {
-        const int kx = kt * kTileKB + xchunk * 16;
+        const int kx = kt * kXKB + xchunk * 16;
 #pragma unroll
-        for(int j = 0; j < MBLK; j++)
+        for(int j = 0; j < kXLoads; j++)
         {
             xv[j] = zero4;
-            if(j < nmb && xvalid[j] && kx < p.k_bytes_x)
-                xv[j] = *reinterpret_cast<const uint4*>(xptr[j] + kt * kTileKB);
+            if(xvalid[j] && kx < p.k_bytes_x)
+                xv[j] = *reinterpret_cast<const uint4*>(xptr[j] + kt * kXKB);
         }
         const int kw = kt * kWKB + wchunk * 16;
 #pragma unroll
@@ -145,7 +149,19 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
         {
             wv[j] = zero4;
             if(kw < p.k_bytes_w)
-                wv[j] = *reinterpret_cast<const uint4*>(wbase + woff[j] + kt * kWKB);
+            {
+                // decode-sized tiles stream every weight exactly once: non-temporal loads reach a
+                // markedly higher HBM rate than cached ones
+                const uint4* src = reinterpret_cast<const uint4*>(wbase + woff[j] + kt * kWKB);
+                if constexpr(MBLK == 1)
+                {
+                    typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+                    const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
+                    wv[j]           = make_uint4(t[0], t[1], t[2], t[3]);
+                }
+                else
+                    wv[j] = *src;
+            }
         }
         if constexpr(kMx)
         {
@@ -173,15 +189,15 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
             for(int v = 0; v < 16; v++)
                 acc[j][b][v] = 0;
 
-    const int kt_count = ceil_div(p.k_bytes_x, kTileKB);
+    const int kt_count = ceil_div(p.k_bytes_x, kXKB);
     load_tiles(0);
     for(int kt = 0; kt < kt_count; kt++)
     {
         // registers -> LDS
 #pragma unroll
-        for(int j = 0; j < MBLK; j++)
-            if(j < nmb)
-                *reinterpret_cast<uint4*>(lds_x + (xrow + 32 * j) * kXStride + xchunk * 16) = xv[j];
+        for(int j = 0; j < kXLoads; j++)
+            if(((xrow + kXRowsPerPass * j) >> 5) < nmb)
+                *reinterpret_cast<uint4*>(lds_x + (xrow + kXRowsPerPass * j) * kXStride + xchunk * 16) = xv[j];
 #pragma unroll
         for(int j = 0; j < kWLoads; j++)
             *reinterpret_cast<uint4*>(lds_w + (wrow + kWRowsPerPass * j) * kWStride + wchunk * 16) = wv[j];
@@ -444,7 +460,7 @@ int launch_gemm(int mblk, const GemmParams& p, int max_tiles, hipStream_t stream
         return MI355_MOE_OK;
 #define MI355_LAUNCH(MB)                                                                               \
     {                                                                                                  \
-        const size_t lds = kWRows * (MT::kWKB + kPadB) + (MB)*32 * (kTileKB + kPadB);                  \
+        const size_t lds = kWRows * (MT::kWKB + kPadB) + (MB)*32 * (MT::kXKB + kPadB);                 \
         hipLaunchKernelGGL((moe_gemm_kernel<MODE, GEMM0, MB>), dim3(grid), dim3(kBlock), lds, stream, p); \
     }
     if(mblk == 1)
@@ -504,7 +520,23 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
     return w;
 }
 
-int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a, hipStream_t stream)
+GemmPlan make_gemm_plan(const mi355_fused_moe_traits& t, void* ws_ptr, int32_t tokens, int32_t experts, int32_t topk,
+                        int32_t hidden, int32_t inter)
+{
+    const WorkspaceLayout ws = workspace_layout(t, tokens, experts, topk, hidden, inter);
+    unsigned char* wsb       = static_cast<unsigned char*>(ws_ptr);
+    GemmPlan g{};
+    g.tile_map      = reinterpret_cast<int*>(wsb + ws.map_off);
+    g.rows_per_tile = pick_mblk(t, tokens, topk, experts, hidden, inter) * 32;
+    g.max_tiles     = ws.max_tiles;
+    g.valid         = reinterpret_cast<int*>(wsb + ws.valid_off);
+    g.n_valid       = tokens * topk;
+    g.zero_page     = reinterpret_cast<int*>(wsb + ws.zero_off);
+    return g;
+}
+
+int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a, hipStream_t stream,
+                         bool prep_done)
 {
     int rc = check_traits(t);
     if(rc != MI355_MOE_OK)
@@ -547,6 +579,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
 
     const int n_valid    = T * K;
     const int prep_grid  = 1 + std::min(ceil_div(n_valid, kPrepBlock * 4), 64);
+    if(!prep_done)
     {
     KernelTimer timer(MI355_MOE_K_PREP, stream);
     hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,

@@ -24,10 +24,7 @@ enum Mode
 
 constexpr int kBlock   = 256;
 constexpr int kWRows   = 256; // weight rows per workgroup tile
-constexpr int kTileKB  = 128; // bytes of K per row of the x tile
 constexpr int kPadB    = 16;
-constexpr int kMapHdr  = 4;   // ints in front of the tile entries
-constexpr int kMapEnt  = 8;   // ints per tile entry: expert,row0,nrows,first,ntiles,0,0,0
 
 struct GemmParams
 {
@@ -65,6 +62,7 @@ struct ModeTraits<kBf16>
     using Acc                  = f32x16_t;
     static constexpr int kOpB  = 16; // operand bytes per lane per MFMA
     static constexpr int kWKB  = 128;
+    static constexpr int kXKB  = 128;
 };
 template <>
 struct ModeTraits<kFp8>
@@ -72,6 +70,7 @@ struct ModeTraits<kFp8>
     using Acc                  = f32x16_t;
     static constexpr int kOpB  = 32;
     static constexpr int kWKB  = 128;
+    static constexpr int kXKB  = 128;
 };
 template <>
 struct ModeTraits<kI8>
@@ -79,13 +78,15 @@ struct ModeTraits<kI8>
     using Acc                  = i32x16_t;
     static constexpr int kOpB  = 16;
     static constexpr int kWKB  = 128;
+    static constexpr int kXKB  = 128;
 };
 template <>
 struct ModeTraits<kBf16W8>
 {
     using Acc                  = f32x16_t;
     static constexpr int kOpB  = 16;
-    static constexpr int kWKB  = 64; // int8 weights: 64 K elements per tile row
+    static constexpr int kWKB  = 128; // int8 weights: 128 K elements per tile row ...
+    static constexpr int kXKB  = 256; // ... against 128 bf16 activations
 };
 
 // MFMA row m of a 32-row weight block holds weight channel chan_of_row(m); with the 32x32

@@ -107,7 +107,7 @@ struct ScanShared
 __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, int Ep, int U,
                                   const int* __restrict__ mask, int T, int K,
                                   int* __restrict__ sorted_ids, float* __restrict__ sorted_w,
-                                  int* __restrict__ sorted_eid, int* __restrict__ total)
+                                  int* __restrict__ sorted_eid, int* __restrict__ total, const GemmPlan& plan)
 {
     const int tid   = threadIdx.x;
     const int e     = tid & (Ep - 1);
@@ -190,6 +190,32 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
         total[0] = total_tiles * U;
         total[1] = T;
     }
+
+    // work list of the grouped GEMMs: the padded rows of an expert split evenly into tiles
+    if(plan.tile_map != nullptr)
+    {
+        const int rows = tid < E ? s.tiles[tid] * U : 0;
+        const int nt   = ceil_div(rows, plan.rows_per_tile);
+        int n_tiles;
+        const int tb = block_exclusive_scan<kScanWaves>(nt, s.wave, n_tiles);
+        if(nt > 0)
+        {
+            const int per = round_up(ceil_div(rows, nt), 32);
+            for(int j = 0; j < nt && tb + j < plan.max_tiles; j++)
+            {
+                int* ent = plan.tile_map + kMapHdr + (tb + j) * kMapEnt;
+                ent[0]   = s.oeid[tid];
+                ent[1]   = s.tbase[tid] * U + j * per;
+                ent[2]   = min(per, rows - j * per);
+                ent[3]   = tb;
+                ent[4]   = nt;
+            }
+        }
+        if(tid == 0)
+            plan.tile_map[0] = min(n_tiles, plan.max_tiles);
+        if(tid < 64)
+            plan.zero_page[tid] = 0;
+    }
 }
 
 __device__ inline void zero_buffer(uint4* buf, int64_t nvec, int64_t first, int64_t stride)
@@ -212,6 +238,7 @@ struct SortParams
     uint4* moe_buf;
     int64_t moe_row_vec16; // 16-byte vectors per token row of moe_buf
     int* counts;           // workspace [nseg][E]
+    GemmPlan plan;         // tile_map == nullptr: nothing to prepare
     int tokens, K, E, Ep, nbits, U, nseg, work_blocks;
 };
 
@@ -240,8 +267,10 @@ __global__ __launch_bounds__(kScanBlock) void moe_sorting_oneshot_kernel(SortPar
     wave_sync();
     walk_segment<false>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, nullptr, nullptr);
     __syncthreads();
+    for(int i = threadIdx.x; i < p.plan.n_valid; i += kScanBlock)
+        p.plan.valid[i] = 0;
     scan_phase(sh, dyn_lds, kScanWaves, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
-               p.sorted_eid, p.total);
+               p.sorted_eid, p.total, p.plan);
     __syncthreads();
     walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w);
 }
@@ -258,6 +287,8 @@ __global__ __launch_bounds__(kWalkBlock) void moe_sorting_count_kernel(SortParam
                     (int64_t)(gridDim.x - p.work_blocks) * kWalkBlock);
         return;
     }
+    for(int i = blockIdx.x * kWalkBlock + threadIdx.x; i < p.plan.n_valid; i += p.work_blocks * kWalkBlock)
+        p.plan.valid[i] = 0;
     const int N    = T * p.K;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -281,7 +312,7 @@ __global__ __launch_bounds__(kScanBlock) void moe_sorting_scan_kernel(SortParams
     __shared__ ScanShared sh;
     const int T = real_tokens(p.local_tokens, p.tokens);
     scan_phase(sh, p.counts, p.nseg, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
-               p.sorted_eid, p.total);
+               p.sorted_eid, p.total, p.plan);
 }
 
 // ---- pass 3
@@ -321,7 +352,7 @@ size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk)
     return round_up<size_t>((size_t)ceil_div<int64_t>(n, kSeg) * experts * sizeof(int), 256);
 }
 
-int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream)
+int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, const GemmPlan* plan)
 {
     if((a.tokens > 0 && (!a.p_topk_ids || !a.p_weights)) || !a.p_sorted_token_ids || !a.p_sorted_weights ||
        !a.p_sorted_expert_ids || !a.p_total_tokens_post_pad)
@@ -348,6 +379,8 @@ int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream)
     p.sorted_w     = static_cast<float*>(a.p_sorted_weights);
     p.sorted_eid   = static_cast<int*>(a.p_sorted_expert_ids);
     p.total        = static_cast<int*>(a.p_total_tokens_post_pad);
+    if(plan != nullptr)
+        p.plan = *plan;
     p.tokens       = a.tokens;
     p.K            = a.topk;
     p.E            = a.num_experts;
