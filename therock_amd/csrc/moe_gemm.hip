@@ -259,35 +259,7 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
     }
 
     // ---- epilogue: lane owns token row (j*32 + r32) and 16 consecutive channels per block
-#pragma unroll
-    for(int j = 0; j < MBLK; j++)
-    {
-        if(j >= nmb)
-            continue;
-        const int r        = j * 32 + r32;
-        const bool in_tile = r < nrows;
-        const int sid      = in_tile ? p.sorted_ids[row0 + r] : p.tokens;
-        const int tok      = sid & 0xffffff;
-        if constexpr(GEMM0)
-        {
-            if(n_base + wave * 32 < p.n_out)
-                epilogue_gemm0<MODE>(p, acc[j][0], acc[j][1], expert, row0 + r, tok, in_tile,
-                                     n_base + wave * 32 + 16 * kg, kg);
-        }
-        else
-        {
-            if(!in_tile || tok >= p.tokens)
-                continue;
-            const int64_t prow = (int64_t)tok * p.topk + static_cast<int>(static_cast<uint32_t>(sid) >> 24);
-            const float tw     = p.sorted_w[row0 + r];
-            if(nt == 0 && wave == 0 && kg == 0)
-                p.valid[prow] = 1;
-#pragma unroll
-            for(int b = 0; b < 2; b++)
-                if(n_base + (wave * 2 + b) * 32 < p.n_out)
-                    epilogue_gemm1<MODE>(p, acc[j][b], expert, prow, tw, n_base + (wave * 2 + b) * 32 + 16 * kg);
-        }
-    }
+    run_epilogue<MODE, GEMM0, MBLK>(p, acc, expert, row0, nrows, 0, 32, nmb, n_base, wave, nt == 0, r32, kg);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -301,36 +301,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     }
 
     // ---- epilogue
-#pragma unroll
-    for(int i = 0; i < kMaxNB; i++)
-    {
-        const int mb = 2 * i + wt;
-        if(mb >= nmb)
-            continue;
-        const int r        = mb * 32 + r32;
-        const bool in_tile = r < nrows;
-        const int sid      = in_tile ? p.sorted_ids[row0 + r] : p.tokens;
-        const int tok      = sid & 0xffffff;
-        if constexpr(GEMM0)
-        {
-            if(n_base + ww * 32 < p.n_out)
-                epilogue_gemm0<MODE>(p, acc[i][0], acc[i][1], expert, row0 + r, tok, in_tile,
-                                     n_base + ww * 32 + 16 * kg, kg);
-        }
-        else
-        {
-            if(!in_tile || tok >= p.tokens)
-                continue;
-            const int64_t prow = (int64_t)tok * p.topk + static_cast<int>(static_cast<uint32_t>(sid) >> 24);
-            const float tw     = p.sorted_w[row0 + r];
-            if(nt == 0 && ww == 0 && kg == 0)
-                p.valid[prow] = 1;
-#pragma unroll
-            for(int b = 0; b < 2; b++)
-                if(n_base + (ww * 2 + b) * 32 < p.n_out)
-                    epilogue_gemm1<MODE>(p, acc[i][b], expert, prow, tw, n_base + (ww * 2 + b) * 32 + 16 * kg);
-        }
-    }
+    run_epilogue<MODE, GEMM0, kMaxNB>(p, acc, expert, row0, nrows, wt * 32, 64, nb_w, n_base, ww, nt == 0, r32, kg);
 }
 
 template <int MODE, bool GEMM0>

@@ -178,30 +178,46 @@ __device__ inline f32x16_t mfma_fp8_unscaled(const Frag& w, const Frag& x, f32x1
 // Epilogues.  With the weight rows on the MFMA's M side and chan_of_row(), a lane holds, for the
 // token in column (lane % 32), the 16 consecutive output channels col0 .. col0+15 in acc[0..15].
 
-// gemm0: y = silu(gate) * up with the per-token and per-channel scales folded in; stored as bf16
-// or (fp8 path) as e4m3 with one power-of-two scale per 32 columns.  Every lane of the wave must
-// call it (the fp8 path exchanges the block maximum with lane ^ 32); `store` masks the writes.
+// The operands of the epilogues (sorted ids, top-k weights, scales) are loaded by the callers in
+// one batch right after the K loop, so that their latencies overlap instead of adding up.
+
+// per-channel scales of the 16 channels a lane owns (1.0 when the path is unscaled)
+__device__ inline void load_channel_scales(const float* scale, float (&out)[16])
+{
+    if(scale != nullptr)
+    {
+        const float4* s4 = reinterpret_cast<const float4*>(scale);
+#pragma unroll
+        for(int q = 0; q < 4; q++)
+        {
+            const float4 t = s4[q];
+            out[4 * q] = t.x; out[4 * q + 1] = t.y; out[4 * q + 2] = t.z; out[4 * q + 3] = t.w;
+        }
+    }
+    else
+    {
+#pragma unroll
+        for(int v = 0; v < 16; v++)
+            out[v] = 1.0f;
+    }
+}
+
+// gemm0: y = silu(gate) * up with the per-token scale sa and the per-channel scales folded in;
+// stored as bf16 or (fp8 path) as e4m3 with one power-of-two scale per 32 columns.  Every lane of
+// the wave must call it (the fp8 path exchanges the block maximum with lane ^ 32); `store` masks
+// the writes.
 template <int MODE>
 __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc_gate,
-                                      const typename ModeTraits<MODE>::Acc& acc_up, int expert, int64_t grow,
-                                      int token, bool store, int col0, int kg)
+                                      const typename ModeTraits<MODE>::Acc& acc_up, const float (&gs)[16],
+                                      const float (&us)[16], float sa, int64_t grow, bool store, int col0, int kg)
 {
     float y[16];
-    float sa = 1.0f;
-    if(p.x_scale != nullptr)
-        sa = (store && token < p.tokens) ? p.x_scale[token] : 0.0f;
-    const float* gs = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total + col0 : nullptr;
 #pragma unroll
     for(int v = 0; v < 16; v++)
     {
-        float g = static_cast<float>(acc_gate[v]);
-        float u = static_cast<float>(acc_up[v]);
-        if(gs != nullptr)
-        {
-            g *= sa * gs[v];
-            u *= sa * gs[p.n_out + v];
-        }
-        y[v] = silu(g) * u;
+        const float g = static_cast<float>(acc_gate[v]) * (sa * gs[v]);
+        const float u = static_cast<float>(acc_up[v]) * (sa * us[v]);
+        y[v]          = silu(g) * u;
     }
     unsigned char* dst = p.out + grow * p.out_row_bytes;
     if constexpr(MODE == kFp8)
@@ -250,27 +266,86 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
 
 // gemm1: * per-channel scale * top-k weight, bf16 partial row (token * topk + slot)
 template <int MODE>
-__device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc, int expert,
-                                      int64_t prow, float topk_weight, int col0)
+__device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc,
+                                      const float (&ds)[16], int64_t prow, float topk_weight, bool store, int col0)
 {
-    const float* ds = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total + col0 : nullptr;
     float y[16];
 #pragma unroll
     for(int v = 0; v < 16; v++)
-    {
-        float o = static_cast<float>(acc[v]);
-        if(ds != nullptr)
-            o *= ds[v];
-        y[v] = o * topk_weight;
-    }
+        y[v] = static_cast<float>(acc[v]) * ds[v] * topk_weight;
     uint4 o0, o1;
     o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
     o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
     o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
     o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
-    uint4* d4 = reinterpret_cast<uint4*>(p.out + prow * p.out_row_bytes + (int64_t)col0 * 2);
-    d4[0]     = o0;
-    d4[1]     = o1;
+    if(store)
+    {
+        uint4* d4 = reinterpret_cast<uint4*>(p.out + prow * p.out_row_bytes + (int64_t)col0 * 2);
+        d4[0]     = o0;
+        d4[1]     = o1;
+    }
+}
+
+// Shared tail of both GEMM kernels.  NBLK token blocks per wave: block i covers sorted rows
+// row0 + first_row + i * row_step + r32; wblk is the wave's first 32-row weight block of the tile.
+template <int MODE, bool GEMM0, int NBLK>
+__device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2], int expert,
+                                    int row0, int nrows, int first_row, int row_step, int nblk_live, int n_base,
+                                    int wblk, bool first_n_tile, int r32, int kg)
+{
+    // ---- one batch of loads
+    int sid[NBLK];
+    float tw[NBLK];
+#pragma unroll
+    for(int i = 0; i < NBLK; i++)
+    {
+        const int r = min(first_row + i * row_step + r32, nrows - 1); // clamped: always a valid cell
+        sid[i]      = p.sorted_ids[row0 + r];
+        tw[i]       = GEMM0 ? 0.f : p.sorted_w[row0 + r];
+    }
+    float sc0[16], sc1[16];
+    const int col_a = GEMM0 ? n_base + wblk * 32 + 16 * kg : n_base + (wblk * 2) * 32 + 16 * kg;
+    const int col_b = GEMM0 ? col_a : col_a + 32;
+    const bool a_ok = (GEMM0 ? n_base + wblk * 32 : n_base + wblk * 64) < p.n_out;
+    const bool b_ok = GEMM0 ? a_ok : (n_base + wblk * 64 + 32) < p.n_out;
+    const float* sbase = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total : nullptr;
+    load_channel_scales(sbase && a_ok ? sbase + col_a : nullptr, sc0);
+    load_channel_scales(sbase && b_ok ? sbase + (GEMM0 ? p.n_out + col_a : col_b) : nullptr, sc1);
+    float sa[NBLK];
+#pragma unroll
+    for(int i = 0; i < NBLK; i++)
+    {
+        const int tok = sid[i] & 0xffffff;
+        sa[i]         = 1.0f;
+        if(GEMM0 && p.x_scale != nullptr)
+            sa[i] = tok < p.tokens ? p.x_scale[tok] : 0.0f;
+    }
+    // ---- apply
+#pragma unroll
+    for(int i = 0; i < NBLK; i++)
+    {
+        if(i >= nblk_live)
+            continue;
+        const int r        = first_row + i * row_step + r32;
+        const bool in_tile = r < nrows;
+        const int tok      = sid[i] & 0xffffff;
+        if constexpr(GEMM0)
+        {
+            if(a_ok)
+                epilogue_gemm0<MODE>(p, acc[i][0], acc[i][1], sc0, sc1, sa[i], row0 + r, in_tile, col_a, kg);
+        }
+        else
+        {
+            const bool real    = in_tile && tok < p.tokens;
+            const int64_t prow = real ? (int64_t)tok * p.topk + static_cast<int>(static_cast<uint32_t>(sid[i]) >> 24) : 0;
+            if(real && first_n_tile && wblk == 0 && kg == 0)
+                p.valid[prow] = 1;
+            if(a_ok)
+                epilogue_gemm1<MODE>(p, acc[i][0], sc0, prow, tw[i], real, col_a);
+            if(b_ok)
+                epilogue_gemm1<MODE>(p, acc[i][1], sc1, prow, tw[i], real, col_b);
+        }
+    }
 }
 
 } // namespace gemm
