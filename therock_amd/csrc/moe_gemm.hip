@@ -417,7 +417,11 @@ inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, 
         return 2;
     const int eb  = t.prec_i == MI355_MOE_BF16 ? 2 : 1;
     const int y_b = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
-    if(avg >= 160 && t.block_m % 4 == 0 && big_tile_supported(t.prec_i, hidden * eb, inter * y_b))
+    // the large-tile kernel addresses each operand as a base plus a 32-bit byte offset
+    const int64_t lim     = (int64_t)1 << 32;
+    const int64_t max_pad = topk * tokens + (int64_t)experts * t.block_m - topk;
+    const bool fits = (int64_t)2 * inter * hidden * eb < lim && max_pad * inter * y_b < lim && tokens * hidden * eb < lim;
+    if(avg >= 160 && t.block_m % 4 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b))
         return big_tile_rows() / 32;
     return 4;
 }
@@ -588,6 +592,9 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.n_out           = I;
     p.n_total         = 2 * I;
     p.n_ntiles        = ceil_div(I, 128);
+    if(mblk > 4 && (int64_t)T * p.x_row_bytes >= ((int64_t)1 << 32))
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: a token buffer of 4 GiB or more (stride_token=%d) is not "
+                                             "supported at this problem size", a.stride_token);
     if(mblk > 4)
         rc = launch_gemm_big(t.prec_i, true, p, ws.max_tiles, stream);
     else if(t.prec_i == MI355_MOE_BF16)

@@ -5,22 +5,28 @@
 //     320 sorted rows of one expert (ten 32-row blocks, interleaved between the two token halves)
 //     and 256 weight rows.  320 rather than 256 so that an expert of the DeepSeek-V3-shaped
 //     workload (about 270 rows) is one tile and its weights are fetched once.
-//   * Both operands go global -> LDS with global_load_lds_dwordx4 (no staging registers) through a
-//     ring of four 64-byte-deep K stages, three of them in flight.  The loads are issued from
-//     inline assembly so that their completion is tracked by hand: s_waitcnt vmcnt(n) with n = the
-//     DMA instructions this wave issued after the stage about to be consumed, then one workgroup
-//     barrier per stage, which also frees the buffer the next stage is written into.
-//   * An LDS row is 64 bytes (four 16-byte chunks); chunk c of row r sits at chunk position
-//     c ^ ((r >> 2) & 3), which makes both the linear DMA writes and the ds_read_b128 operand
-//     fetches conflict-free on the 64-bank LDS.  Rows that must read as zero (padding ids, rows
-//     past the tile) are fetched from a zero page, so the number of DMA instructions per wave and
-//     stage, and with it every wait count, is a compile-time constant.
+//   * Both operands go global -> LDS with global_load_lds_dwordx4 (no staging registers).  The K loop
+//     advances in 64-byte steps.  Tokens (re-read from L2 by every column tile) arrive one 64-byte
+//     step at a time through a ring of three stages.  Weights are streamed from HBM exactly once,
+//     and for them the request shape decides the rate: they arrive as full 128-byte lines, half
+//     of the tile's rows per unit (unit u = rows (u&1)*128.., K bytes [128*(u>>1), +128)), through a
+//     ring of six units issued four steps ahead.  Measured on the fp8 workload, the weight stream
+//     alone runs at 7.3 TB/s in this shape against 4.8 TB/s as 64-byte pieces.
+//   * The loads are issued from inline assembly so that their completion is tracked by hand:
+//     s_waitcnt vmcnt(n) with n = the DMA instructions this wave issued after the data about to be
+//     consumed (token step issued before weight unit in every iteration, so that waiting for the
+//     tokens does not wait for the younger weight units), then one workgroup barrier per step,
+//     which also frees the buffers the next issues write into.
+//   * LDS rows are swizzled: 64-byte token rows keep chunk c of row r at c ^ ((r >> 2) & 3), 128-byte
+//     weight rows at c ^ ((r >> 1) & 7); both the linear DMA writes and the ds_read_b128 operand
+//     fetches are then conflict-free on the 64-bank LDS.  Rows that must read as zero (padding ids,
+//     rows past the tile) are fetched from a zero page, so the number of DMA instructions per wave
+//     and step, and with it every wait count, is a compile-time constant.
 //   * The K loop is specialised on the number of token blocks a wave owns, so the MFMA region is
 //     straight-line code.
 #include "moe_gemm_device.hpp"
 
 #include <algorithm>
-#include <cstdlib>
 #include <type_traits>
 
 namespace mi355 {
@@ -28,19 +34,21 @@ using namespace gemm;
 namespace {
 
 constexpr int kBigThreads   = 512;
-constexpr int kStageKB      = 64; // bytes of K per stage and row
-constexpr int kStages       = 4;
-constexpr int kChunks       = kStageKB / 16;
-constexpr int kRowsPerDma   = 64 / kChunks; // rows one 64-lane DMA instruction fills (16)
+constexpr int kStepKB       = 64;  // bytes of K per compute step and row
 constexpr int kBigWRows     = 256;
 constexpr int kBigXRows     = 320;
 constexpr int kMaxNB        = kBigXRows / 64; // token blocks per wave (5)
-constexpr int kWRegion      = kBigWRows * kStageKB;
-constexpr int kXRegion      = kBigXRows * kStageKB;
-constexpr int kStageBytes   = kWRegion + kXRegion;
-constexpr int kYsRows       = 512;                       // padded rows per K block of the scale stage
-constexpr int kYsStageBytes = (kStageKB / 32) * kYsRows; // fp8 gemm1: e8m0 scales of 2 K blocks
-constexpr int kDmaMax       = 5;                         // DMA instructions per wave and stage (4 or 5)
+constexpr int kWHalfRows    = kBigWRows / 2;
+constexpr int kWUnitBytes   = kWHalfRows * 2 * kStepKB; // 128 rows x 128 B
+constexpr int kWSlots       = 6;
+constexpr int kXStageBytes  = kBigXRows * kStepKB;
+constexpr int kXStages      = 3;
+constexpr int kYsRows       = 512;                      // padded rows per K block of a scale stage
+constexpr int kYsStageBytes = (kStepKB / 32) * kYsRows; // fp8 gemm1: e8m0 scales of 2 K blocks
+constexpr int kXOffset      = kWSlots * kWUnitBytes;
+constexpr int kYsOffset     = kXOffset + kXStages * kXStageBytes;
+constexpr int kLdsBytes     = kYsOffset + kXStages * kYsStageBytes;
+static_assert(kLdsBytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 
 typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
 
@@ -49,14 +57,24 @@ __device__ inline uint32_t lds_offset(const void* p)
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const lds_byte_t*)p));
 }
 
-// lane i of the wave copies 16 (4) bytes from its global address to LDS byte m0 + 16*i (4*i)
-__device__ inline void dma16(const void* gptr, uint32_t m0_uniform)
+// lane i of the wave copies 16 (4) bytes from base + off (a wave-uniform base, a per-lane 32-bit offset)
+// to LDS byte m0 + 16*i (4*i)
+__device__ inline void dma16(const unsigned char* base_uniform, uint32_t off, uint32_t m0_uniform)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0_uniform), "v"(gptr) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0_uniform), "v"(off), "s"(base_uniform)
+                 : "memory");
 }
-__device__ inline void dma4(const void* gptr, uint32_t m0_uniform)
+__device__ inline void dma4(const unsigned char* base_uniform, uint32_t off, uint32_t m0_uniform)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(m0_uniform), "v"(gptr) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0_uniform), "v"(off), "s"(base_uniform)
+                 : "memory");
+}
+__device__ inline const unsigned char* uniform_ptr(const unsigned char* p)
+{
+    const uint64_t v  = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    return reinterpret_cast<const unsigned char*>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
 template <int N>
@@ -71,7 +89,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     using MT  = ModeTraits<MODE>;
     using Acc = typename MT::Acc;
     constexpr int kOpB   = MT::kOpB;
-    constexpr int kSteps = kStageKB / (2 * kOpB); // MFMAs along K per stage: 1 (fp8) or 2 (bf16, i8)
+    constexpr int kSteps = kStepKB / (2 * kOpB); // MFMAs along K per compute step: 1 (fp8) or 2 (bf16, i8)
     constexpr bool kMx   = MODE == kFp8 && !GEMM0;
     static_assert(MODE == kBf16 || MODE == kFp8 || MODE == kI8, "no large-tile kernel for this mode");
 
@@ -112,83 +130,97 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     const int nmb    = ceil_div(nrows, 32);
     const int n_base = nt * (GEMM0 ? 128 : 256);
 
-    // ---- DMA assignments.  A stage is 16 weight slabs then 20 token slabs of 1 KB (16 rows x 64 B).
-    // Wave w fills weight slabs w, w+8 and token slabs w, w+8; waves 0..3 also token slab 16+w.
-    // On the fp8 down-GEMM waves 4..7 fetch the e8m0 scales instead, so every wave issues five.
-    const int lrow16 = lane >> 2;
-    const int cchunk = (lane & 3) ^ ((lane >> 4) & 3); // logical chunk this lane fetches
-    const int n_dma  = (kMx || wave < 4) ? 5 : 4;
-    const unsigned char* gptr[kDmaMax];
-    int ginc[kDmaMax];
-#pragma unroll
-    for(int j = 0; j < kDmaMax; j++)
+    // ---- DMA assignments.
+    // Loads of one wave return in order, so a wave that mixed the two streams would see its L2-hit
+    // token loads queue behind HBM-miss weight loads.  The streams are therefore issued by different
+    // waves: waves 0..3 the weights, waves 4..7 the tokens (and, on the fp8 down-GEMM, the e8m0 scales).
+    // Weights: unit u = rows (u & 1) * 128 .. + 127 of the tile, K bytes [128 * (u >> 1), + 128).  One unit
+    // is 16 instructions of 8 rows x 128 B (full cache lines); wave w issues instructions w, w+4, w+8, w+12.
+    // Tokens: step x = all 320 rows, K bytes [64 x, + 64), 20 slabs of 16 rows x 64 B; wave 4+q fills slabs
+    // q, q+4, .. q+16 and fetches 256 scale bytes.
+    // Every source address is a wave-uniform base (operand base + K offset of the unit, kept in
+    // scalar registers) plus a per-lane 32-bit row offset doff[] that never changes: weights
+    // doff[4 * half + j]; tokens doff[0..4], scales doff[5].  Token rows that do not exist (padding
+    // ids, rows past the tile) read row 0 instead: their MFMA columns are never stored.
+    const bool w_role = wave < 4;
+    const int q4      = wave & 3;
+    uint32_t doff[8];
+    const unsigned char* dbase;
+    if(w_role)
     {
-        gptr[j] = p.zero_page;
-        ginc[j] = 0;
-        if(j < 2)
+        dbase = uniform_ptr(p.w + (int64_t)expert * p.w_expert_bytes);
+#pragma unroll
+        for(int h = 0; h < 2; h++)
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+            {
+                const int rih    = (q4 + 4 * j) * 8 + (lane >> 3); // row inside the half
+                const int trow   = h * kWHalfRows + rih;
+                const int blk    = trow >> 5;
+                const int c      = chan_of_row(trow & 31);
+                const int cchunk = (lane & 7) ^ ((rih >> 1) & 7);
+                int grow;
+                if constexpr(GEMM0)
+                    grow = (blk & 1) * p.n_out + min(n_base + (blk >> 1) * 32 + c, p.n_out - 1);
+                else
+                    grow = min(n_base + blk * 32 + c, p.n_total - 1);
+                doff[h * 4 + j] = (uint32_t)grow * (uint32_t)p.w_row_bytes + cchunk * 16;
+            }
+    }
+    else
+    {
+        dbase            = uniform_ptr(p.x);
+        const int lrow16 = lane >> 2;
+        const int cchunk = (lane & 3) ^ ((lane >> 4) & 3);
+#pragma unroll
+        for(int j = 0; j < 5; j++)
         {
-            const int lrow = (wave + 8 * j) * kRowsPerDma + lrow16;
-            const int blk  = lrow >> 5;
-            const int c    = chan_of_row(lrow & 31);
-            int grow;
-            if constexpr(GEMM0)
-                grow = (blk & 1) * p.n_out + min(n_base + (blk >> 1) * 32 + c, p.n_out - 1);
-            else
-                grow = min(n_base + blk * 32 + c, p.n_total - 1);
-            gptr[j] = p.w + (int64_t)expert * p.w_expert_bytes + (int64_t)grow * p.w_row_bytes + cchunk * 16;
-            ginc[j] = kStageKB;
-        }
-        else if(j < 4 || wave < 4)
-        {
-            const int xslab = j < 4 ? wave + 8 * (j - 2) : 16 + wave;
-            const int lrow  = xslab * kRowsPerDma + lrow16;
-            bool ok         = lrow < nrows;
-            int64_t src     = row0 + lrow;
+            const int lrow = (q4 + 4 * j) * 16 + lrow16;
+            uint32_t src   = lrow < nrows ? row0 + lrow : row0;
             if constexpr(GEMM0)
             {
                 int tok = p.tokens;
-                if(ok)
+                if(lrow < nrows)
                     tok = p.sorted_ids[row0 + lrow] & 0xffffff;
-                ok  = tok < p.tokens;
-                src = tok;
+                src = tok < p.tokens ? tok : 0;
             }
-            gptr[j] = ok ? p.x + src * p.x_row_bytes + cchunk * 16 : p.zero_page + cchunk * 16;
-            ginc[j] = ok ? kStageKB : 0;
+            doff[j] = src * (uint32_t)p.x_row_bytes + cchunk * 16;
         }
-        else if constexpr(kMx)
-        {
-            // wave 4+q: K block (q >> 1) of the stage, rows (q & 1) * 256 .. + 255
-            const int q = wave - 4;
-            gptr[j]     = p.y_scale + (int64_t)(q >> 1) * p.ys_kb_stride + row0 + (q & 1) * 256 + lane * 4;
-        }
+        // scales: K block (q >> 1) of the step, rows (q & 1) * 256 .. + 255 (the rows are padded)
+        doff[5] = (uint32_t)((q4 >> 1) * p.ys_kb_stride + row0 + (q4 & 1) * 256 + lane * 4);
+        doff[6] = doff[7] = 0;
     }
-    const int64_t ys_step = (kStageKB / 32) * p.ys_kb_stride;
+    const int64_t ys_step = (kStepKB / 32) * p.ys_kb_stride;
 
     const uint32_t lds_base = lds_offset(lds);
-    const uint32_t ys_base  = lds_base + kStages * kStageBytes;
+    const int kt_count      = p.k_bytes_x / kStepKB; // compute steps = weight units (even)
 
-    auto issue = [&](int k) {
-        const uint32_t sbase = lds_base + (k & (kStages - 1)) * kStageBytes;
+    // weight role: unit u (half u & 1) -> ring slot u % 6
+    auto issue_w = [&](int u, auto half_tag) __attribute__((always_inline)) {
+        constexpr int H = decltype(half_tag)::value;
+        if(u >= kt_count)
+            return;
+        const uint32_t sbase     = lds_base + (u % kWSlots) * kWUnitBytes + q4 * 1024;
+        const unsigned char* src = dbase + (u >> 1) * (2 * kStepKB);
 #pragma unroll
         for(int j = 0; j < 4; j++)
-        {
-            const int slab_off = (j < 2 ? 0 : kWRegion) + (wave + 8 * (j & 1)) * 1024;
-            dma16(gptr[j], __builtin_amdgcn_readfirstlane(sbase + slab_off));
-            gptr[j] += ginc[j];
-        }
-        if(wave < 4)
-        {
-            dma16(gptr[4], __builtin_amdgcn_readfirstlane(sbase + kWRegion + (16 + wave) * 1024));
-            gptr[4] += ginc[4];
-        }
-        else if constexpr(kMx)
-        {
-            const int q = wave - 4;
-            dma4(gptr[4], __builtin_amdgcn_readfirstlane(ys_base + (k & (kStages - 1)) * kYsStageBytes +
-                                                        (q >> 1) * kYsRows + (q & 1) * 256));
-            gptr[4] += ys_step;
-        }
+            dma16(src, doff[H * 4 + j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));
     };
+    // token role: step x -> ring stage x % 3
+    auto issue_x = [&](int x) __attribute__((always_inline)) {
+        if(x >= kt_count)
+            return;
+        const uint32_t sbase     = lds_base + kXOffset + (x % kXStages) * kXStageBytes + q4 * 1024;
+        const unsigned char* src = dbase + x * kStepKB;
+#pragma unroll
+        for(int j = 0; j < 5; j++)
+            dma16(src, doff[j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));
+        if constexpr(kMx)
+            dma4(p.y_scale + x * ys_step, doff[5],
+                 __builtin_amdgcn_readfirstlane(lds_base + kYsOffset + (x % kXStages) * kYsStageBytes +
+                                                (q4 >> 1) * kYsRows + (q4 & 1) * 256));
+    };
+    constexpr int kXInstr = kMx ? 6 : 5; // token-role DMA instructions per step
 
     Acc acc[kMaxNB][2];
 #pragma unroll
@@ -199,75 +231,87 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             for(int v = 0; v < 16; v++)
                 acc[i][b][v] = 0;
 
-    const int kt_count = p.k_bytes_x / kStageKB;
-    for(int k = 0; k < kStages - 1 && k < kt_count; k++)
-        issue(k);
+    // prologue: weight units 0..3, token steps 0 and 1
+    using H0 = std::integral_constant<int, 0>;
+    using H1 = std::integral_constant<int, 1>;
+    if(w_role)
+    {
+        issue_w(0, H0{});
+        issue_w(1, H1{});
+        issue_w(2, H0{});
+        issue_w(3, H1{});
+    }
+    else
+    {
+        issue_x(0);
+        issue_x(1);
+    }
 
-    // per-lane LDS read offsets inside a stage (swizzled chunk positions are per-lane constants)
-    const int sw    = (r32 >> 2) & 3;
-    const int w_off = (ww * 64 + r32) * kStageKB;
-    const int x_off = kWRegion + (wt * 32 + r32) * kStageKB;
+    // per-lane LDS read offsets (swizzled chunk positions are per-lane constants)
+    const int sw_w  = (r32 >> 1) & 7; // 128-byte weight rows
+    const int sw_x  = (r32 >> 2) & 3; // 64-byte token rows
+    const int w_off = ((ww & 1) * 64 + r32) * (2 * kStepKB);
+    const int w_h   = ww >> 1;
+    const int x_off = kXOffset + (wt * 32 + r32) * kStepKB;
 
     auto k_loop = [&](auto nb_tag) {
         constexpr int NB = decltype(nb_tag)::value;
         constexpr int NF = NB > 0 ? NB : 1;
-        for(int k = 0; k < kt_count; k++)
-        {
-            // stage k has landed once at most the DMA instructions of the later stages are pending
-            const int later = min(kt_count - 1 - k, kStages - 2);
-            if(later >= 2)
+        // one compute step; PAR = k & 1
+        auto step = [&](int k, auto par_tag) __attribute__((always_inline)) {
+            constexpr int PAR = decltype(par_tag)::value;
+            // Needed now: token step k and the weight units of pair k >> 1.  Issued after them and allowed
+            // to stay pending: token step k+1; weight units k+2, k+3 (even k) or k+1 .. k+3 (odd k).
+            if(k + 3 < kt_count)
             {
-                if(n_dma == 5)
-                    wait_vmcnt<10>();
+                if(w_role)
+                    wait_vmcnt<PAR ? 12 : 8>();
                 else
-                    wait_vmcnt<8>();
-            }
-            else if(later == 1)
-            {
-                if(n_dma == 5)
-                    wait_vmcnt<5>();
-                else
-                    wait_vmcnt<4>();
+                    wait_vmcnt<kXInstr>();
             }
             else
                 wait_vmcnt<0>();
-            // stage k visible to all waves; everyone is done reading stage k-1 (a bare barrier: the
-            // DMA completion was awaited above and LDS reads are consumed by MFMAs before a wave
-            // gets here)
+            // data of step k visible to all waves; everyone is done reading step k-1 (a bare barrier:
+            // the DMA completion was awaited above and LDS reads are consumed by MFMAs before a
+            // wave gets here)
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if(k + kStages - 1 < kt_count && !(p.debug & 1))
-                issue(k + kStages - 1);
-            if(p.debug & 2)
-                continue;
+            if(w_role)
+                issue_w(k + 4, par_tag);
+            else
+                issue_x(k + 2);
 
-            const unsigned char* st = lds + (k & (kStages - 1)) * kStageBytes;
+            const unsigned char* wst = lds + (((k & ~1) + w_h) % kWSlots) * kWUnitBytes + w_off;
+            const unsigned char* xst = lds + x_off + (k % kXStages) * kXStageBytes;
             [[maybe_unused]] const unsigned char* ysl =
-                lds + kStages * kStageBytes + (k & (kStages - 1)) * kYsStageBytes + kg * kYsRows + wt * 32 + r32;
+                lds + kYsOffset + (k % kXStages) * kYsStageBytes + kg * kYsRows + wt * 32 + r32;
+            constexpr int kh = PAR * 4; // first chunk of this step inside the 128-byte weight row
 #pragma unroll
             for(int s = 0; s < kSteps; s++)
             {
                 Frag wf[2];
                 Frag xf[NF];
                 uint32_t xs[NF];
-                const int c_lo = kOpB == 16 ? ((2 * s + kg) ^ sw) * 16 : (kg ^ sw) * 16;
-                const int c_hi = ((2 + kg) ^ sw) * 16;
+                const int cx_lo = kOpB == 16 ? ((2 * s + kg) ^ sw_x) * 16 : (kg ^ sw_x) * 16;
+                const int cx_hi = ((2 + kg) ^ sw_x) * 16;
+                const int cw_lo = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_w) * 16 : ((kh + kg) ^ sw_w) * 16;
+                const int cw_hi = ((kh + 2 + kg) ^ sw_w) * 16;
 #pragma unroll
                 for(int b = 0; b < 2; b++)
                 {
-                    const unsigned char* wp = st + w_off + b * 32 * kStageKB;
-                    wf[b].lo                = *reinterpret_cast<const uint4*>(wp + c_lo);
+                    const unsigned char* wp = wst + b * 32 * (2 * kStepKB);
+                    wf[b].lo                = *reinterpret_cast<const uint4*>(wp + cw_lo);
                     if constexpr(kOpB == 32)
-                        wf[b].hi = *reinterpret_cast<const uint4*>(wp + c_hi);
+                        wf[b].hi = *reinterpret_cast<const uint4*>(wp + cw_hi);
                 }
 #pragma unroll
                 for(int i = 0; i < NB; i++)
                 {
-                    const unsigned char* xp = st + x_off + i * 64 * kStageKB;
-                    xf[i].lo                = *reinterpret_cast<const uint4*>(xp + c_lo);
+                    const unsigned char* xp = xst + i * 64 * kStepKB;
+                    xf[i].lo                = *reinterpret_cast<const uint4*>(xp + cx_lo);
                     if constexpr(kOpB == 32)
-                        xf[i].hi = *reinterpret_cast<const uint4*>(xp + c_hi);
+                        xf[i].hi = *reinterpret_cast<const uint4*>(xp + cx_hi);
                     xs[i] = 127;
                     if constexpr(kMx)
                         xs[i] = ysl[i * 64];
@@ -287,6 +331,11 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                     }
                 }
             }
+        };
+        for(int k = 0; k < kt_count; k += 2)
+        {
+            step(k, H0{});
+            step(k + 1, H1{});
         }
     };
     const int nb_w = max(0, min(kMaxNB, (nmb - wt + 1) / 2));
@@ -308,7 +357,7 @@ template <int MODE, bool GEMM0>
 int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
 {
     constexpr bool kMx  = MODE == kFp8 && !GEMM0;
-    const size_t lds    = kStages * kStageBytes + (kMx ? kStages * kYsStageBytes : 0);
+    const size_t lds    = kMx ? kLdsBytes : kYsOffset;
     static bool attr_ok = false; // the limit is a per-function attribute; setting it again is harmless
     if(!attr_ok)
     {
@@ -319,11 +368,8 @@ int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
     const int grid = round_up(max_tiles * p.n_ntiles, 8);
     if(grid <= 0)
         return MI355_MOE_OK;
-    GemmParams q = p;
-    if(const char* dbg = getenv("MI355_MOE_DEBUG"))
-        q.debug = atoi(dbg);
     KernelTimer timer(GEMM0 ? MI355_MOE_K_GEMM0 : MI355_MOE_K_GEMM1, stream);
-    hipLaunchKernelGGL((moe_gemm_big_kernel<MODE, GEMM0>), dim3(grid), dim3(kBigThreads), lds, stream, q);
+    hipLaunchKernelGGL((moe_gemm_big_kernel<MODE, GEMM0>), dim3(grid), dim3(kBigThreads), lds, stream, p);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }
@@ -334,7 +380,7 @@ int big_tile_rows() { return kBigXRows; }
 
 bool big_tile_supported(int prec, int k_bytes0, int k_bytes1)
 {
-    return (prec == MI355_MOE_BF16 || prec == MI355_MOE_FP8) && k_bytes0 % kStageKB == 0 && k_bytes1 % kStageKB == 0;
+    return (prec == MI355_MOE_BF16 || prec == MI355_MOE_FP8) && k_bytes0 % (2 * kStepKB) == 0 && k_bytes1 % (2 * kStepKB) == 0;
 }
 
 int launch_gemm_big(int prec, bool gemm0, const GemmParams& p, int max_tiles, hipStream_t stream)

@@ -51,7 +51,6 @@ struct GemmParams
     int n_ntiles;            // tiles along n
     int tokens;
     int topk;
-    int debug; // experiments only: bit0 = no DMA after the first stage, bit1 = no MFMA work
 };
 
 template <int MODE>
