@@ -2,12 +2,17 @@
 """Benchmark of the fused-MoE path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--headline-only] [--no-cpu-baseline]
+                    [--calibrate-copy]
 
 One "step" is one pass of the whole path (moe_sorting + gate/up GEMM with SiLU*up + down GEMM +
 top-k combine) over one batch of synthetic, already-quantised inputs resident in HBM.  The headline
 workload is the DeepSeek-V3-shaped fp8 layer at 8192 tokens (the configuration the target of the
 metric is quoted on); the other benchmark configurations are reported under "workloads" in the
 same JSON line.  Prints exactly one JSON line on stdout.
+
+--calibrate-copy appends one plain device copy of 1 GiB (torch's copy kernel) after the timed
+region: under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` its reading gives the factor that
+turns the counter into bytes for the GEMM kernels of the same run.
 """
 from __future__ import annotations
 
@@ -67,7 +72,8 @@ def run_workload(cfg, steps, warmup, seed=0):
     gemm_ms = kavg.get("moe_gemm0_gate_up_silu", 0) + kavg.get("moe_gemm1_down", 0) + kavg.get("moe_combine", 0) + kavg.get("moe_prep", 0)
     res = {
         "workload": cfg.name, "dtype": cfg.dtype, "tokens": T, "hidden": H, "inter": I, "experts": cfg.experts,
-        "topk": K, "block_m": cfg.unit, "ms_per_step": ms, "tflops": cfg.flops / ms / 1e9,
+        "topk": K, "block_m": cfg.unit, "tile_rows": ta.fused_moe_tile_rows(traits, T, cfg.experts, K, H, I),
+        "ms_per_step": ms, "tflops": cfg.flops / ms / 1e9,
         "tokens_per_s": T / ms * 1e3, "algorithmic_GB": byt / 1e9, "hbm_GBps": byt / ms / 1e6,
         "frac_mfma_peak": cfg.flops / ms / 1e9 / PEAK_MFMA[cfg.dtype], "frac_hbm_peak": byt / ms / 1e6 / PEAK_HBM,
         "gemm_only_ms": gemm_ms, "post_pad": post_pad, "active_experts": active,
@@ -78,23 +84,37 @@ def run_workload(cfg, steps, warmup, seed=0):
     return res, inp, buf
 
 
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "moe_gemm0_hbm_traffic.txt")
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the gate+up GEMM as measured with rocprofv3 counters (a committed
+    summary: lines of `workload fetch_bytes write_bytes`); None when there is no entry."""
+    try:
+        for ln in open(TRAFFIC_FILE):
+            f = ln.split()
+            if len(f) >= 3 and f[0] == workload:
+                return float(f[1]) + float(f[2])
+    except OSError:
+        pass
+    return None
+
+
 def roofline_of(cfg, res):
     """Roofline entry for the dominant kernel of a workload."""
     k0, k1 = res["kernel_avg_ms"].get("moe_gemm0_gate_up_silu"), res["kernel_avg_ms"].get("moe_gemm1_down")
     T, K, H, I = cfg.tokens, cfg.topk, cfg.hidden, cfg.inter
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(cfg.name, {}).get("gemm0_hbm_bytes_per_launch")
+    traffic = measured_traffic(cfg.name)
+    kname = ("moe_gemm_big_kernel" if res["tile_rows"] > 128 else "moe_gemm_kernel") + " (gemm0: gate+up, SiLU*up)"
     if cfg.flops / (res["algorithmic_GB"] * 1e9) > PEAK_MFMA[cfg.dtype] * 1e12 / (PEAK_HBM * 1e9):
         ach = 4.0 * T * K * H * I / k0 / 1e9  # gate+up GEMM: 2/3 of the FLOPs
-        return {"kernel": "moe_gemm_kernel (gemm0: gate+up, SiLU*up)", "bound": "mfma", "achieved": ach,
+        return {"kernel": kname, "bound": "mfma", "achieved": ach,
                 "peak": PEAK_MFMA[cfg.dtype], "unit": "TFLOP/s", "frac": ach / PEAK_MFMA[cfg.dtype],
                 "avg_launch_ms": k0, "traffic": traffic}
     b = {"bf16": 2, "fp8": 1, "int8": 1}[cfg.dtype]
     byt0 = res["active_experts"] * 2 * I * H * b + res["active_experts"] * 2 * I * 4 + T * H * b + res["post_pad"] * I * 2
     ach = byt0 / k0 / 1e6
-    return {"kernel": "moe_gemm_kernel (gemm0: gate+up, SiLU*up)", "bound": "hbm", "achieved": ach, "peak": PEAK_HBM,
+    return {"kernel": kname, "bound": "hbm", "achieved": ach, "peak": PEAK_HBM,
             "unit": "GB/s", "frac": ach / PEAK_HBM, "avg_launch_ms": k0, "traffic": traffic}
 
 
@@ -153,6 +173,7 @@ def main():
     ap.add_argument("--workload", default=HEADLINE)
     ap.add_argument("--headline-only", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures one GPU only; run with --gpus 1 (the path is single-GPU, "
@@ -168,6 +189,14 @@ def main():
     res, inp, buf = run_workload(cfg, a.steps, a.warmup)
     log(f"[bench] {cfg.name}: {res['ms_per_step']:.3f} ms/step, {res['tflops']:.1f} TFLOP/s, kernels {res['kernel_avg_ms']}")
     roof = roofline_of(cfg, res)
+    if a.calibrate_copy:
+        src = torch.arange(1 << 28, dtype=torch.int32, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        log(f"[bench] calibration copy: {src.numel() * 4} bytes read, {dst.numel() * 4} bytes written")
+        del src, dst
     cpu = None
     if not a.no_cpu_baseline:
         try:

@@ -164,6 +164,12 @@ size_t mi355_fused_moe_workspace_size(const mi355_fused_moe_traits* traits, int3
                                       int32_t num_experts, int32_t topk, int32_t hidden_size,
                                       int32_t intermediate_size);
 
+/* sorted rows one GEMM workgroup owns at this problem size: 32, 64 or 128 (moe_gemm_kernel) or 320
+ * (moe_gemm_big_kernel); 0 for unsupported traits.  The counterpart of Block_M0 of the instance
+ * ck_tile's dispatcher selects (fused_moegemm_shape.hpp:43-64); here it is chosen per problem size. */
+int32_t mi355_fused_moe_tile_rows(const mi355_fused_moe_traits* traits, int32_t tokens, int32_t num_experts,
+                                  int32_t topk, int32_t hidden_size, int32_t intermediate_size);
+
 /* replaces fused_moegemm(traits, args, stream): FusedMoeGemmKernel (fused_moegemm_kernel.hpp:238-259).
  * Gate+up GEMM with SiLU*up, down GEMM, top-k weighted combine into o. */
 int mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_moegemm_args* args,

@@ -171,6 +171,15 @@ mi355_fused_moe_workspace_size(const mi355_fused_moe_traits* traits, int32_t tok
     return workspace_layout(*traits, tokens, num_experts, topk, hidden_size, intermediate_size).total;
 }
 
+__attribute__((visibility("default"))) int32_t
+mi355_fused_moe_tile_rows(const mi355_fused_moe_traits* traits, int32_t tokens, int32_t num_experts, int32_t topk,
+                          int32_t hidden_size, int32_t intermediate_size)
+{
+    if(traits == nullptr || check_traits(*traits) != MI355_MOE_OK || num_experts <= 0)
+        return 0;
+    return gemm_tile_rows(*traits, tokens, num_experts, topk, hidden_size, intermediate_size);
+}
+
 __attribute__((visibility("default"))) int
 mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_moegemm_args* args, void* stream)
 {

@@ -472,6 +472,12 @@ int check_traits(const mi355_fused_moe_traits& t)
     return MI355_MOE_OK;
 }
 
+int gemm_tile_rows(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk, int32_t hidden,
+                   int32_t inter)
+{
+    return pick_mblk(t, tokens, topk, experts, hidden, inter) * 32;
+}
+
 WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk,
                                  int32_t hidden, int32_t inter)
 {

@@ -26,6 +26,10 @@ int check_traits(const mi355_fused_moe_traits& t);
 WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts,
                                  int32_t topk, int32_t hidden, int32_t inter);
 
+// sorted rows per GEMM workgroup at this problem size
+int gemm_tile_rows(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk, int32_t hidden,
+                   int32_t inter);
+
 // prep_done: the tile list, valid flags and zero page were already written by the sort (GemmPlan)
 int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a,
                          hipStream_t stream, bool prep_done = false);

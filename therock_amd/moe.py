@@ -204,6 +204,13 @@ def rowwise_quant(x, q_dtype: str, stream=None):
 
 
 # ------------------------------------------------------------------ convenience for harnesses
+def fused_moe_tile_rows(traits: fused_moe_traits, tokens, num_experts, topk, hidden_size, intermediate_size) -> int:
+    """Sorted rows one GEMM workgroup owns at this problem size (320 selects the large-tile kernel)."""
+    t = traits.pod()
+    return int(_lib.load().mi355_fused_moe_tile_rows(C.byref(t), tokens, num_experts, topk, hidden_size,
+                                                     intermediate_size))
+
+
 class MoeBuffers:
     """Caller-side allocation of everything fused_moe needs (what CK's example main does with
     DeviceMem): sort outputs, workspace and the output tensor."""
