@@ -147,6 +147,8 @@ def moe_sorting(topk_ids, weights, experts, unit, local_expert_mask=None, skip_e
     weights = _c(weights, np.float32)
     T, K = topk_ids.shape
     mp = max_num_tokens_padded(T, K, experts, unit)
+    if not skip_empty:  # every expert owns a tile: with fewer than K distinct experts in use the bound above is short
+        mp = max(mp, experts * unit)
     ids = np.full((mp,), fill_id, dtype=np.int32)
     w = np.full((mp,), fill_w, dtype=np.float32)
     eid = np.full(((mp + unit - 1) // unit,), fill_eid, dtype=np.int32)
@@ -169,6 +171,8 @@ def ck_moe_sorting(topk_ids, weights, experts, unit, local_expert_mask=None, ski
     weights = _c(weights, np.float32)
     T, K = topk_ids.shape
     mp = max_num_tokens_padded(T, K, experts, unit)
+    if not skip_empty:  # every expert owns a tile: with fewer than K distinct experts in use the bound above is short
+        mp = max(mp, experts * unit)
     ids = np.full((mp,), fill_id, dtype=np.int32)
     w = np.full((mp,), fill_w, dtype=np.float32)
     eid = np.full(((mp + unit - 1) // unit,), fill_eid, dtype=np.int32)

@@ -84,8 +84,7 @@ struct GemmPlan
     int* tile_map;     // work list, see above
     int rows_per_tile; // sorted rows per GEMM tile (multiple of 32)
     int max_tiles;     // capacity of tile_map
-    int* valid;        // [n_valid] flags to clear
-    int n_valid;
+    int* inv;          // [tokens * topk]: sorted position of every (token, slot), -1 when dropped
     int* zero_page;    // 64 ints to clear
 };
 

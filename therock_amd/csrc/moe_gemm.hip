@@ -8,8 +8,8 @@
 // Instead of ck_tile's single kernel (32 sorted rows x 512 intermediate columns per workgroup,
 // bf16 atomics into the output) the path is three launches over a tile list built from the sort:
 //   gemm0  Y[row, n]   = silu(x . Wgate[n]) * (x . Wup[n])      (gather rows by sorted token id)
-//   gemm1  P[t*K+k, h] = (Y[row] . Wdown[h]) * topk_weight      (bf16 partial per (token, slot))
-//   combine O[t, h]    = sum_k P[t*K+k, h]  in slot order, fp32, one rounding to bf16
+//   gemm1  P[row, h]   = Y[row] . Wdown[h]                      (bf16 partial per sorted row)
+//   combine O[t, h]    = sum_k w[t,k] * P[pos(t,k), h]  in slot order, fp32, one rounding to bf16
 // A workgroup (4 waves) owns up to MBLK*32 sorted rows of ONE expert and 256 weight rows
 // (gemm0: 128 gate + 128 up rows = 128 Y columns).  The MFMA's M side is the weight rows and its
 // N side the tokens, so every lane ends up with 16 consecutive output channels of one token and
@@ -259,12 +259,13 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
     }
 
     // ---- epilogue: lane owns token row (j*32 + r32) and 16 consecutive channels per block
-    run_epilogue<MODE, GEMM0, MBLK>(p, acc, expert, row0, nrows, 0, 32, nmb, n_base, wave, nt == 0, r32, kg);
+    run_epilogue<MODE, GEMM0, MBLK, true>(p, acc, expert, row0, nrows, 0, 32, nmb, n_base, wave, r32, kg);
 }
 
 // ---------------------------------------------------------------------------------------------
 // Tile list: one entry per (expert, group of <= rows_per_tile sorted rows), rows split evenly.
-// Block 0 builds the list from sorted_expert_ids; every block helps clear the valid flags.
+// Block 0 builds the list from sorted_expert_ids; every block helps reset the inverse map, which
+// moe_inv_kernel then fills from the sorted ids (the sort does both itself in the fused entry point).
 constexpr int kPrepBlock = 1024;
 constexpr int kPrepWaves = kPrepBlock / kWave;
 
@@ -286,11 +287,11 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
                                                                const int* __restrict__ post_pad_ptr, int unit,
                                                                int experts, int rows_per_tile, int max_units,
                                                                int max_tiles, int* __restrict__ tile_map,
-                                                               int* __restrict__ valid, int n_valid,
+                                                               int* __restrict__ inv, int n_inv,
                                                                int* __restrict__ zero_page)
 {
-    for(int i = blockIdx.x * kPrepBlock + threadIdx.x; i < n_valid; i += gridDim.x * kPrepBlock)
-        valid[i] = 0;
+    for(int i = blockIdx.x * kPrepBlock + threadIdx.x; i < n_inv; i += gridDim.x * kPrepBlock)
+        inv[i] = -1;
     if(blockIdx.x != 0)
         return;
     if(threadIdx.x < 64)
@@ -334,9 +335,26 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
         tile_map[0] = min(total, max_tiles);
 }
 
-// O[t, h] = sum over slots (in slot order) of the bf16 partials, fp32 accumulate, one rounding
+// inv[token * topk + slot] = sorted position, for every real entry of the sorted id list
+__global__ __launch_bounds__(256) void moe_inv_kernel(const int* __restrict__ sorted_ids,
+                                                       const int* __restrict__ post_pad_ptr, int max_pad, int tokens,
+                                                       int topk, int* __restrict__ inv)
+{
+    const int post_pad = min(post_pad_ptr[0], max_pad);
+    for(int pos = blockIdx.x * 256 + threadIdx.x; pos < post_pad; pos += gridDim.x * 256)
+    {
+        const int id   = sorted_ids[pos];
+        const int tok  = id & 0xffffff;
+        const int slot = static_cast<int>(static_cast<uint32_t>(id) >> 24);
+        if(tok < tokens && slot < topk)
+            inv[tok * topk + slot] = pos;
+    }
+}
+
+// O[t, h] = sum over slots (in slot order) of top-k weight * bf16 partial, fp32 accumulate, one rounding
 __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* __restrict__ part,
-                                                           const int* __restrict__ valid,
+                                                           const int* __restrict__ inv,
+                                                           const float* __restrict__ sorted_w,
                                                            unsigned char* __restrict__ out, int topk, int hidden,
                                                            int64_t out_row_bytes)
 {
@@ -347,16 +365,17 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     for(int k = 0; k < topk; k++)
     {
-        const int64_t prow = (int64_t)t * topk + k;
-        if(valid[prow] == 0)
+        const int pos = inv[t * topk + k];
+        if(pos < 0)
             continue;
-        const uint4 v = *reinterpret_cast<const uint4*>(part + (prow * hidden + h0) * 2);
+        const float w = sorted_w[pos];
+        const uint4 v = *reinterpret_cast<const uint4*>(part + ((int64_t)pos * hidden + h0) * 2);
         const uint32_t d[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for(int i = 0; i < 4; i++)
         {
-            acc[2 * i] += __uint_as_float(d[i] << 16);
-            acc[2 * i + 1] += __uint_as_float(d[i] & 0xffff0000u);
+            acc[2 * i] += w * __uint_as_float(d[i] << 16);
+            acc[2 * i + 1] += w * __uint_as_float(d[i] & 0xffff0000u);
         }
     }
     uint4 o;
@@ -493,12 +512,12 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
     const int y_b    = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
     w.sort_off       = bump(sorting_workspace_bytes(tokens, experts, topk));
     w.map_off        = bump(sizeof(int) * (kMapHdr + (size_t)kMapEnt * w.max_tiles));
-    w.valid_off      = bump(sizeof(int) * (size_t)tokens * topk);
+    w.inv_off        = bump(sizeof(int) * (size_t)tokens * topk);
     w.y_off          = bump((size_t)w.max_pad * inter * y_b);
     w.ys_kb_stride   = round_up<int64_t>(w.max_pad, 256) + 512;
     w.ys_off         = bump(t.prec_i == MI355_MOE_FP8 ? (size_t)w.ys_kb_stride * (inter / 32) : 0);
     w.zero_off       = bump(256);
-    w.p_off          = bump((size_t)tokens * topk * hidden * 2);
+    w.p_off          = bump((size_t)w.max_pad * hidden * 2);
     return w;
 }
 
@@ -511,8 +530,7 @@ GemmPlan make_gemm_plan(const mi355_fused_moe_traits& t, void* ws_ptr, int32_t t
     g.tile_map      = reinterpret_cast<int*>(wsb + ws.map_off);
     g.rows_per_tile = pick_mblk(t, tokens, topk, experts, hidden, inter) * 32;
     g.max_tiles     = ws.max_tiles;
-    g.valid         = reinterpret_cast<int*>(wsb + ws.valid_off);
-    g.n_valid       = tokens * topk;
+    g.inv           = reinterpret_cast<int*>(wsb + ws.inv_off);
     g.zero_page     = reinterpret_cast<int*>(wsb + ws.zero_off);
     return g;
 }
@@ -555,29 +573,29 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
         return fail(MI355_MOE_E_INVALID, "fused_moegemm: workspace must be 256-byte aligned");
     unsigned char* wsb = static_cast<unsigned char*>(a.ws_ptr);
     int* tile_map      = reinterpret_cast<int*>(wsb + ws.map_off);
-    int* valid         = reinterpret_cast<int*>(wsb + ws.valid_off);
+    int* inv           = reinterpret_cast<int*>(wsb + ws.inv_off);
     const int mblk     = pick_mblk(t, T, K, E, H, I);
     const int max_units = (int)ceil_div<int64_t>(ws.max_pad, t.block_m);
 
-    const int n_valid    = T * K;
-    const int prep_grid  = 1 + std::min(ceil_div(n_valid, kPrepBlock * 4), 64);
+    const int n_inv      = T * K;
+    const int prep_grid  = 1 + std::min(ceil_div(n_inv, kPrepBlock * 4), 64);
     if(!prep_done)
     {
-    KernelTimer timer(MI355_MOE_K_PREP, stream);
-    hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
-                       static_cast<const int*>(a.sorted_expert_ids_ptr), static_cast<const int*>(a.num_sorted_tiles_ptr),
-                       t.block_m, E, mblk * 32, max_units, ws.max_tiles, tile_map, valid, n_valid,
-                       reinterpret_cast<int*>(wsb + ws.zero_off));
+        KernelTimer timer(MI355_MOE_K_PREP, stream);
+        hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
+                           static_cast<const int*>(a.sorted_expert_ids_ptr),
+                           static_cast<const int*>(a.num_sorted_tiles_ptr), t.block_m, E, mblk * 32, max_units,
+                           ws.max_tiles, tile_map, inv, n_inv, reinterpret_cast<int*>(wsb + ws.zero_off));
+        hipLaunchKernelGGL(moe_inv_kernel, dim3(std::min<int>(ceil_div<int64_t>(ws.max_pad, 256), 1024)), dim3(256), 0,
+                           stream, static_cast<const int*>(a.sorted_token_ids_ptr),
+                           static_cast<const int*>(a.num_sorted_tiles_ptr), (int)ws.max_pad, T, K, inv);
     }
     MI355_HIP_TRY(hipGetLastError());
 
     GemmParams p{};
     p.sorted_ids = static_cast<const int*>(a.sorted_token_ids_ptr);
-    p.sorted_w   = static_cast<const float*>(a.sorted_weight_ptr);
     p.tile_map   = tile_map;
-    p.valid      = valid;
     p.tokens     = T;
-    p.topk       = K;
     p.y_scale    = wsb + ws.ys_off;
     p.ys_kb_stride = ws.ys_kb_stride;
     p.zero_page    = wsb + ws.zero_off;
@@ -641,8 +659,9 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     // ---- combine
     {
     KernelTimer timer(MI355_MOE_K_COMBINE, stream);
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, valid,
-                       static_cast<unsigned char*>(a.o_ptr), K, H, (int64_t)a.stride_token * 2);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, inv,
+                       static_cast<const float*>(a.sorted_weight_ptr), static_cast<unsigned char*>(a.o_ptr), K, H,
+                       (int64_t)a.stride_token * 2);
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;

@@ -350,7 +350,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     }
 
     // ---- epilogue
-    run_epilogue<MODE, GEMM0, kMaxNB>(p, acc, expert, row0, nrows, wt * 32, 64, nb_w, n_base, ww, nt == 0, r32, kg);
+    run_epilogue<MODE, GEMM0, kMaxNB, false>(p, acc, expert, row0, nrows, wt * 32, 64, nb_w, n_base, ww, r32, kg);
 }
 
 template <int MODE, bool GEMM0>

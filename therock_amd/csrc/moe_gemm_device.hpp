@@ -33,11 +33,9 @@ struct GemmParams
     const float* x_scale;    // gemm0: per-token scale or null
     const float* w_scale;    // [experts, n_total] or null
     const int* sorted_ids;
-    const float* sorted_w;
     const int* tile_map;
-    unsigned char* out;      // gemm0: Y; gemm1: P
+    unsigned char* out;      // gemm0: Y; gemm1: P (both in sorted-row order)
     unsigned char* y_scale;  // e8m0 block scales of Y (fp8 path): written by gemm0, read by gemm1
-    int* valid;              // gemm1: flags per (token, slot)
     int64_t x_row_bytes;
     int64_t w_row_bytes;
     int64_t w_expert_bytes;
@@ -50,7 +48,6 @@ struct GemmParams
     int n_total;             // weight rows per expert (gemm0: 2*inter, gemm1: hidden)
     int n_ntiles;            // tiles along n
     int tokens;
-    int topk;
 };
 
 template <int MODE>
@@ -263,15 +260,15 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
     }
 }
 
-// gemm1: * per-channel scale * top-k weight, bf16 partial row (token * topk + slot)
+// gemm1: * per-channel scale, bf16 partial row in sorted-row order (the combine applies the top-k weight)
 template <int MODE>
 __device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc,
-                                      const float (&ds)[16], int64_t prow, float topk_weight, bool store, int col0)
+                                      const float (&ds)[16], int64_t prow, bool store, int col0)
 {
     float y[16];
 #pragma unroll
     for(int v = 0; v < 16; v++)
-        y[v] = static_cast<float>(acc[v]) * ds[v] * topk_weight;
+        y[v] = static_cast<float>(acc[v]) * ds[v];
     uint4 o0, o1;
     o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
     o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
@@ -287,21 +284,14 @@ __device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTr
 
 // Shared tail of both GEMM kernels.  NBLK token blocks per wave: block i covers sorted rows
 // row0 + first_row + i * row_step + r32; wblk is the wave's first 32-row weight block of the tile.
-template <int MODE, bool GEMM0, int NBLK>
+// SKIP_PAD (gemm1): look the sorted id up and do not store partial rows of padding ids - worth the
+// load where padding dominates (decode: a handful of real rows per 32-row unit).
+template <int MODE, bool GEMM0, int NBLK, bool SKIP_PAD>
 __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2], int expert,
                                     int row0, int nrows, int first_row, int row_step, int nblk_live, int n_base,
-                                    int wblk, bool first_n_tile, int r32, int kg)
+                                    int wblk, int r32, int kg)
 {
     // ---- one batch of loads
-    int sid[NBLK];
-    float tw[NBLK];
-#pragma unroll
-    for(int i = 0; i < NBLK; i++)
-    {
-        const int r = min(first_row + i * row_step + r32, nrows - 1); // clamped: always a valid cell
-        sid[i]      = p.sorted_ids[row0 + r];
-        tw[i]       = GEMM0 ? 0.f : p.sorted_w[row0 + r];
-    }
     float sc0[16], sc1[16];
     const int col_a = GEMM0 ? n_base + wblk * 32 + 16 * kg : n_base + (wblk * 2) * 32 + 16 * kg;
     const int col_b = GEMM0 ? col_a : col_a + 32;
@@ -311,13 +301,20 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
     load_channel_scales(sbase && a_ok ? sbase + col_a : nullptr, sc0);
     load_channel_scales(sbase && b_ok ? sbase + (GEMM0 ? p.n_out + col_a : col_b) : nullptr, sc1);
     float sa[NBLK];
+    bool real[NBLK];
 #pragma unroll
     for(int i = 0; i < NBLK; i++)
     {
-        const int tok = sid[i] & 0xffffff;
-        sa[i]         = 1.0f;
-        if(GEMM0 && p.x_scale != nullptr)
-            sa[i] = tok < p.tokens ? p.x_scale[tok] : 0.0f;
+        sa[i]   = 1.0f;
+        real[i] = true;
+        if((GEMM0 && p.x_scale != nullptr) || (!GEMM0 && SKIP_PAD))
+        {
+            const int r   = min(first_row + i * row_step + r32, nrows - 1); // clamped: always a valid cell
+            const int tok = p.sorted_ids[row0 + r] & 0xffffff;
+            real[i]       = tok < p.tokens;
+            if constexpr(GEMM0)
+                sa[i] = real[i] ? p.x_scale[tok] : 0.0f;
+        }
     }
     // ---- apply
 #pragma unroll
@@ -327,7 +324,6 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
             continue;
         const int r        = first_row + i * row_step + r32;
         const bool in_tile = r < nrows;
-        const int tok      = sid[i] & 0xffffff;
         if constexpr(GEMM0)
         {
             if(a_ok)
@@ -335,14 +331,10 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
         }
         else
         {
-            const bool real    = in_tile && tok < p.tokens;
-            const int64_t prow = real ? (int64_t)tok * p.topk + static_cast<int>(static_cast<uint32_t>(sid[i]) >> 24) : 0;
-            if(real && first_n_tile && wblk == 0 && kg == 0)
-                p.valid[prow] = 1;
             if(a_ok)
-                epilogue_gemm1<MODE>(p, acc[i][0], sc0, prow, tw[i], real, col_a);
+                epilogue_gemm1<MODE>(p, acc[i][0], sc0, row0 + r, in_tile && real[i], col_a);
             if(b_ok)
-                epilogue_gemm1<MODE>(p, acc[i][1], sc1, prow, tw[i], real, col_b);
+                epilogue_gemm1<MODE>(p, acc[i][1], sc1, row0 + r, in_tile && real[i], col_b);
         }
     }
 }

@@ -56,7 +56,8 @@ __device__ inline int real_tokens(const int* local_tokens, int tokens)
 template <bool SCATTER>
 __device__ inline void walk_segment(const int* __restrict__ ids, const float* __restrict__ weights,
                                     int begin, int end, int K, int E, int nbits, int* cnt,
-                                    int* __restrict__ out_ids, float* __restrict__ out_w)
+                                    int* __restrict__ out_ids, float* __restrict__ out_w,
+                                    int* __restrict__ inv = nullptr)
 {
     const int lane = threadIdx.x & (kWave - 1);
     for(int i0 = begin; i0 < end; i0 += kWave)
@@ -72,6 +73,12 @@ __device__ inline void walk_segment(const int* __restrict__ ids, const float* __
         if(valid)
             base = cnt[e];
         wave_sync(); // every lane has read cnt[] before a leader updates it
+        if constexpr(SCATTER)
+        {
+            // inverse map for the grouped GEMMs' combine: where entry i went, -1 when it was dropped
+            if(inv != nullptr && i < end)
+                inv[i] = valid && base >= 0 ? base + before : -1;
+        }
         if(valid)
         {
             if constexpr(SCATTER)
@@ -267,12 +274,11 @@ __global__ __launch_bounds__(kScanBlock) void moe_sorting_oneshot_kernel(SortPar
     wave_sync();
     walk_segment<false>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, nullptr, nullptr);
     __syncthreads();
-    for(int i = threadIdx.x; i < p.plan.n_valid; i += kScanBlock)
-        p.plan.valid[i] = 0;
     scan_phase(sh, dyn_lds, kScanWaves, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
                p.sorted_eid, p.total, p.plan);
     __syncthreads();
-    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w);
+    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w,
+                       p.plan.tile_map != nullptr ? p.plan.inv : nullptr);
 }
 
 // ---- pass 1: per-segment expert histogram; trailing blocks zero moe_buf
@@ -287,8 +293,6 @@ __global__ __launch_bounds__(kWalkBlock) void moe_sorting_count_kernel(SortParam
                     (int64_t)(gridDim.x - p.work_blocks) * kWalkBlock);
         return;
     }
-    for(int i = blockIdx.x * kWalkBlock + threadIdx.x; i < p.plan.n_valid; i += p.work_blocks * kWalkBlock)
-        p.plan.valid[i] = 0;
     const int N    = T * p.K;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -332,7 +336,8 @@ __global__ __launch_bounds__(kWalkBlock) void moe_sorting_scatter_kernel(SortPar
     wave_sync();
     const int begin = min(seg * kSeg, N);
     const int end   = min(begin + kSeg, N);
-    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w);
+    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w,
+                       p.plan.tile_map != nullptr ? p.plan.inv : nullptr);
 }
 
 inline bool use_oneshot(int64_t entries, int experts)
