@@ -74,8 +74,10 @@ struct KernelTimer
 };
 
 // ---- work list of the grouped GEMMs: int32 [kMapHdr + kMapEnt * max_tiles]; [0] = live tiles, then per
-// tile (local expert id, first sorted row, rows, first tile of the expert, tiles of the expert, 0, 0, 0)
-constexpr int kMapHdr = 4;
+// tile (local expert id, first sorted row, rows, first tile of the expert, tiles of the expert, first sorted
+// row of the expert, rows of the expert, rows per tile of the expert): any tile of an expert can be worked
+// out from the entry of any other.  Entries are 32-byte aligned.
+constexpr int kMapHdr = 8;
 constexpr int kMapEnt = 8;
 
 // what the sort can prepare for the GEMMs while it has the per-expert counts at hand

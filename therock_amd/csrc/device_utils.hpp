@@ -66,9 +66,16 @@ __device__ inline uint32_t float_to_bf16_bits(float f)
     return u >> 16;
 }
 
+// two floats -> packed bf16 pair, round-to-nearest-even: a single v_cvt_pk_bf16_f32 on gfx950
 __device__ inline uint32_t pack_bf16x2(float lo, float hi)
 {
-    return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    const f32x2_t v  = {lo, hi};
+    const bf16x2_t b = __builtin_convertvector(v, bf16x2_t);
+    uint32_t r;
+    __builtin_memcpy(&r, &b, sizeof(r));
+    return r;
 }
 
 } // namespace mi355

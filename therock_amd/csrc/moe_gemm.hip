@@ -328,6 +328,9 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
                 ent[2]   = min(per, rows - j * per);
                 ent[3]   = tb;
                 ent[4]   = nt;
+                ent[5]   = lo * unit;
+                ent[6]   = rows;
+                ent[7]   = per;
             }
         }
     }
@@ -615,11 +618,16 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.k_bytes_w       = H * eb;
     p.n_out           = I;
     p.n_total         = 2 * I;
-    p.n_ntiles        = ceil_div(I, 128);
+    // decode-sized problems (one 32-row block per tile) have their own kernel
+    const bool decode = mblk == 1 && decode_supported((int64_t)T * a.stride_token * eb, ws.max_pad * (int64_t)I * y_b,
+                                                      (int64_t)2 * I * H * eb);
+    p.n_ntiles        = decode ? ceil_div(I, decode_tile_cols(true)) : ceil_div(I, 128);
     if(mblk > 4 && (int64_t)T * p.x_row_bytes >= ((int64_t)1 << 32))
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: a token buffer of 4 GiB or more (stride_token=%d) is not "
                                              "supported at this problem size", a.stride_token);
-    if(mblk > 4)
+    if(decode)
+        rc = launch_gemm_decode(t.prec_i, true, p, ws.max_tiles, stream);
+    else if(mblk > 4)
         rc = launch_gemm_big(t.prec_i, true, p, ws.max_tiles, stream);
     else if(t.prec_i == MI355_MOE_BF16)
         rc = launch_gemm<kBf16, true>(mblk, p, ws.max_tiles, stream);
@@ -644,8 +652,14 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.k_bytes_w      = I * eb;
     p.n_out          = H;
     p.n_total        = H;
-    p.n_ntiles       = ceil_div(H, 256);
-    if(mblk > 4)
+    // down GEMM: rows of I bytes are short enough for the 256-row tiles to stream well, and the narrow
+    // decode tiles re-read Y once per 64 output columns; they pay off only where the wide tiles would
+    // leave most compute units without a workgroup
+    const bool decode1 = decode && (int64_t)std::min<int64_t>(E, (int64_t)T * K) * ceil_div(H, 256) < device_info().num_cu;
+    p.n_ntiles       = decode1 ? ceil_div(H, decode_tile_cols(false)) : ceil_div(H, 256);
+    if(decode1)
+        rc = launch_gemm_decode(t.prec_i, false, p, ws.max_tiles, stream);
+    else if(mblk > 4)
         rc = launch_gemm_big(t.prec_i, false, p, ws.max_tiles, stream);
     else if(t.prec_i == MI355_MOE_BF16)
         rc = launch_gemm<kBf16, false>(mblk, p, ws.max_tiles, stream);

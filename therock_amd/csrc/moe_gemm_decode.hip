@@ -1,0 +1,297 @@
+// Grouped GEMM for decode-sized expert batches (at most one 32-row block per expert tile; gfx950).
+//
+// With a handful of tokens per expert the two GEMMs are pure weight streaming, and what decides
+// the rate is the shape of the HBM requests: 128-byte pieces of 256 different rows (the tile shape
+// of moe_gemm_kernel) reach about 5.3 TB/s on rows of 4 KB, 512 contiguous bytes per row about
+// 6.9 TB/s.  So here a workgroup owns only 64 weight rows (gate+up GEMM: 32 gate + 32 up rows = 32 Y
+// columns) and walks K in steps of 512 bytes per row.  The four waves split each step along K: wave
+// w multiplies bytes [128 w, 128 w + 128) of every row with the matching token columns, and the four
+// partial accumulators are added through LDS at the end (in wave order, so the result is
+// deterministic).  Same MFMA orientation (weight rows on the M side), operand layouts and epilogues
+// as moe_gemm_kernel; operand tiles are staged through LDS with the next step prefetched into
+// registers, weights with non-temporal loads.
+#include "moe_gemm_device.hpp"
+
+#include <algorithm>
+#include <type_traits>
+
+namespace mi355 {
+using namespace gemm;
+namespace {
+
+constexpr int kDecWRows = 64;  // weight rows per workgroup
+constexpr int kDecWKB   = 512; // weight bytes per row and step
+
+template <int MODE, bool GEMM0>
+__global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) void moe_gemm_decode_kernel(const GemmParams p)
+{
+    using MT  = ModeTraits<MODE>;
+    using Acc = typename MT::Acc;
+    constexpr int kOpB     = MT::kOpB;
+    constexpr int kXMul    = MT::kXKB / MT::kWKB;     // token bytes per weight byte (2 for bf16 x int8)
+    constexpr int kXKB     = kDecWKB * kXMul;         // token bytes per row and step
+    constexpr int kWStride = kDecWKB + kPadB;
+    constexpr int kXStride = kXKB + kPadB;
+    constexpr int kWaveWB  = kDecWKB / 4;             // weight bytes of a row one wave multiplies per step
+    constexpr int kSteps   = kWaveWB * kXMul / (2 * kOpB); // MFMAs along K per wave and step
+    constexpr int kWLoads  = kDecWRows * (kDecWKB / 16) / kBlock; // 8
+    constexpr int kXLoads  = 32 * (kXKB / 16) / kBlock;           // 4 or 8
+    constexpr int kWRowsPerPass = kBlock / (kDecWKB / 16);        // 8
+    constexpr int kXRowsPerPass = kBlock / (kXKB / 16);
+    constexpr bool kMx     = MODE == kFp8 && !GEMM0;
+    constexpr int kNTile   = GEMM0 ? 32 : 64;
+
+    extern __shared__ __align__(16) unsigned char lds[];
+    unsigned char* lds_w = lds;
+    unsigned char* lds_x = lds + kDecWRows * kWStride;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int r32  = lane & 31;
+    const int kg   = lane >> 5;
+
+    // ---- work item (same XCD-aware order as moe_gemm_kernel)
+    const int live_tiles = p.tile_map[0];
+    const int total      = live_tiles * p.n_ntiles;
+    const int per_xcd    = ceil_div(total, 8);
+    const int slot       = blockIdx.x >> 3;
+    const int work       = (blockIdx.x & 7) * per_xcd + slot;
+    if(slot >= per_xcd || work >= total)
+        return;
+    int mt, nt;
+    {
+        const int t0     = work / p.n_ntiles;
+        const int* ent0  = p.tile_map + kMapHdr + t0 * kMapEnt;
+        const int first  = ent0[3];
+        const int ntiles = ent0[4];
+        const int rel    = work - first * p.n_ntiles;
+        nt               = rel / ntiles;
+        mt               = first + (rel - nt * ntiles);
+    }
+    const int* ent   = p.tile_map + kMapHdr + mt * kMapEnt;
+    const int expert = ent[0];
+    const int row0   = ent[1];
+    const int nrows  = min(ent[2], 32);
+    const int n_base = nt * kNTile;
+
+    // ---- global -> register staging assignments: 32 consecutive lanes fetch 512 contiguous bytes
+    const int xchunk = tid % (kXKB / 16);
+    const int xrow   = tid / (kXKB / 16);
+    // addresses are a uniform base plus a 32-bit byte offset (the launcher checks that this suffices)
+    uint32_t xoff[kXLoads];
+    bool xvalid[kXLoads];
+#pragma unroll
+    for(int j = 0; j < kXLoads; j++)
+    {
+        const int r = xrow + kXRowsPerPass * j;
+        if constexpr(GEMM0)
+        {
+            int tok = p.tokens;
+            if(r < nrows)
+                tok = p.sorted_ids[row0 + r] & 0xffffff;
+            xvalid[j] = tok < p.tokens;
+            xoff[j]   = (uint32_t)(xvalid[j] ? tok : 0) * (uint32_t)p.x_row_bytes + xchunk * 16;
+        }
+        else
+        {
+            xvalid[j] = r < nrows;
+            xoff[j]   = (uint32_t)(row0 + (xvalid[j] ? r : 0)) * (uint32_t)p.x_row_bytes + xchunk * 16;
+        }
+    }
+    const int wchunk = tid % (kDecWKB / 16);
+    const int wrow   = tid / (kDecWKB / 16);
+    const unsigned char* wbase = p.w + (int64_t)expert * p.w_expert_bytes;
+    uint32_t woff[kWLoads];
+#pragma unroll
+    for(int j = 0; j < kWLoads; j++)
+    {
+        const int lrow = wrow + kWRowsPerPass * j;
+        const int blk  = lrow >> 5;
+        const int c    = chan_of_row(lrow & 31);
+        int grow;
+        if constexpr(GEMM0)
+            grow = blk * p.n_out + min(n_base + c, p.n_out - 1);
+        else
+            grow = min(n_base + blk * 32 + c, p.n_total - 1);
+        woff[j] = (uint32_t)grow * (uint32_t)p.w_row_bytes + wchunk * 16;
+    }
+
+    // two steps are kept in flight per workgroup: with three workgroups on a compute unit that is what it
+    // takes to have enough bytes outstanding to cover the HBM latency
+    uint4 xv_[2][kXLoads];
+    uint4 wv_[2][kWLoads];
+    uint32_t ys_next_[2] = {0x7f7f7f7fu, 0x7f7f7f7fu}, ys_cur = 0x7f7f7f7fu;
+    const uint4 zero4 = {0u, 0u, 0u, 0u};
+
+    auto load_tiles = [&](int kt, auto buf_tag) __attribute__((always_inline)) {
+        constexpr int B   = decltype(buf_tag)::value;
+        auto& xv          = xv_[B];
+        auto& wv          = wv_[B];
+        uint32_t& ys_next = ys_next_[B];
+        const int kx = kt * kXKB + xchunk * 16;
+#pragma unroll
+        for(int j = 0; j < kXLoads; j++)
+        {
+            xv[j] = zero4;
+            if(xvalid[j] && kx < p.k_bytes_x)
+                xv[j] = *reinterpret_cast<const uint4*>(p.x + (xoff[j] + (uint32_t)(kt * kXKB)));
+        }
+        const int kw = kt * kDecWKB + wchunk * 16;
+#pragma unroll
+        for(int j = 0; j < kWLoads; j++)
+        {
+            wv[j] = zero4;
+            if(kw < p.k_bytes_w)
+            {
+                typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+                const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wbase + (woff[j] + (uint32_t)(kt * kDecWKB))));
+                wv[j]           = make_uint4(t[0], t[1], t[2], t[3]);
+            }
+        }
+        if constexpr(kMx)
+        {
+            // the four e8m0 scales of this wave's 128 columns of the step
+            ys_next         = 0x7f7f7f7fu;
+            const int kb    = kt * (kDecWKB / 32) + wave * 4;
+            if(r32 < nrows && kb * 32 < p.k_bytes_x)
+            {
+                const unsigned char* sp = p.y_scale + (int64_t)kb * p.ys_kb_stride + row0 + r32;
+                ys_next = sp[0] | (sp[p.ys_kb_stride] << 8) | (sp[2 * p.ys_kb_stride] << 16) |
+                          (static_cast<uint32_t>(sp[3 * p.ys_kb_stride]) << 24);
+            }
+        }
+    };
+
+    Acc acc[1][2];
+#pragma unroll
+    for(int b = 0; b < 2; b++)
+#pragma unroll
+        for(int v = 0; v < 16; v++)
+            acc[0][b][v] = 0;
+
+    const int kt_count = ceil_div(p.k_bytes_w, kDecWKB);
+    auto k_step = [&](int kt, auto buf_tag) __attribute__((always_inline)) {
+        constexpr int B = decltype(buf_tag)::value;
+        auto& xv        = xv_[B];
+        auto& wv        = wv_[B];
+#pragma unroll
+        for(int j = 0; j < kXLoads; j++)
+            *reinterpret_cast<uint4*>(lds_x + (xrow + kXRowsPerPass * j) * kXStride + xchunk * 16) = xv[j];
+#pragma unroll
+        for(int j = 0; j < kWLoads; j++)
+            *reinterpret_cast<uint4*>(lds_w + (wrow + kWRowsPerPass * j) * kWStride + wchunk * 16) = wv[j];
+        ys_cur = ys_next_[B];
+        __syncthreads();
+        if(kt + 2 < kt_count)
+            load_tiles(kt + 2, buf_tag);
+        const unsigned char* xp = lds_x + r32 * kXStride + wave * kWaveWB * kXMul;
+#pragma unroll
+        for(int s = 0; s < kSteps; s++)
+        {
+            Frag wf[2], xf;
+            uint32_t xs = 127;
+#pragma unroll
+            for(int b = 0; b < 2; b++)
+            {
+                const unsigned char* wp = lds_w + (b * 32 + r32) * kWStride + wave * kWaveWB;
+                if constexpr(MODE == kBf16W8)
+                    wf[b].lo = int8x8_to_bf16x8(*reinterpret_cast<const uint2*>(wp + (2 * s + kg) * 8));
+                else if constexpr(kOpB == 16)
+                    wf[b].lo = *reinterpret_cast<const uint4*>(wp + (2 * s + kg) * 16);
+                else
+                {
+                    wf[b].lo = *reinterpret_cast<const uint4*>(wp + (4 * s + kg) * 16);
+                    wf[b].hi = *reinterpret_cast<const uint4*>(wp + (4 * s + 2 + kg) * 16);
+                }
+            }
+            if constexpr(kOpB == 16)
+                xf.lo = *reinterpret_cast<const uint4*>(xp + (2 * s + kg) * 16);
+            else
+            {
+                xf.lo = *reinterpret_cast<const uint4*>(xp + (4 * s + kg) * 16);
+                xf.hi = *reinterpret_cast<const uint4*>(xp + (4 * s + 2 + kg) * 16);
+                if constexpr(kMx)
+                    xs = (ys_cur >> (8 * (2 * s + kg))) & 0xffu;
+            }
+            acc[0][0] = mfma<MODE>(wf[0], xf, xs, acc[0][0]);
+            acc[0][1] = mfma<MODE>(wf[1], xf, xs, acc[0][1]);
+        }
+        __syncthreads();
+    };
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    load_tiles(0, B0{});
+    if(1 < kt_count)
+        load_tiles(1, B1{});
+    for(int kt = 0; kt < kt_count; kt += 2)
+    {
+        k_step(kt, B0{});
+        if(kt + 1 < kt_count)
+            k_step(kt + 1, B1{});
+    }
+
+    // ---- add the four K slices: waves 1..3 park their accumulators in LDS, wave 0 sums in wave order
+    using AccElem   = decltype(acc[0][0][0] + acc[0][0][0]);
+    AccElem* red    = reinterpret_cast<AccElem*>(lds); // [3][2][16][64]
+    if(wave > 0)
+    {
+#pragma unroll
+        for(int b = 0; b < 2; b++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                red[(((wave - 1) * 2 + b) * 16 + v) * 64 + lane] = acc[0][b][v];
+    }
+    __syncthreads();
+    if(wave > 0)
+        return;
+#pragma unroll
+    for(int w = 0; w < 3; w++)
+#pragma unroll
+        for(int b = 0; b < 2; b++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                acc[0][b][v] += red[((w * 2 + b) * 16 + v) * 64 + lane];
+
+    run_epilogue<MODE, GEMM0, 1, true>(p, acc, expert, row0, nrows, 0, 32, 1, n_base, 0, r32, kg);
+}
+
+template <int MODE, bool GEMM0>
+int launch_decode_t(const GemmParams& p, int max_tiles, hipStream_t stream)
+{
+    using MT            = ModeTraits<MODE>;
+    constexpr int kXMul = MT::kXKB / MT::kWKB;
+    const size_t lds    = kDecWRows * (kDecWKB + kPadB) + 32 * (kDecWKB * kXMul + kPadB);
+    static_assert(3 * 2 * 16 * 64 * 4 <= kDecWRows * (kDecWKB + kPadB), "reduction buffer fits in the weight tile");
+    const int grid = round_up(max_tiles * p.n_ntiles, 8);
+    if(grid <= 0)
+        return MI355_MOE_OK;
+    KernelTimer timer(GEMM0 ? MI355_MOE_K_GEMM0 : MI355_MOE_K_GEMM1, stream);
+    hipLaunchKernelGGL((moe_gemm_decode_kernel<MODE, GEMM0>), dim3(grid), dim3(kBlock), lds, stream, p);
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+} // namespace
+
+int decode_tile_cols(bool gemm0) { return gemm0 ? 32 : 64; }
+
+// byte offsets inside the token buffer, Y and one expert's weights must fit 32 bits
+bool decode_supported(int64_t x_bytes, int64_t y_bytes, int64_t w_expert_bytes)
+{
+    const int64_t lim = (int64_t)1 << 32;
+    return x_bytes < lim && y_bytes < lim && w_expert_bytes < lim;
+}
+
+int launch_gemm_decode(int prec, bool gemm0, const GemmParams& p, int max_tiles, hipStream_t stream)
+{
+    if(prec == MI355_MOE_BF16)
+        return gemm0 ? launch_decode_t<kBf16, true>(p, max_tiles, stream) : launch_decode_t<kBf16, false>(p, max_tiles, stream);
+    if(prec == MI355_MOE_FP8)
+        return gemm0 ? launch_decode_t<kFp8, true>(p, max_tiles, stream) : launch_decode_t<kFp8, false>(p, max_tiles, stream);
+    if(prec == MI355_MOE_INT8)
+        return gemm0 ? launch_decode_t<kI8, true>(p, max_tiles, stream) : launch_decode_t<kBf16W8, false>(p, max_tiles, stream);
+    return fail(MI355_MOE_E_UNSUPPORTED, "no decode kernel for precision %d", prec);
+}
+
+} // namespace mi355

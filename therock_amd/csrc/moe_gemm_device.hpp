@@ -316,6 +316,15 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
                 sa[i] = real[i] ? p.x_scale[tok] : 0.0f;
         }
     }
+    // every load above completes here, on every path: a load left pending on a path that does not use
+    // its result would make the compiler guard later register reuse with a wait for all vector memory
+    // operations - inside the caller's K loop when the caller is a persistent kernel
+#pragma unroll
+    for(int v = 0; v < 16; v++)
+        asm volatile("" : "+v"(sc0[v]), "+v"(sc1[v]));
+#pragma unroll
+    for(int i = 0; i < NBLK; i++)
+        asm volatile("" : "+v"(sa[i]));
     // ---- apply
 #pragma unroll
     for(int i = 0; i < NBLK; i++)

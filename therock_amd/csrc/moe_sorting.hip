@@ -216,6 +216,9 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
                 ent[2]   = min(per, rows - j * per);
                 ent[3]   = tb;
                 ent[4]   = nt;
+                ent[5]   = s.tbase[tid] * U;
+                ent[6]   = rows;
+                ent[7]   = per;
             }
         }
         if(tid == 0)
