@@ -106,27 +106,13 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     const int ww   = wave & 3;  // weight-row quarter
 
     // ---- work item (same XCD-aware order as moe_gemm_kernel)
-    const int live_tiles = p.tile_map[0];
-    const int total      = live_tiles * p.n_ntiles;
-    const int per_xcd    = ceil_div(total, 8);
-    const int slot       = blockIdx.x >> 3;
-    const int work       = (blockIdx.x & 7) * per_xcd + slot;
-    if(slot >= per_xcd || work >= total)
+    const TileRef tile = lookup_tile(p.tile_map, p.n_ntiles, blockIdx.x);
+    if(!tile.ok)
         return;
-    int mt, nt;
-    {
-        const int t0     = work / p.n_ntiles;
-        const int* ent0  = p.tile_map + kMapHdr + t0 * kMapEnt;
-        const int first  = ent0[3];
-        const int ntiles = ent0[4];
-        const int rel    = work - first * p.n_ntiles;
-        nt               = rel / ntiles;
-        mt               = first + (rel - nt * ntiles);
-    }
-    const int* ent   = p.tile_map + kMapHdr + mt * kMapEnt;
-    const int expert = ent[0];
-    const int row0   = ent[1];
-    const int nrows  = ent[2];
+    const int expert = tile.expert;
+    const int row0   = tile.row0;
+    const int nt     = tile.nt;
+    const int nrows  = tile.nrows;
     const int nmb    = ceil_div(nrows, 32);
     const int n_base = nt * (GEMM0 ? 128 : 256);
 

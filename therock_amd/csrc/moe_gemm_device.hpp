@@ -50,6 +50,35 @@ struct GemmParams
     int tokens;
 };
 
+// Work item -> tile.  XCD x gets a contiguous range of the work list (workgroup ids are dealt
+// round-robin to the 8 XCDs); inside an expert the row tiles of one weight tile are adjacent.  One
+// entry of the list describes the whole expert, so a single load resolves any of its tiles.
+struct TileRef
+{
+    int expert, row0, nrows, nt; // nt: column tile
+    bool ok;
+};
+__device__ inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_ntiles, int block)
+{
+    TileRef t;
+    const int total   = tile_map[0] * n_ntiles;
+    const int per_xcd = ceil_div(total, 8);
+    const int slot    = block >> 3;
+    const int work    = (block & 7) * per_xcd + slot;
+    t.ok              = slot < per_xcd && work < total;
+    const int t0      = t.ok ? work / n_ntiles : 0;
+    const int4* e     = reinterpret_cast<const int4*>(tile_map + kMapHdr + t0 * kMapEnt);
+    const int4 a      = e[0]; // expert, row0, nrows, first tile of the expert
+    const int4 b      = e[1]; // tiles of the expert, its first row, its rows, rows per tile
+    const int rel     = work - a.w * n_ntiles;
+    t.nt              = rel / max(b.x, 1);
+    const int j       = rel - t.nt * b.x;
+    t.expert          = a.x;
+    t.row0            = b.y + j * b.w;
+    t.nrows           = min(b.w, b.z - j * b.w);
+    return t;
+}
+
 template <int MODE>
 struct ModeTraits;
 template <>
