@@ -149,6 +149,36 @@ inline float moe_sorting(moe_sorting_trait t, moe_sorting_args a, stream_config 
     });
 }
 
+// --------------------------------------------------------------------------------- topk_softmax
+// topk_softmax_trait / topk_softmax_kargs of CK's example/ck_tile/09_topk_softmax
+struct topk_softmax_trait
+{
+    std::string input_type  = "fp32"; // fp32 | bf16
+    std::string weight_type = "fp32";
+    int experts             = 0;
+    std::string activation  = "softmax"; // softmax | sigmoid
+    bool renormalize        = false;     // extension: divide the chosen weights by their sum
+};
+
+// ck_tile::TopkSoftmaxHostArgs (ops/topk_softmax/kernel/topk_softmax_kernel.hpp:15-25)
+struct topk_softmax_kargs : public mi355_topk_softmax_args
+{
+};
+
+inline float topk_softmax(topk_softmax_trait t, topk_softmax_kargs a, stream_config s = {})
+{
+    if((t.activation != "softmax" && t.activation != "sigmoid") || t.weight_type != "fp32" ||
+       (t.input_type != "fp32" && t.input_type != "bf16"))
+        return -1.f;
+    const mi355_topk_softmax_traits p{detail::dtype_of(t.input_type), detail::dtype_of(t.weight_type), t.experts,
+                                      t.activation == "sigmoid" ? 1 : 0, t.renormalize ? 1 : 0};
+    return detail::run_timed(s, [&] {
+        const int rc = mi355_topk_softmax(&p, &a, s.stream_id_);
+        detail::throw_on_error(rc, "topk_softmax");
+        return rc;
+    });
+}
+
 // ------------------------------------------------------------------------------------ fused_moe
 struct fused_moe_traits
 {

@@ -83,6 +83,36 @@ size_t mi355_moe_sorting_workspace_size(int32_t tokens, int32_t num_experts, int
  * example/ck_tile/13_moe_sorting; index type int32 and weight type fp32 are the only ones CK has */
 int mi355_moe_sorting(const mi355_moe_sorting_args* args, void* stream);
 
+/* ----------------------------------------------------------------------------- topk_softmax
+ * Router front-end.  Replaces ck_tile::TopkSoftmaxKernel behind TopkSoftmaxHostArgs
+ * (ops/topk_softmax/kernel/topk_softmax_kernel.hpp:15-25): softmax (or sigmoid) over the expert
+ * logits of every row, then the topk largest values in descending order with their expert ids.
+ * Output contract = ck_tile::reference_softmax + reference_topk (host/reference/reference_softmax.hpp:12-78,
+ * host/reference/reference_topk.hpp:30-103), fp32; equal values are ordered by expert id. */
+typedef struct mi355_topk_softmax_args
+{
+    const void* p_input;   /* [num_rows, stride_input] logits */
+    void* p_output;        /* [num_rows, stride_output] fp32 weights of the chosen experts */
+    void* p_indices;       /* [num_rows, stride_output] int32 expert ids */
+    int32_t num_rows;
+    int32_t num_experts;   /* at most 1024 */
+    int32_t topk;          /* at most 64 */
+    int32_t stride_input;  /* row stride of p_input in elements, at least num_experts */
+    int32_t stride_output; /* row stride of p_output / p_indices in elements, at least topk */
+} mi355_topk_softmax_args;
+
+/* topk_softmax_trait of CK's example/ck_tile/09_topk_softmax, enums for its strings */
+typedef struct mi355_topk_softmax_traits
+{
+    int32_t input_type;  /* mi355_moe_dtype: FP32 | BF16 */
+    int32_t weight_type; /* FP32 */
+    int32_t experts;     /* CK selects an instance by this upper bound; here informational */
+    int32_t activation;  /* 0 = softmax, 1 = sigmoid (TopkSoftmaxWarpPerRowProblem::ActivationIsSoftmax) */
+    int32_t renormalize; /* extension, 0 in CK: 1 = divide the chosen weights by their sum */
+} mi355_topk_softmax_traits;
+
+int mi355_topk_softmax(const mi355_topk_softmax_traits* traits, const mi355_topk_softmax_args* args, void* stream);
+
 /* ------------------------------------------------------------------------------- fused MoE */
 typedef struct mi355_fused_moe_traits
 {
@@ -202,7 +232,8 @@ enum mi355_moe_kernel_kind
     MI355_MOE_K_GEMM1        = 6,
     MI355_MOE_K_COMBINE      = 7,
     MI355_MOE_K_QUANT        = 8,
-    MI355_MOE_NUM_KERNELS    = 9
+    MI355_MOE_K_ROUTER       = 9,
+    MI355_MOE_NUM_KERNELS    = 10
 };
 int mi355_moe_profile_start(void);
 int mi355_moe_profile_stop(double* ms, int32_t* launches);

@@ -182,6 +182,36 @@ def ck_moe_sorting(topk_ids, weights, experts, unit, local_expert_mask=None, ski
     return ids, w, eid, int(pp)
 
 
+# ----------------------------------------------------------------------------- router
+def topk_softmax(logits, topk, sigmoid=False, renorm=False):
+    """Oracle router: softmax (or sigmoid) over the last axis of fp32 `logits` [rows, experts], then the
+    top-k values (descending; ties to the lower expert id) and expert ids."""
+    x = _c(logits, np.float32)
+    rows, experts = x.shape
+    w = np.empty((rows, topk), dtype=np.float32)
+    idx = np.empty((rows, topk), dtype=np.int32)
+    f = lib().moe_oracle_topk_softmax
+    f.restype = C.c_int
+    rc = f(_p(x), C.c_int32(rows), C.c_int32(experts), C.c_int32(topk), C.c_int32(int(bool(sigmoid))),
+           C.c_int32(int(bool(renorm))), _p(w), _p(idx))
+    if rc != 0:
+        raise ValueError(f"moe_oracle_topk_softmax failed ({rc})")
+    return w, idx
+
+
+def ck_topk_softmax(logits, topk):
+    """ck_tile::reference_softmax + reference_topk on fp32 logits."""
+    r = ck_ref()
+    if r is None:
+        raise RuntimeError("oracle/_ref is not built")
+    x = _c(logits, np.float32)
+    rows, experts = x.shape
+    w = np.empty((rows, topk), dtype=np.float32)
+    idx = np.empty((rows, topk), dtype=np.int32)
+    r.ck_ref_topk_softmax(_p(x), C.c_int32(rows), C.c_int32(experts), C.c_int32(topk), _p(w), _p(idx))
+    return w, idx
+
+
 # ----------------------------------------------------------------------------- fused MoE
 def fused_moe(a, a_dt, g, g_dt, d, d_dt, sorted_ids, sorted_w, sorted_eid, post_pad, block_m,
               tokens, experts, hidden, inter, topk, a_scale=None, g_scale=None, d_scale=None,

@@ -17,6 +17,8 @@
 #include "ck_tile/ops/elementwise/unary_element_wise_operation.hpp"
 #include "ck_tile/host/reference/reference_moe_sorting.hpp"
 #include "ck_tile/host/reference/reference_fused_moe.hpp"
+#include "ck_tile/host/reference/reference_softmax.hpp"
+#include "ck_tile/host/reference/reference_topk.hpp"
 
 using ck_tile::HostTensor;
 using ck_tile::index_t;
@@ -123,6 +125,21 @@ ck_ref_fused_moe_f32(const void* a, const void* g, const void* d, void* o, const
 {
     return run_fused<float, float, float>(a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad,
                                           block_m, T, E, H, I, K, gate_only);
+}
+
+// router: reference_softmax over the experts of each row, then reference_topk (sorted, largest)
+__attribute__((visibility("default"))) int
+ck_ref_topk_softmax(const float* x, int32_t rows, int32_t experts, int32_t topk, float* out_w, int32_t* out_idx)
+{
+    auto x_h = make_tensor<float>({(std::size_t)rows, (std::size_t)experts}, x);
+    HostTensor<float> y_h({(std::size_t)rows, (std::size_t)experts});
+    ck_tile::reference_softmax<float, float, float>(x_h, y_h);
+    HostTensor<float> v_h({(std::size_t)rows, (std::size_t)topk});
+    HostTensor<index_t> i_h({(std::size_t)rows, (std::size_t)topk});
+    ck_tile::reference_topk<float, index_t>(y_h, v_h, i_h, topk);
+    std::memcpy(out_w, v_h.data(), sizeof(float) * (std::size_t)rows * topk);
+    std::memcpy(out_idx, i_h.data(), sizeof(int32_t) * (std::size_t)rows * topk);
+    return 0;
 }
 
 // scalar conversions of the reference, for pinning the oracle's bf16 / e4m3 tables

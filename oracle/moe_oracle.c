@@ -16,6 +16,8 @@
  *   e4m3 (OCP) encode/decode  <- core/numeric/float8.hpp:600-660 (saturating RNE, +-448)
  *   row-wise quantisation     <- host/reference/reference_rowwise_quantization2d.hpp:12-31
  *   scale placement           <- host/reference/reference_moe_gemm.hpp:94-113,202-203
+ *   moe_oracle_topk_softmax   <- host/reference/reference_softmax.hpp:12-78 + host/reference/reference_topk.hpp:30-103
+ *                                (sigmoid variant: ops/topk_softmax/pipeline/topk_softmax_warp_per_row_pipeline.hpp:88-92)
  *
  * ck_tile's reference_fused_moe ignores its four scale tensors (:200-203).  For quantised
  * inputs the oracle is therefore *defined* as "de-quantise every operand to fp32 (q * scale)
@@ -28,6 +30,9 @@
  *   fused moe   - ck_tile's reference_fused_moe in oracle/_ref on the same inputs; an
  *                 independent dense (sorting-free) float64 formulation in numpy.
  *   bf16 / e4m3 - exhaustive comparison with torch's bfloat16 / float8_e4m3fn casts.
+ *   topk softmax- ck_tile's reference_softmax + reference_topk in oracle/_ref; closed forms (equal
+ *                 logits, shift invariance, weights of all experts sum to one), scipy's softmax and
+ *                 numpy's argsort on random rows.
  */
 #include <math.h>
 #include <stdint.h>
@@ -412,6 +417,59 @@ ORACLE_API int moe_oracle_fused_moe(const void* a, int a_dt, const float* a_scal
     if(!out_topk)
         free(part);
     return rc;
+}
+
+/* ------------------------------------------------------------------------------ router
+ * reference_softmax.hpp:39-74 (row maximum, sum of exp(x - max) in ascending expert order, exp / sum)
+ * followed by reference_topk.hpp:73-95 (the k largest, descending).  sigmoid != 0 replaces the softmax
+ * by 1 / (1 + exp(-x)) as the device pipeline does.  Ties, which the reference leaves to
+ * std::nth_element, go to the lower expert id.  x is fp32 [rows, experts] (the caller up-converts);
+ * renorm != 0 divides the k weights by their sum (an extension of this build's router, not in ck_tile). */
+ORACLE_API int moe_oracle_topk_softmax(const float* x, int32_t rows, int32_t experts, int32_t topk, int32_t sigmoid,
+                                       int32_t renorm, float* out_w, int32_t* out_idx)
+{
+    if(rows < 0 || experts <= 0 || topk <= 0 || topk > experts)
+        return -1;
+    float* y = (float*)malloc(sizeof(float) * (size_t)experts);
+    if(!y)
+        return -2;
+    for(int64_t r = 0; r < rows; r++)
+    {
+        const float* xr = x + r * experts;
+        if(sigmoid)
+        {
+            for(int e = 0; e < experts; e++)
+                y[e] = 1.0f / (1.0f + expf(-xr[e]));
+        }
+        else
+        {
+            float m = -INFINITY;
+            for(int e = 0; e < experts; e++)
+                m = m < xr[e] ? xr[e] : m;
+            float sum = 0.f;
+            for(int e = 0; e < experts; e++)
+                sum += expf(xr[e] - m);
+            for(int e = 0; e < experts; e++)
+                y[e] = expf(xr[e] - m) / sum;
+        }
+        float wsum = 0.f;
+        for(int i = 0; i < topk; i++)
+        {
+            int be = 0;
+            for(int e = 1; e < experts; e++)
+                if(y[e] > y[be])
+                    be = e;
+            out_w[r * topk + i]   = y[be];
+            out_idx[r * topk + i] = be;
+            wsum += y[be];
+            y[be] = -INFINITY;
+        }
+        if(renorm)
+            for(int i = 0; i < topk; i++)
+                out_w[r * topk + i] /= wsum;
+    }
+    free(y);
+    return 0;
 }
 
 /* threads the OpenMP loops above will use (reported as "cores" by the CPU baseline) */

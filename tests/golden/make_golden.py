@@ -103,6 +103,12 @@ def main():
                 "max_count": int(counts.max())}
     with open(os.path.join(HERE, "sorting_hashes.json"), "w") as f:
         json.dump(hashes, f, indent=1, sort_keys=True)
+    # 5. router: ck_tile::reference_softmax + reference_topk on seeded logits (64 rows x 128 experts, top-8)
+    rng = np.random.default_rng(2024)
+    logits = (rng.standard_normal((64, 128)) * 2.5).astype(np.float32)
+    rw, rids = oracle.ck_topk_softmax(logits, 8)
+    np.savez_compressed(os.path.join(HERE, "router_ck_reference.npz"), logits=logits, topk=np.int32(8), weights=rw,
+                        ids=rids)
     print("golden fixtures written to", HERE)
 
 

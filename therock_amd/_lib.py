@@ -55,11 +55,26 @@ class FusedMoeArgs(C.Structure):
     ]
 
 
+class TopkSoftmaxArgs(C.Structure):
+    _fields_ = [
+        ("p_input", C.c_void_p), ("p_output", C.c_void_p), ("p_indices", C.c_void_p), ("num_rows", C.c_int32),
+        ("num_experts", C.c_int32), ("topk", C.c_int32), ("stride_input", C.c_int32), ("stride_output", C.c_int32),
+    ]
+
+
+class TopkSoftmaxTraits(C.Structure):
+    _fields_ = [
+        ("input_type", C.c_int32), ("weight_type", C.c_int32), ("experts", C.c_int32), ("activation", C.c_int32),
+        ("renormalize", C.c_int32),
+    ]
+
+
 # every symbol include/mi355_moe.h declares: name -> (restype, argtypes)
 PROTOTYPES = {
     "mi355_moe_max_num_tokens_padded": (C.c_int64, [C.c_int32] * 4),
     "mi355_moe_sorting_workspace_size": (C.c_size_t, [C.c_int32] * 3),
     "mi355_moe_sorting": (C.c_int, [C.POINTER(SortingArgs), C.c_void_p]),
+    "mi355_topk_softmax": (C.c_int, [C.POINTER(TopkSoftmaxTraits), C.POINTER(TopkSoftmaxArgs), C.c_void_p]),
     "mi355_fused_moe_supported": (C.c_int, [C.POINTER(FusedMoeTraits)]),
     "mi355_fused_moe_workspace_size": (C.c_size_t, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
     "mi355_fused_moe_tile_rows": (C.c_int32, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
@@ -93,7 +108,7 @@ def load():
     return _lib
 
 
-NUM_KERNELS = 9
+NUM_KERNELS = 10
 
 
 def profile_start() -> None:

@@ -101,7 +101,7 @@ __attribute__((visibility("default"))) const char* mi355_moe_kernel_name(int32_t
 {
     static const char* names[MI355_MOE_NUM_KERNELS] = {
         "moe_sorting_oneshot", "moe_sorting_count", "moe_sorting_scan", "moe_sorting_scatter", "moe_prep",
-        "moe_gemm0_gate_up_silu", "moe_gemm1_down", "moe_combine", "rowwise_quant"};
+        "moe_gemm0_gate_up_silu", "moe_gemm1_down", "moe_combine", "rowwise_quant", "topk_softmax"};
     return kind >= 0 && kind < MI355_MOE_NUM_KERNELS ? names[kind] : "?";
 }
 
@@ -155,6 +155,14 @@ __attribute__((visibility("default"))) int mi355_moe_sorting(const mi355_moe_sor
     if(args == nullptr)
         return fail(MI355_MOE_E_INVALID, "moe_sorting: args is null");
     return launch_moe_sorting(*args, static_cast<hipStream_t>(stream));
+}
+
+__attribute__((visibility("default"))) int
+mi355_topk_softmax(const mi355_topk_softmax_traits* traits, const mi355_topk_softmax_args* args, void* stream)
+{
+    if(traits == nullptr || args == nullptr)
+        return fail(MI355_MOE_E_INVALID, "topk_softmax: traits or args is null");
+    return launch_topk_softmax(*traits, *args, static_cast<hipStream_t>(stream));
 }
 
 __attribute__((visibility("default"))) int mi355_fused_moe_supported(const mi355_fused_moe_traits* t)

@@ -93,6 +93,8 @@ struct GemmPlan
 // ---- sorting launcher shared by the stand-alone and the fused entry points
 int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, const GemmPlan* plan = nullptr);
 
+int launch_topk_softmax(const mi355_topk_softmax_traits& t, const mi355_topk_softmax_args& a, hipStream_t stream);
+
 size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk);
 
 } // namespace mi355

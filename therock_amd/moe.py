@@ -203,6 +203,24 @@ def rowwise_quant(x, q_dtype: str, stream=None):
     return q, scale
 
 
+def topk_softmax(logits, topk: int, activation: str = "softmax", renormalize: bool = False, stream=None):
+    """Router front-end (CK's topk_softmax(trait, kargs, stream)): softmax or sigmoid over the experts of
+    each row of `logits` [rows, experts] (fp32 or bf16), then the top-k weights (fp32, descending) and
+    expert ids (int32).  Returns (weights[rows, topk], ids[rows, topk])."""
+    import torch
+
+    rows, experts = logits.shape
+    assert logits.stride(1) == 1
+    kind = {torch.float32: "fp32", torch.bfloat16: "bf16"}[logits.dtype]
+    w = torch.empty((rows, topk), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((rows, topk), dtype=torch.int32, device=logits.device)
+    t = _lib.TopkSoftmaxTraits(_lib.DTYPES[kind], _lib.DTYPES["fp32"], experts,
+                               {"softmax": 0, "sigmoid": 1}[activation], int(bool(renormalize)))
+    a = _lib.TopkSoftmaxArgs(_ptr(logits), _ptr(w), _ptr(ids), rows, experts, topk, logits.stride(0) if rows else experts, topk)
+    _check(_lib.load().mi355_topk_softmax(C.byref(t), C.byref(a), _stream(stream)), "topk_softmax")
+    return w, ids
+
+
 # ------------------------------------------------------------------ convenience for harnesses
 def fused_moe_tile_rows(traits: fused_moe_traits, tokens, num_experts, topk, hidden_size, intermediate_size) -> int:
     """Sorted rows one GEMM workgroup owns at this problem size (320 selects the large-tile kernel)."""
