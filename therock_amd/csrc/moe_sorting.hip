@@ -53,6 +53,48 @@ __device__ inline int real_tokens(const int* local_tokens, int tokens)
 // One wave walks routing entries [begin, end) in order, 64 at a time.
 // cnt[e] holds (COUNT) the number of entries of expert e seen so far, or (SCATTER) the output
 // position of the next entry of expert e (negative: expert masked out, entries dropped).
+// One 64-entry step of a wave's walk: lane handles routing entry i (expert e, weight w; e = -1 past
+// the end).  cnt[e] holds (COUNT) the number of entries of expert e seen so far, or (SCATTER) the
+// output position of the next entry of expert e (negative: expert masked out, entries dropped).
+template <bool SCATTER>
+__device__ inline void walk_step(int i, int e, float w, bool in_range, int K, int E, int nbits, int* cnt,
+                                 int* __restrict__ out_ids, float* __restrict__ out_w, int* __restrict__ inv)
+{
+    const int lane   = threadIdx.x & (kWave - 1);
+    const bool valid = e >= 0 && e < E;
+    if(!valid)
+        e = 0;
+    const uint64_t same = match_expert(e, nbits) & __ballot(valid);
+    const int before    = __popcll(same & ((1ull << lane) - 1ull));
+    int base            = 0;
+    if(valid)
+        base = cnt[e];
+    wave_sync(); // every lane has read cnt[] before a leader updates it
+    if constexpr(SCATTER)
+    {
+        // inverse map for the grouped GEMMs' combine: where entry i went, -1 when it was dropped
+        if(inv != nullptr && in_range)
+            inv[i] = valid && base >= 0 ? base + before : -1;
+    }
+    if(valid)
+    {
+        if constexpr(SCATTER)
+        {
+            if(base >= 0)
+            {
+                const int t            = i / K;
+                const int k            = i - t * K;
+                out_ids[base + before] = mock_id(t, k);
+                out_w[base + before]   = w;
+            }
+        }
+        if(before == 0 && base >= 0)
+            cnt[e] = base + __popcll(same);
+    }
+    wave_sync();
+}
+
+// One wave walks routing entries [begin, end) in order, 64 at a time.
 template <bool SCATTER>
 __device__ inline void walk_segment(const int* __restrict__ ids, const float* __restrict__ weights,
                                     int begin, int end, int K, int E, int nbits, int* cnt,
@@ -62,39 +104,10 @@ __device__ inline void walk_segment(const int* __restrict__ ids, const float* __
     const int lane = threadIdx.x & (kWave - 1);
     for(int i0 = begin; i0 < end; i0 += kWave)
     {
-        const int i = i0 + lane;
-        int e       = i < end ? ids[i] : -1;
-        const bool valid = e >= 0 && e < E;
-        if(!valid)
-            e = 0;
-        const uint64_t same = match_expert(e, nbits) & __ballot(valid);
-        const int before    = __popcll(same & ((1ull << lane) - 1ull));
-        int base            = 0;
-        if(valid)
-            base = cnt[e];
-        wave_sync(); // every lane has read cnt[] before a leader updates it
-        if constexpr(SCATTER)
-        {
-            // inverse map for the grouped GEMMs' combine: where entry i went, -1 when it was dropped
-            if(inv != nullptr && i < end)
-                inv[i] = valid && base >= 0 ? base + before : -1;
-        }
-        if(valid)
-        {
-            if constexpr(SCATTER)
-            {
-                if(base >= 0)
-                {
-                    const int t        = i / K;
-                    const int k        = i - t * K;
-                    out_ids[base + before] = mock_id(t, k);
-                    out_w[base + before]   = weights[i];
-                }
-            }
-            if(before == 0 && base >= 0)
-                cnt[e] = base + __popcll(same);
-        }
-        wave_sync();
+        const int i   = i0 + lane;
+        const int e   = i < end ? ids[i] : -1;
+        const float w = SCATTER && i < end ? weights[i] : 0.f;
+        walk_step<SCATTER>(i, e, w, i < end, K, E, nbits, cnt, out_ids, out_w, inv);
     }
 }
 
@@ -275,13 +288,29 @@ __global__ __launch_bounds__(kScanBlock) void moe_sorting_oneshot_kernel(SortPar
     for(int e = lane; e < p.E; e += kWave)
         cnt[e] = 0;
     wave_sync();
+    int* inv = p.plan.tile_map != nullptr ? p.plan.inv : nullptr;
+    if(seglen == kWave)
+    {
+        // a single step per wave (at most 1024 entries: the decode regime): the entry is read once
+        // and stays in registers for both walks
+        const int i   = begin + lane;
+        const int e   = i < end ? p.ids[i] : -1;
+        const float w = i < end ? p.weights[i] : 0.f;
+        walk_step<false>(i, e, w, i < end, p.K, p.E, p.nbits, cnt, nullptr, nullptr, nullptr);
+        __syncthreads();
+        scan_phase(sh, dyn_lds, kScanWaves, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
+                   p.sorted_eid, p.total, p.plan);
+        __syncthreads();
+        if(begin < end)
+            walk_step<true>(i, e, w, i < end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w, inv);
+        return;
+    }
     walk_segment<false>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, nullptr, nullptr);
     __syncthreads();
     scan_phase(sh, dyn_lds, kScanWaves, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
                p.sorted_eid, p.total, p.plan);
     __syncthreads();
-    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w,
-                       p.plan.tile_map != nullptr ? p.plan.inv : nullptr);
+    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w, inv);
 }
 
 // ---- pass 1: per-segment expert histogram; trailing blocks zero moe_buf
