@@ -179,6 +179,31 @@ inline float topk_softmax(topk_softmax_trait t, topk_softmax_kargs a, stream_con
     });
 }
 
+// ------------------------------------------------------------------------------ moe_smoothquant
+// moe_smoothquant_traits / moe_smoothquant_args of CK's example/ck_tile/14_moe_smoothquant
+struct moe_smoothquant_traits
+{
+    std::string in_type  = "bf16"; // input type
+    std::string out_type = "int8"; // int8 | fp8
+};
+
+// ck_tile::MoeSmoothquantHostArgs (ops/smoothquant/kernel/moe_smoothquant_kernel.hpp:12-27)
+struct moe_smoothquant_args : public mi355_moe_smoothquant_args
+{
+};
+
+inline float moe_smoothquant(moe_smoothquant_traits t, moe_smoothquant_args a, stream_config s = {})
+{
+    if(t.in_type != "bf16" || (t.out_type != "int8" && t.out_type != "fp8"))
+        return -1.f;
+    const int32_t q = detail::dtype_of(t.out_type);
+    return detail::run_timed(s, [&] {
+        const int rc = mi355_moe_smoothquant(&a, q, s.stream_id_);
+        detail::throw_on_error(rc, "moe_smoothquant");
+        return rc;
+    });
+}
+
 // ------------------------------------------------------------------------------------ fused_moe
 struct fused_moe_traits
 {

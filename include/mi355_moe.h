@@ -210,10 +210,33 @@ int mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_
 int mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* args, void* stream);
 
 /* per-row dynamic quantisation of bf16 activations, the step in front of the quantised path:
- * scale[m] = amax(row)/qmax, q = saturate(x/scale) (host/reference/reference_rowwise_quantization2d.hpp:12-31).
+ * scale[m] = amax(row)/qmax, q = convert(saturate(x/scale)) (host/reference/reference_rowwise_quantization2d.hpp:12-31);
+ * as in ck_tile the int8 conversion truncates toward zero (core/numeric/int8.hpp:101), e4m3 rounds to nearest even.
  * x [rows, stride_x] bf16 -> q [rows, cols] (FP8 or INT8), scale [rows] fp32. */
 int mi355_moe_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype,
                             void* q, void* scale, void* stream);
+
+/* MoE smooth-quant in front of the int8 / fp8 path.  Replaces ck_tile::MoeSmoothquant behind
+ * MoeSmoothquantHostArgs (ops/smoothquant/kernel/moe_smoothquant_kernel.hpp:12-27): for slot k of token t
+ * routed to expert e = topk_ids[t, k]: y = x[t, :] * smscale[e, :] (fp32), yscale[k * tokens + t] =
+ * amax|y| / qmax, qy[k * tokens + t, :] = convert(saturate(y / yscale))
+ * (ops/smoothquant/pipeline/smoothquant_pipeline_one_pass.hpp:73-118). */
+typedef struct mi355_moe_smoothquant_args
+{
+    const void* p_x;        /* [tokens, x_stride] bf16 */
+    const void* p_smscale;  /* [experts, hidden_size] fp32 column-wise smooth scale */
+    const void* p_topk_ids; /* [tokens, topk] int32 */
+    void* p_yscale;         /* [topk * tokens] fp32 row-wise quantisation scale */
+    void* p_qy;             /* [topk * tokens, y_stride] int8 or e4m3 */
+    int32_t tokens;
+    int32_t hidden_size;
+    int32_t experts;
+    int32_t topk;
+    int32_t x_stride; /* row stride of x in elements */
+    int32_t y_stride; /* row stride of qy in elements */
+} mi355_moe_smoothquant_args;
+
+int mi355_moe_smoothquant(const mi355_moe_smoothquant_args* args, int32_t q_dtype, void* stream);
 
 /* ------------------------------------------------------------------------------ kernel timing
  * Counterpart of ck_tile::stream_config::time_kernel_ (host/stream_config.hpp:29-39,

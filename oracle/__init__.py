@@ -126,16 +126,46 @@ def to_f32(x: np.ndarray, dt: int) -> np.ndarray:
     return np.asarray(x, dtype=np.int8).astype(np.float32)
 
 
-def rowwise_quant(x: np.ndarray, dt: int):
-    """Per-row dynamic quantisation of a float32 [M,N] matrix -> (q, scale[M])."""
+def rowwise_quant(x: np.ndarray, dt: int, nearest: bool = False):
+    """Per-row dynamic quantisation of a float32 [M,N] matrix -> (q, scale[M]).  int8 values are
+    converted as ck_tile does (truncation toward zero) unless nearest=True (round to nearest even, the
+    quantiser of the synthetic benchmark inputs)."""
     x = _c(x, np.float32)
     M, N = x.shape
     q = np.empty((M, N), dtype=_NP_OF_DT[dt])
     s = np.empty((M,), dtype=np.float32)
-    rc = lib().moe_oracle_rowwise_quant(_p(x), C.c_int64(M), C.c_int64(N), C.c_int(dt), _p(q), _p(s))
+    rc = lib().moe_oracle_rowwise_quant2(_p(x), C.c_int64(M), C.c_int64(N), C.c_int(dt), C.c_int(int(nearest)),
+                                         _p(q), _p(s))
     if rc != 0:
         raise ValueError("rowwise_quant: unsupported dtype")
     return q, s
+
+
+def ck_rowwise_quant(x: np.ndarray, scale: np.ndarray, dt: int):
+    """ck_tile::reference_rowwise_quantization2d on fp32 rows with the given per-row scales."""
+    r = ck_ref()
+    if r is None:
+        raise RuntimeError("oracle/_ref is not built")
+    x, scale = _c(x, np.float32), _c(scale, np.float32)
+    M, N = x.shape
+    q = np.empty((M, N), dtype=_NP_OF_DT[dt])
+    r.ck_ref_rowwise_quant(_p(x), _p(scale), C.c_int32(M), C.c_int32(N), C.c_int32(int(dt == DT_E4M3)), _p(q))
+    return q
+
+
+def smoothquant(x, smscale, topk_ids, dt):
+    """MoE smooth-quant oracle: fp32 x [T,H], smscale [E,H], topk_ids [T,K] -> (qy [K,T,H], yscale [K,T])."""
+    x, smscale, topk_ids = _c(x, np.float32), _c(smscale, np.float32), _c(topk_ids, np.int32)
+    T, H = x.shape
+    E = smscale.shape[0]
+    K = topk_ids.shape[1]
+    qy = np.empty((K, T, H), dtype=_NP_OF_DT[dt])
+    ys = np.empty((K, T), dtype=np.float32)
+    rc = lib().moe_oracle_smoothquant(_p(x), _p(smscale), _p(topk_ids), C.c_int32(T), C.c_int32(H), C.c_int32(E),
+                                      C.c_int32(K), C.c_int(dt), _p(qy), _p(ys))
+    if rc != 0:
+        raise ValueError(f"moe_oracle_smoothquant failed ({rc})")
+    return qy, ys
 
 
 # ------------------------------------------------------------------------------- sorting

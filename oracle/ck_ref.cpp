@@ -19,6 +19,7 @@
 #include "ck_tile/host/reference/reference_fused_moe.hpp"
 #include "ck_tile/host/reference/reference_softmax.hpp"
 #include "ck_tile/host/reference/reference_topk.hpp"
+#include "ck_tile/host/reference/reference_rowwise_quantization2d.hpp"
 
 using ck_tile::HostTensor;
 using ck_tile::index_t;
@@ -139,6 +140,27 @@ ck_ref_topk_softmax(const float* x, int32_t rows, int32_t experts, int32_t topk,
     ck_tile::reference_topk<float, index_t>(y_h, v_h, i_h, topk);
     std::memcpy(out_w, v_h.data(), sizeof(float) * (std::size_t)rows * topk);
     std::memcpy(out_idx, i_h.data(), sizeof(int32_t) * (std::size_t)rows * topk);
+    return 0;
+}
+
+// reference_rowwise_quantization2d on fp32 rows with caller-provided scales; q_is_fp8: e4m3 else int8
+__attribute__((visibility("default"))) int
+ck_ref_rowwise_quant(const float* x, const float* scale, int32_t M, int32_t N, int32_t q_is_fp8, void* q)
+{
+    auto x_h = make_tensor<float>({(std::size_t)M, (std::size_t)N}, x);
+    auto s_h = make_tensor<float>({(std::size_t)M}, scale);
+    if(q_is_fp8)
+    {
+        HostTensor<ck_tile::fp8_t> q_h({(std::size_t)M, (std::size_t)N});
+        ck_tile::reference_rowwise_quantization2d<float, float, ck_tile::fp8_t>(x_h, s_h, q_h);
+        std::memcpy(q, q_h.data(), (std::size_t)M * N);
+    }
+    else
+    {
+        HostTensor<ck_tile::int8_t> q_h({(std::size_t)M, (std::size_t)N});
+        ck_tile::reference_rowwise_quantization2d<float, float, ck_tile::int8_t>(x_h, s_h, q_h);
+        std::memcpy(q, q_h.data(), (std::size_t)M * N);
+    }
     return 0;
 }
 

@@ -142,11 +142,27 @@ ORACLE_API float moe_oracle_silu(float x) { return silu_f32(x); }
 
 /* -------------------------------------------------------------------------- quantisation */
 
-/* per-row dynamic quantisation: scale[m] = amax(row)/qmax, q = convert(saturate(x/scale)).
+/* one quantised element: saturate, then ck_tile's type_convert (core/numeric/int8.hpp:101: a plain
+ * static_cast for int8, i.e. truncation toward zero; core/numeric/float8.hpp: saturating RNE for e4m3).
+ * nearest != 0 rounds int8 to nearest-even instead (what the synthetic-input generator uses). */
+static inline void quant_store(void* q, int64_t i, float v, int dt, int nearest)
+{
+    if(dt == MOE_DT_E4M3)
+        ((uint8_t*)q)[i] = moe_oracle_f32_to_e4m3(v);
+    else
+    {
+        float c          = v > 127.f ? 127.f : (v < -128.f ? -128.f : v);
+        ((int8_t*)q)[i]  = nearest ? (int8_t)nearbyintf(c) : (int8_t)c;
+    }
+}
+
+/* per-row dynamic quantisation: scale[m] = amax(row)/qmax, q = convert(saturate(x/scale))
+ * (host/reference/reference_rowwise_quantization2d.hpp:12-31 with the scale the smooth-quant pipeline
+ * computes, ops/smoothquant/pipeline/smoothquant_pipeline_one_pass.hpp:103-117).
  * x is fp32 [M,N] (caller up-converts bf16).  dt = MOE_DT_E4M3 (qmax 448) or MOE_DT_I8 (127).
  * A row of zeros gets scale 1 so that no division by zero happens. */
-ORACLE_API int moe_oracle_rowwise_quant(const float* x, int64_t M, int64_t N, int dt, void* q,
-                                        float* scale)
+ORACLE_API int moe_oracle_rowwise_quant2(const float* x, int64_t M, int64_t N, int dt, int nearest, void* q,
+                                         float* scale)
 {
     if(dt != MOE_DT_E4M3 && dt != MOE_DT_I8)
         return -1;
@@ -165,17 +181,46 @@ ORACLE_API int moe_oracle_rowwise_quant(const float* x, int64_t M, int64_t N, in
         float s  = amax > 0.f ? amax / qmax : 1.0f;
         scale[m] = s;
         for(int64_t n = 0; n < N; n++)
-        {
-            float v = r[n] / s;
-            if(dt == MOE_DT_E4M3)
-                ((uint8_t*)q)[m * N + n] = moe_oracle_f32_to_e4m3(v);
-            else
-            {
-                float c = v > 127.f ? 127.f : (v < -128.f ? -128.f : v);
-                ((int8_t*)q)[m * N + n] = (int8_t)nearbyintf(c);
-            }
-        }
+            quant_store(q, m * N + n, r[n] / s, dt, nearest);
     }
+    return 0;
+}
+
+/* nearest-even variant kept under the old name: the quantiser of the synthetic benchmark inputs */
+ORACLE_API int moe_oracle_rowwise_quant(const float* x, int64_t M, int64_t N, int dt, void* q, float* scale)
+{
+    return moe_oracle_rowwise_quant2(x, M, N, dt, 1, q, scale);
+}
+
+/* MoE smooth-quant (ops/smoothquant/kernel/moe_smoothquant_kernel.hpp:12-27, 152-175 and
+ * pipeline/smoothquant_pipeline_one_pass.hpp:73-118): for slot k of token t routed to expert e,
+ * y = x[t,:] * smscale[e,:] in fp32, yscale[k*tokens + t] = amax|y| / qmax, qy[k*tokens + t, :] =
+ * convert(saturate(y / yscale)).  Outputs are [topk, tokens, hidden] and [topk, tokens]. */
+ORACLE_API int moe_oracle_smoothquant(const float* x, const float* smscale, const int32_t* topk_ids, int32_t tokens,
+                                      int32_t hidden, int32_t experts, int32_t topk, int dt, void* qy, float* yscale)
+{
+    if(dt != MOE_DT_E4M3 && dt != MOE_DT_I8)
+        return -1;
+    const float qmax = dt == MOE_DT_E4M3 ? 448.0f : 127.0f;
+    for(int64_t k = 0; k < topk; k++)
+        for(int64_t t = 0; t < tokens; t++)
+        {
+            const int e = topk_ids[t * topk + k];
+            if(e < 0 || e >= experts)
+                return -2;
+            const float* xr = x + t * hidden;
+            const float* sr = smscale + (int64_t)e * hidden;
+            float amax      = 0.f;
+            for(int64_t h = 0; h < hidden; h++)
+            {
+                const float a = fabsf(xr[h] * sr[h]);
+                amax          = a > amax ? a : amax;
+            }
+            const float ys           = amax / qmax;
+            yscale[k * tokens + t]   = ys;
+            for(int64_t h = 0; h < hidden; h++)
+                quant_store(qy, (k * tokens + t) * hidden + h, (xr[h] * sr[h]) / ys, dt, 0);
+        }
     return 0;
 }
 

@@ -84,7 +84,8 @@ def test_rowwise_quant_matches_definition():
     rng = np.random.default_rng(3)
     x = (rng.standard_normal((9, 160)) * np.array([1e-3, 0.1, 1, 3, 10, 50, 0, 1, 1])[:, None]).astype(np.float32)
     for dt, key, qmax in ((oracle.DT_I8, "int8", 127.0), (oracle.DT_E4M3, "fp8", 448.0)):
-        q, s = oracle.rowwise_quant(x, dt)
+        # nearest=True is the quantiser of the synthetic benchmark inputs (therock_amd.inputs)
+        q, s = oracle.rowwise_quant(x, dt, nearest=True)
         q2, s2 = mi.rowwise_quant_np(x, key)
         assert np.array_equal(s, s2) and np.array_equal(q, q2)
         amax = np.abs(x).max(axis=1)
@@ -94,6 +95,35 @@ def test_rowwise_quant_matches_definition():
         assert np.all(np.abs(deq - x) <= 0.5 * step[:, None] + 1e-12)
         # the row maximum is hit exactly
         assert np.all(np.abs(oracle.to_f32(q, dt)).max(axis=1)[amax > 0] == qmax)
+        # the default follows ck_tile's conversion: int8 truncates toward zero, e4m3 rounds to nearest
+        qt, st = oracle.rowwise_quant(x, dt)
+        assert np.array_equal(st, s)
+        if key == "int8":
+            assert np.array_equal(qt, np.trunc(np.clip(x / s[:, None], -128, 127)).astype(np.int8))
+        else:
+            assert np.array_equal(qt, q)
+
+
+@pytest.mark.skipif(oracle.ck_ref() is None, reason="oracle/_ref not built")
+def test_quantisers_match_ck_tile_reference():
+    """reference_rowwise_quantization2d on the same rows and scales, and the smooth-quant oracle against
+    that reference applied to x * smscale[expert]."""
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((37, 192)) * 4).astype(np.float32)
+    for dt in (oracle.DT_I8, oracle.DT_E4M3):
+        q, s = oracle.rowwise_quant(x, dt)
+        assert np.array_equal(q, oracle.ck_rowwise_quant(x, s, dt))
+    T, H, E, K = 19, 96, 6, 3
+    xb = oracle.to_f32(oracle.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32)), oracle.DT_BF16)
+    sm = (0.5 + rng.random((E, H))).astype(np.float32)
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
+    for dt, qmax in ((oracle.DT_I8, 127.0), (oracle.DT_E4M3, 448.0)):
+        qy, ys = oracle.smoothquant(xb, sm, ids, dt)
+        assert qy.shape == (K, T, H) and ys.shape == (K, T)
+        for k in range(K):
+            y = xb * sm[ids[:, k]]
+            assert np.array_equal(ys[k], np.abs(y).max(axis=1) / np.float32(qmax))
+            assert np.array_equal(qy[k], oracle.ck_rowwise_quant(y, ys[k], dt))
 
 
 @pytest.mark.skipif(oracle.ck_ref() is None, reason="oracle/_ref not built")

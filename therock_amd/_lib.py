@@ -69,6 +69,14 @@ class TopkSoftmaxTraits(C.Structure):
     ]
 
 
+class SmoothquantArgs(C.Structure):
+    _fields_ = [
+        ("p_x", C.c_void_p), ("p_smscale", C.c_void_p), ("p_topk_ids", C.c_void_p), ("p_yscale", C.c_void_p),
+        ("p_qy", C.c_void_p), ("tokens", C.c_int32), ("hidden_size", C.c_int32), ("experts", C.c_int32),
+        ("topk", C.c_int32), ("x_stride", C.c_int32), ("y_stride", C.c_int32),
+    ]
+
+
 # every symbol include/mi355_moe.h declares: name -> (restype, argtypes)
 PROTOTYPES = {
     "mi355_moe_max_num_tokens_padded": (C.c_int64, [C.c_int32] * 4),
@@ -80,6 +88,7 @@ PROTOTYPES = {
     "mi355_fused_moe_tile_rows": (C.c_int32, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
     "mi355_fused_moegemm": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeGemmArgs), C.c_void_p]),
     "mi355_fused_moe": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.c_void_p]),
+    "mi355_moe_smoothquant": (C.c_int, [C.POINTER(SmoothquantArgs), C.c_int32, C.c_void_p]),
     "mi355_moe_rowwise_quant": (C.c_int, [C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_int32, C.c_void_p,
                                           C.c_void_p, C.c_void_p]),
     "mi355_moe_profile_start": (C.c_int, []),

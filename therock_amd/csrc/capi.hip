@@ -262,6 +262,14 @@ mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args
 }
 
 __attribute__((visibility("default"))) int
+mi355_moe_smoothquant(const mi355_moe_smoothquant_args* args, int32_t q_dtype, void* stream)
+{
+    if(args == nullptr)
+        return fail(MI355_MOE_E_INVALID, "moe_smoothquant: args is null");
+    return launch_moe_smoothquant(*args, q_dtype, static_cast<hipStream_t>(stream));
+}
+
+__attribute__((visibility("default"))) int
 mi355_moe_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype, void* q,
                         void* scale, void* stream)
 {

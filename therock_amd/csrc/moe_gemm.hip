@@ -408,8 +408,56 @@ __global__ __launch_bounds__(256) void rowwise_quant_kernel(const uint16_t* __re
         }
         else
         {
+            // ck_tile's float -> int8 conversion is a static_cast: truncation toward zero
             const float cl = fminf(fmaxf(v, -128.f), 127.f);
-            q[row * cols + c] = static_cast<unsigned char>(static_cast<signed char>(__float2int_rn(cl)));
+            q[row * cols + c] = static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
+        }
+    }
+}
+
+// MoE smooth-quant: row (slot k, token t) = x[t, :] * smscale[expert(t, k), :], per-row dynamic quantisation
+template <bool FP8>
+__global__ __launch_bounds__(256) void moe_smoothquant_kernel(const uint16_t* __restrict__ x,
+                                                               const float* __restrict__ smscale,
+                                                               const int* __restrict__ topk_ids, int tokens, int hidden,
+                                                               int experts, int topk, int64_t x_stride, int64_t y_stride,
+                                                               unsigned char* __restrict__ qy, float* __restrict__ yscale)
+{
+    __shared__ float s_red[4];
+    const int t = blockIdx.x;
+    const int k = blockIdx.y;
+    int e       = topk_ids[(int64_t)t * topk + k];
+    e           = min(max(e, 0), experts - 1);
+    const uint16_t* xr = x + (int64_t)t * x_stride;
+    const float* sr    = smscale + (int64_t)e * hidden;
+    float amax         = 0.f;
+    for(int c = threadIdx.x; c < hidden; c += 256)
+        amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c]) * sr[c]));
+#pragma unroll
+    for(int d = 32; d > 0; d >>= 1)
+        amax = fmaxf(amax, __shfl_xor(amax, d));
+    if((threadIdx.x & 63) == 0)
+        s_red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax            = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    const float qmx = FP8 ? 448.0f : 127.0f;
+    const float ys  = amax / qmx;
+    const int64_t r = (int64_t)k * tokens + t;
+    if(threadIdx.x == 0)
+        yscale[r] = ys;
+    unsigned char* qr = qy + r * y_stride;
+    for(int c = threadIdx.x; c < hidden; c += 256)
+    {
+        const float v = (bf16_bits_to_float(xr[c]) * sr[c]) / ys;
+        if constexpr(FP8)
+        {
+            const float cl = fminf(fmaxf(v, -448.f), 448.f);
+            qr[c] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
+        }
+        else
+        {
+            const float cl = fminf(fmaxf(v, -128.f), 127.f);
+            qr[c] = static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
         }
     }
 }
@@ -663,6 +711,34 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
                        static_cast<const float*>(a.sorted_weight_ptr), static_cast<unsigned char*>(a.o_ptr), K, H,
                        (int64_t)a.stride_token * 2);
     }
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+int launch_moe_smoothquant(const mi355_moe_smoothquant_args& a, int32_t q_dtype, hipStream_t stream)
+{
+    if(q_dtype != MI355_MOE_FP8 && q_dtype != MI355_MOE_INT8)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_smoothquant: q_dtype must be fp8 or int8");
+    if(a.tokens < 0 || a.hidden_size <= 0 || a.experts <= 0 || a.topk <= 0 || a.topk > 65535 || a.x_stride < a.hidden_size ||
+       a.y_stride < a.hidden_size)
+        return fail(MI355_MOE_E_INVALID, "moe_smoothquant: bad sizes (tokens=%d hidden=%d experts=%d topk=%d strides=%d,%d)",
+                    a.tokens, a.hidden_size, a.experts, a.topk, a.x_stride, a.y_stride);
+    if(a.tokens == 0)
+        return MI355_MOE_OK;
+    if(!a.p_x || !a.p_smscale || !a.p_topk_ids || !a.p_yscale || !a.p_qy)
+        return fail(MI355_MOE_E_INVALID, "moe_smoothquant: null pointer");
+    KernelTimer timer(MI355_MOE_K_QUANT, stream);
+    const dim3 grid((unsigned)a.tokens, (unsigned)a.topk);
+    if(q_dtype == MI355_MOE_FP8)
+        hipLaunchKernelGGL(moe_smoothquant_kernel<true>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
+                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
+                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
+                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
+    else
+        hipLaunchKernelGGL(moe_smoothquant_kernel<false>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
+                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
+                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
+                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }

@@ -203,6 +203,22 @@ def rowwise_quant(x, q_dtype: str, stream=None):
     return q, scale
 
 
+def moe_smoothquant(x, smscale, topk_ids, q_dtype: str = "int8", stream=None):
+    """CK's moe_smoothquant(traits, args, stream): x [tokens, hidden] bf16, smscale [experts, hidden] fp32,
+    topk_ids [tokens, topk] int32 -> (qy [topk, tokens, hidden] int8 / e4m3, yscale [topk, tokens] fp32)."""
+    import torch
+
+    tokens, hidden = x.shape
+    experts, topk = smscale.shape[0], topk_ids.shape[1]
+    st = {"fp8": torch.float8_e4m3fn, "int8": torch.int8}[q_dtype]
+    qy = torch.empty((topk, tokens, hidden), dtype=st, device=x.device)
+    ys = torch.empty((topk, tokens), dtype=torch.float32, device=x.device)
+    a = _lib.SmoothquantArgs(_ptr(x), _ptr(smscale), _ptr(topk_ids), _ptr(ys), _ptr(qy), tokens, hidden, experts, topk,
+                             x.stride(0) if tokens else hidden, hidden)
+    _check(_lib.load().mi355_moe_smoothquant(C.byref(a), _lib.DTYPES[q_dtype], _stream(stream)), "moe_smoothquant")
+    return qy, ys
+
+
 def topk_softmax(logits, topk: int, activation: str = "softmax", renormalize: bool = False, stream=None):
     """Router front-end (CK's topk_softmax(trait, kargs, stream)): softmax or sigmoid over the experts of
     each row of `logits` [rows, experts] (fp32 or bf16), then the top-k weights (fp32, descending) and
