@@ -238,6 +238,15 @@ typedef struct mi355_moe_smoothquant_args
 
 int mi355_moe_smoothquant(const mi355_moe_smoothquant_args* args, int32_t q_dtype, void* stream);
 
+/* Load-time layout tool for checkpoints that were pre-shuffled for ck_tile's device kernel
+ * (FusedMoeGemmWeightPermuteEnum::b_nr_kr_kw_nw_kv, ops/fused_moe/pipeline/fused_moegemm_traits.hpp:10-17):
+ * the row-major weight [experts, n, k] viewed as [experts, n/nw, nw, k/(kw*kv), kw, kv] and permuted with
+ * (0, 1, 3, 4, 2, 5) (host/reference/reference_permute.hpp:20-57).  inverse = 0 produces that layout from
+ * row-major, inverse = 1 turns it back into the row-major layout this library's GEMMs take.  CK's example
+ * uses nw = 16, kw = 4 with kv = 8 for 16-bit and kv = 16 for 8-bit weights.  src and dst must not overlap. */
+int mi355_moe_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
+                              int32_t nw, int32_t kw, int32_t kv, int32_t inverse, void* stream);
+
 /* ------------------------------------------------------------------------------ kernel timing
  * Counterpart of ck_tile::stream_config::time_kernel_ (host/stream_config.hpp:29-39,
  * host/kernel_launch.hpp:106-143): between _start and _stop every kernel the library launches is

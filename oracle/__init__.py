@@ -153,6 +153,30 @@ def ck_rowwise_quant(x: np.ndarray, scale: np.ndarray, dt: int):
     return q
 
 
+def permute_weights(w: np.ndarray, nw: int, kw: int, kv: int, inverse: bool = False) -> np.ndarray:
+    """ck_tile's b_nr_kr_kw_nw_kv pre-shuffle of [experts, n, k] weights (any dtype), or its inverse:
+    view [e, n/nw, nw, k/(kw*kv), kw, kv], permute (0, 1, 3, 4, 2, 5) (reference_permute.hpp:20-57)."""
+    e, n, k = w.shape
+    if inverse:
+        v = np.ascontiguousarray(w).reshape(e, n // nw, k // (kw * kv), kw, nw, kv)
+        return np.ascontiguousarray(v.transpose(0, 1, 4, 2, 3, 5)).reshape(e, n, k)
+    v = np.ascontiguousarray(w).reshape(e, n // nw, nw, k // (kw * kv), kw, kv)
+    return np.ascontiguousarray(v.transpose(0, 1, 3, 4, 2, 5)).reshape(e, n, k)
+
+
+def ck_permute_weights(w: np.ndarray, nw: int, kw: int, kv: int) -> np.ndarray:
+    """The same permutation computed by ck_tile::reference_permute on the byte view."""
+    r = ck_ref()
+    if r is None:
+        raise RuntimeError("oracle/_ref is not built")
+    e, n, k = w.shape
+    b = np.ascontiguousarray(w).view(np.uint8)
+    out = np.empty_like(b)
+    r.ck_ref_permute_b_nr_kr_kw_nw_kv(_p(b), C.c_int32(e), C.c_int32(n // nw), C.c_int32(nw), C.c_int32(k // (kw * kv)),
+                                      C.c_int32(kw), C.c_int32(kv * w.itemsize), _p(out))
+    return out.view(w.dtype).reshape(e, n, k)
+
+
 def smoothquant(x, smscale, topk_ids, dt):
     """MoE smooth-quant oracle: fp32 x [T,H], smscale [E,H], topk_ids [T,K] -> (qy [K,T,H], yscale [K,T])."""
     x, smscale, topk_ids = _c(x, np.float32), _c(smscale, np.float32), _c(topk_ids, np.int32)

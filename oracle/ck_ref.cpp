@@ -20,6 +20,7 @@
 #include "ck_tile/host/reference/reference_softmax.hpp"
 #include "ck_tile/host/reference/reference_topk.hpp"
 #include "ck_tile/host/reference/reference_rowwise_quantization2d.hpp"
+#include "ck_tile/host/reference/reference_permute.hpp"
 
 using ck_tile::HostTensor;
 using ck_tile::index_t;
@@ -161,6 +162,18 @@ ck_ref_rowwise_quant(const float* x, const float* scale, int32_t M, int32_t N, i
         ck_tile::reference_rowwise_quantization2d<float, float, ck_tile::int8_t>(x_h, s_h, q_h);
         std::memcpy(q, q_h.data(), (std::size_t)M * N);
     }
+    return 0;
+}
+
+// reference_permute with (0, 1, 3, 4, 2, 5) on the byte view [e, nr, nw, kr, kw, kv_bytes]
+__attribute__((visibility("default"))) int
+ck_ref_permute_b_nr_kr_kw_nw_kv(const uint8_t* x, int32_t e, int32_t nr, int32_t nw, int32_t kr, int32_t kw,
+                                int32_t kv_bytes, uint8_t* y)
+{
+    auto x_h = make_tensor<uint8_t>({(std::size_t)e, (std::size_t)nr, (std::size_t)nw, (std::size_t)kr, (std::size_t)kw,
+                                     (std::size_t)kv_bytes}, x);
+    auto y_h = ck_tile::reference_permute(x_h, {0, 1, 3, 4, 2, 5});
+    std::memcpy(y, y_h.data(), (std::size_t)e * nr * nw * kr * kw * kv_bytes);
     return 0;
 }
 

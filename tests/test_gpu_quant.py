@@ -51,3 +51,23 @@ def test_moe_smoothquant(tokens, hidden, experts, topk, kind):
     rq, rs = oracle.smoothquant(x.float().cpu().numpy(), sm.cpu().numpy(), ids, dt)
     assert np.array_equal(ys.cpu().numpy(), rs)
     assert np.array_equal(_raw(qy), rq)
+
+
+@pytest.mark.parametrize("shape,dtype,nw,kw,kv", [((4, 256, 512), "bf16", 16, 4, 8), ((3, 64, 256), "int8", 16, 4, 16),
+                                                   ((2, 64, 64), "bf16", 32, 2, 8), ((8, 4096, 1024), "fp8", 16, 4, 16)])
+def test_permute_weights(shape, dtype, nw, kw, kv):
+    """ck_tile's pre-shuffled weight layout and back: exact data movement."""
+    import torch
+    import therock_amd as ta
+
+    rng = np.random.default_rng(shape[1])
+    npdt = np.uint16 if dtype == "bf16" else np.uint8
+    w_np = rng.integers(0, 255, size=shape).astype(npdt)
+    tdt = {"bf16": torch.bfloat16, "int8": torch.int8, "fp8": torch.float8_e4m3fn}[dtype]
+    w = torch.from_numpy(w_np.view(np.int16) if dtype == "bf16" else w_np.view(np.int8)).cuda().view(tdt)
+    p = ta.permute_weights(w, nw, kw, kv)
+    back = ta.permute_weights(p, nw, kw, kv, inverse=True)
+    torch.cuda.synchronize()
+    as_np = lambda t: t.view(torch.int16 if dtype == "bf16" else torch.int8).cpu().numpy().view(npdt)
+    assert np.array_equal(as_np(p), oracle.permute_weights(w_np, nw, kw, kv))
+    assert np.array_equal(as_np(back), w_np)

@@ -139,3 +139,23 @@ def test_conversions_match_ck_tile():
         assert r.ck_ref_f32_to_fp8(v) == l.moe_oracle_f32_to_e4m3(v)
         assert r.ck_ref_f32_to_bf16(v) == l.moe_oracle_f32_to_bf16(v)
         assert r.ck_ref_silu(v) == l.moe_oracle_silu(v)
+
+
+@pytest.mark.parametrize("dtype,nw,kw,kv", [(np.uint16, 16, 4, 8), (np.uint8, 16, 4, 16), (np.uint16, 32, 2, 8), (np.int8, 32, 2, 16)])
+def test_weight_permutation(dtype, nw, kw, kv):
+    """b_nr_kr_kw_nw_kv: an index formula on a tiny case, the inverse, and ck_tile::reference_permute."""
+    rng = np.random.default_rng(nw + kv)
+    e, n, k = 3, 2 * nw, 3 * kw * kv
+    w = rng.integers(0, 200, size=(e, n, k)).astype(dtype)
+    p = oracle.permute_weights(w, nw, kw, kv)
+    flat = p.reshape(e, -1)
+    for _ in range(200):  # element (n_, k_) of expert x lands at ((nr*KR + kr)*kw + kw_)*nw*kv + nw_*kv + kv_
+        x, n_, k_ = int(rng.integers(e)), int(rng.integers(n)), int(rng.integers(k))
+        nr, nw_ = divmod(n_, nw)
+        kr, rem = divmod(k_, kw * kv)
+        kw_, kv_ = divmod(rem, kv)
+        pos = (((nr * (k // (kw * kv)) + kr) * kw + kw_) * nw + nw_) * kv + kv_
+        assert flat[x, pos] == w[x, n_, k_]
+    assert np.array_equal(oracle.permute_weights(p, nw, kw, kv, inverse=True), w)
+    if oracle.ck_ref() is not None:
+        assert np.array_equal(p, oracle.ck_permute_weights(w, nw, kw, kv))

@@ -4,4 +4,5 @@ libmi355_moe.so (hand-written HIP for gfx950, C ABI in include/mi355_moe.h); thi
 host-side mirror of the CK example API plus the synthetic-input harness."""
 from .moe import (MoeBuffers, fused_moe, fused_moe_args, fused_moe_get_workspace_size, fused_moe_tile_rows, fused_moe_traits,  # noqa: F401
                   fused_moegemm, make_args, moe_max_num_tokens_padded, moe_sorting, moe_sorting_args,
-                  moe_smoothquant, moe_sorting_get_workspace_size, moe_sorting_trait, rowwise_quant, topk_softmax)
+                  moe_smoothquant, moe_sorting_get_workspace_size, moe_sorting_trait, permute_weights, rowwise_quant,
+                  topk_softmax)

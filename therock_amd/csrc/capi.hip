@@ -262,6 +262,13 @@ mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args
 }
 
 __attribute__((visibility("default"))) int
+mi355_moe_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
+                          int32_t nw, int32_t kw, int32_t kv, int32_t inverse, void* stream)
+{
+    return launch_permute_weights(src, dst, experts, n, k, elem_bytes, nw, kw, kv, inverse, static_cast<hipStream_t>(stream));
+}
+
+__attribute__((visibility("default"))) int
 mi355_moe_smoothquant(const mi355_moe_smoothquant_args* args, int32_t q_dtype, void* stream)
 {
     if(args == nullptr)

@@ -715,6 +715,61 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     return MI355_MOE_OK;
 }
 
+// ck_tile's pre-shuffled weight layout b_nr_kr_kw_nw_kv: the row-major [e, n, k] tensor viewed as
+// [e, nr, nw, kr, kw, kv] and permuted to [e, nr, kr, kw, nw, kv].  One thread moves one kv granule.
+template <typename G>
+__global__ __launch_bounds__(256) void permute_weights_kernel(const G* __restrict__ src, G* __restrict__ dst,
+                                                               int64_t granules, int n, int kgran, int nw, int kw,
+                                                               int inverse)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if(i >= granules)
+        return;
+    // i enumerates the permuted layout: (e, nr, kr, kw, nw)
+    const int kr_n = kgran / kw;
+    int64_t r      = i;
+    const int a_nw = (int)(r % nw);
+    r /= nw;
+    const int a_kw = (int)(r % kw);
+    r /= kw;
+    const int a_kr = (int)(r % kr_n);
+    r /= kr_n;
+    const int a_nr = (int)(r % (n / nw));
+    const int64_t e = r / (n / nw);
+    const int64_t row_major = (e * n + (int64_t)a_nr * nw + a_nw) * kgran + (int64_t)a_kr * kw + a_kw;
+    if(inverse)
+        dst[row_major] = src[i];
+    else
+        dst[i] = src[row_major];
+}
+
+int launch_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
+                           int32_t nw, int32_t kw, int32_t kv, int32_t inverse, hipStream_t stream)
+{
+    if(!src || !dst || src == dst || experts <= 0 || n <= 0 || k <= 0 || nw <= 0 || kw <= 0 || kv <= 0 ||
+       (elem_bytes != 1 && elem_bytes != 2))
+        return fail(MI355_MOE_E_INVALID, "permute_weights: bad arguments");
+    const int gran = kv * elem_bytes;
+    if(n % nw != 0 || k % (kw * kv) != 0 || (gran != 4 && gran != 8 && gran != 16))
+        return fail(MI355_MOE_E_UNSUPPORTED,
+                    "permute_weights: n %% nw, k %% (kw*kv) must be 0 and kv*elem_bytes 4, 8 or 16 (n=%d k=%d nw=%d kw=%d kv=%d)",
+                    n, k, nw, kw, kv);
+    const int kgran        = k / kv;
+    const int64_t granules = (int64_t)experts * n * kgran;
+    const unsigned grid    = (unsigned)ceil_div<int64_t>(granules, 256);
+    if(gran == 16)
+        hipLaunchKernelGGL(permute_weights_kernel<uint4>, dim3(grid), dim3(256), 0, stream, static_cast<const uint4*>(src),
+                           static_cast<uint4*>(dst), granules, n, kgran, nw, kw, inverse);
+    else if(gran == 8)
+        hipLaunchKernelGGL(permute_weights_kernel<uint2>, dim3(grid), dim3(256), 0, stream, static_cast<const uint2*>(src),
+                           static_cast<uint2*>(dst), granules, n, kgran, nw, kw, inverse);
+    else
+        hipLaunchKernelGGL(permute_weights_kernel<uint32_t>, dim3(grid), dim3(256), 0, stream,
+                           static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst), granules, n, kgran, nw, kw, inverse);
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
 int launch_moe_smoothquant(const mi355_moe_smoothquant_args& a, int32_t q_dtype, hipStream_t stream)
 {
     if(q_dtype != MI355_MOE_FP8 && q_dtype != MI355_MOE_INT8)

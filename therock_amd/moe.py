@@ -203,6 +203,20 @@ def rowwise_quant(x, q_dtype: str, stream=None):
     return q, scale
 
 
+def permute_weights(w, nw: int = 16, kw: int = 4, kv: int | None = None, inverse: bool = False, stream=None):
+    """[experts, n, k] weights to (inverse=False) or from (inverse=True) ck_tile's pre-shuffled layout
+    b_nr_kr_kw_nw_kv.  kv defaults to 16 bytes worth of elements (CK's example: 8 for bf16, 16 for 8-bit)."""
+    import torch
+
+    experts, n, k = w.shape
+    eb = w.element_size()
+    kv = kv if kv is not None else 16 // eb
+    out = torch.empty_like(w)
+    _check(_lib.load().mi355_moe_permute_weights(_ptr(w), _ptr(out), experts, n, k, eb, nw, kw, kv, int(bool(inverse)),
+                                                 _stream(stream)), "permute_weights")
+    return out
+
+
 def moe_smoothquant(x, smscale, topk_ids, q_dtype: str = "int8", stream=None):
     """CK's moe_smoothquant(traits, args, stream): x [tokens, hidden] bf16, smscale [experts, hidden] fp32,
     topk_ids [tokens, topk] int32 -> (qy [topk, tokens, hidden] int8 / e4m3, yscale [topk, tokens] fp32)."""
