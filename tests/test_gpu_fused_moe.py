@@ -110,6 +110,17 @@ def test_decode_shapes_int8():
         check(mi.CONFIGS["cfg4_decode_int8_t64"].scaled(tokens=T, hidden=1024, inter=512))
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
+def test_decode_kernel_ragged(dtype):
+    # <= 32 rows per expert selects the decode kernel (64 weight rows, 512-byte K runs split over the four
+    # waves): K depths that are not a multiple of 512 bytes, column tails, a single token, empty experts
+    inter = 384 if dtype == "fp8" else 288
+    check(mi.MoeConfig("d", 24, 1056, inter, 16, 4, dtype, "softmax_renorm"), seed=1)
+    # (a single fp8 token is too small a sample for a stable rel-L2 of the e4m3 rounding of Y: four there)
+    check(mi.MoeConfig("d", 4 if dtype == "fp8" else 1, 480, 128, 8, 2, dtype, "softmax"), seed=2)
+    check(mi.MoeConfig("d", 40, 2080, 640, 64, 8, dtype, "sigmoid_renorm", unit=16), seed=3)
+
+
 def test_traits_without_kernel_return_minus_one():
     import torch
     import therock_amd as ta
