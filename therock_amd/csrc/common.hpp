@@ -87,7 +87,6 @@ struct GemmPlan
     int rows_per_tile; // sorted rows per GEMM tile (multiple of 32)
     int max_tiles;     // capacity of tile_map
     int* inv;          // [tokens * topk]: sorted position of every (token, slot), -1 when dropped
-    int* zero_page;    // 64 ints to clear
 };
 
 // ---- sorting launcher shared by the stand-alone and the fused entry points

@@ -273,15 +273,12 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
                                                                const int* __restrict__ post_pad_ptr, int unit,
                                                                int experts, int rows_per_tile, int max_units,
                                                                int max_tiles, int* __restrict__ tile_map,
-                                                               int* __restrict__ inv, int n_inv,
-                                                               int* __restrict__ zero_page)
+                                                               int* __restrict__ inv, int n_inv)
 {
     for(int i = blockIdx.x * kPrepBlock + threadIdx.x; i < n_inv; i += gridDim.x * kPrepBlock)
         inv[i] = -1;
     if(blockIdx.x != 0)
         return;
-    if(threadIdx.x < 64)
-        zero_page[threadIdx.x] = 0;
     __shared__ int s_wave[kPrepWaves + 1];
     const int post_pad = post_pad_ptr[0];
     int nunits         = post_pad / unit;
@@ -553,7 +550,6 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
     w.y_off          = bump((size_t)w.max_pad * inter * y_b);
     w.ys_kb_stride   = round_up<int64_t>(w.max_pad, 256) + 512;
     w.ys_off         = bump(t.prec_i == MI355_MOE_FP8 ? (size_t)w.ys_kb_stride * (inter / 32) : 0);
-    w.zero_off       = bump(256);
     w.p_off          = bump((size_t)w.max_pad * hidden * 2);
     return w;
 }
@@ -568,7 +564,6 @@ GemmPlan make_gemm_plan(const mi355_fused_moe_traits& t, void* ws_ptr, int32_t t
     g.rows_per_tile = pick_mblk(t, tokens, topk, experts, hidden, inter) * 32;
     g.max_tiles     = ws.max_tiles;
     g.inv           = reinterpret_cast<int*>(wsb + ws.inv_off);
-    g.zero_page     = reinterpret_cast<int*>(wsb + ws.zero_off);
     return g;
 }
 
@@ -622,7 +617,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
         hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
                            static_cast<const int*>(a.sorted_expert_ids_ptr),
                            static_cast<const int*>(a.num_sorted_tiles_ptr), t.block_m, E, mblk * 32, max_units,
-                           ws.max_tiles, tile_map, inv, n_inv, reinterpret_cast<int*>(wsb + ws.zero_off));
+                           ws.max_tiles, tile_map, inv, n_inv);
         hipLaunchKernelGGL(moe_inv_kernel, dim3(std::min<int>(ceil_div<int64_t>(ws.max_pad, 256), 1024)), dim3(256), 0,
                            stream, static_cast<const int*>(a.sorted_token_ids_ptr),
                            static_cast<const int*>(a.num_sorted_tiles_ptr), (int)ws.max_pad, T, K, inv);
@@ -635,7 +630,6 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.tokens     = T;
     p.y_scale    = wsb + ws.ys_off;
     p.ys_kb_stride = ws.ys_kb_stride;
-    p.zero_page    = wsb + ws.zero_off;
 
     // ---- gemm0: gate+up, SiLU*up
     const int y_b     = t.prec_i == MI355_MOE_FP8 ? 1 : 2;

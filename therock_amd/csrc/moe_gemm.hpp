@@ -13,7 +13,6 @@ struct WorkspaceLayout
     size_t inv_off;    // int32 [tokens * topk]: sorted position of the (token, slot) entry, -1 when dropped
     size_t y_off;      // intermediate activations Y [max_pad, inter] (bf16 or e4m3)
     size_t ys_off;     // e8m0 block scales of Y [inter / 32][ys_kb_stride] (fp8 path only)
-    size_t zero_off;   // 256 zero bytes
     int64_t ys_kb_stride;
     size_t p_off;      // partial outputs per sorted row [max_pad, hidden] bf16
     size_t total;
@@ -30,7 +29,7 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
 int gemm_tile_rows(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk, int32_t hidden,
                    int32_t inter);
 
-// prep_done: the tile list, inverse map and zero page were already written by the sort (GemmPlan)
+// prep_done: the tile list and the inverse map were already written by the sort (GemmPlan)
 int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a,
                          hipStream_t stream, bool prep_done = false);
 

@@ -7,21 +7,24 @@
 //     workload (about 270 rows) is one tile and its weights are fetched once.
 //   * Both operands go global -> LDS with global_load_lds_dwordx4 (no staging registers).  The K loop
 //     advances in 64-byte steps.  Tokens (re-read from L2 by every column tile) arrive one 64-byte
-//     step at a time through a ring of three stages.  Weights are streamed from HBM exactly once,
-//     and for them the request shape decides the rate: they arrive as full 128-byte lines, half
-//     of the tile's rows per unit (unit u = rows (u&1)*128.., K bytes [128*(u>>1), +128)), through a
-//     ring of six units issued four steps ahead.  Measured on the fp8 workload, the weight stream
-//     alone runs at 7.3 TB/s in this shape against 4.8 TB/s as 64-byte pieces.
+//     step at a time through a ring of three stages.  Weights are streamed from HBM exactly once, as
+//     full 128-byte lines, half of the tile's rows per unit (unit u = rows (u&1)*128.., K bytes
+//     [128*(u>>1), +128)), through a ring of six units issued four steps ahead.
 //   * The loads are issued from inline assembly so that their completion is tracked by hand:
 //     s_waitcnt vmcnt(n) with n = the DMA instructions this wave issued after the data about to be
-//     consumed (token step issued before weight unit in every iteration, so that waiting for the
-//     tokens does not wait for the younger weight units), then one workgroup barrier per step,
-//     which also frees the buffers the next issues write into.
+//     consumed, then one workgroup barrier per step, which also frees the buffers the next issues
+//     write into.  Loads of one wave return in order, so the two streams are issued by different
+//     waves (0..3 weights, 4..7 tokens): mixed in one wave, the L2-hit token loads would queue
+//     behind the HBM-miss weight loads.
+//   * What bounds the kernel is the rate at which a compute unit's LDS can be filled: with both
+//     streams running it is about 19 bytes per clock (each stream alone is much faster), and a step
+//     of this tile needs 36.9 KB for 1400 clocks of MFMA work.
 //   * LDS rows are swizzled: 64-byte token rows keep chunk c of row r at c ^ ((r >> 2) & 3), 128-byte
 //     weight rows at c ^ ((r >> 1) & 7); both the linear DMA writes and the ds_read_b128 operand
-//     fetches are then conflict-free on the 64-bank LDS.  Rows that must read as zero (padding ids,
-//     rows past the tile) are fetched from a zero page, so the number of DMA instructions per wave
-//     and step, and with it every wait count, is a compile-time constant.
+//     fetches are then conflict-free on the 64-bank LDS.  Token rows that do not exist (padding ids,
+//     rows past the tile) fetch some real row instead - their MFMA columns are never stored - so
+//     the number of DMA instructions per wave and step, and with it every wait count, is a
+//     compile-time constant.
 //   * The K loop is specialised on the number of token blocks a wave owns, so the MFMA region is
 //     straight-line code.
 #include "moe_gemm_device.hpp"

@@ -41,7 +41,6 @@ struct GemmParams
     int64_t w_expert_bytes;
     int64_t out_row_bytes;
     int64_t ys_kb_stride;    // bytes between consecutive 32-column blocks of y_scale ([inter/32][rows])
-    const unsigned char* zero_page; // >= 256 zero bytes (rows that must read as zero)
     int k_bytes_x;           // bytes of K in a row of x
     int k_bytes_w;           // bytes of K in a row of w
     int n_out;               // gemm0: inter; gemm1: hidden

@@ -236,8 +236,6 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
         }
         if(tid == 0)
             plan.tile_map[0] = min(n_tiles, plan.max_tiles);
-        if(tid < 64)
-            plan.zero_page[tid] = 0;
     }
 }
 
