@@ -179,6 +179,44 @@ inline float topk_softmax(topk_softmax_trait t, topk_softmax_kargs a, stream_con
     });
 }
 
+// ----------------------------------------------------------------------------------- moe_flatmm
+// ck_tile::MoeFlatmmHostArgs (ops/flatmm/kernel/moe_flatmm_kernel.hpp:17-127) and MoeFlatmmKind (:130-135)
+enum class MoeFlatmmKind
+{
+    kFFN_gemm1_gate_only = MI355_MOE_GEMM1_GATE_ONLY,
+    kFFN_gemm1_gate_up   = MI355_MOE_GEMM1_GATE_UP,
+    kFFN_gemm2           = MI355_MOE_GEMM2,
+};
+
+struct moe_flatmm_args : public mi355_moe_flatmm_args
+{
+};
+
+// ws_ptr may be left null: a cached per-device workspace is used.  Returns -1 when no kernel matches.
+inline float moe_flatmm(MoeFlatmmKind kind, moe_flatmm_args a, stream_config s = {})
+{
+    const int k = static_cast<int>(kind);
+    if(a.ws_ptr == nullptr)
+    {
+        a.ws_bytes = mi355_moe_flatmm_workspace_size(k, &a);
+        if(a.ws_bytes == 0)
+            return -1.f;
+        a.ws_ptr = detail::cached_workspace(a.ws_bytes);
+    }
+    bool unsupported = false;
+    const float ms   = detail::run_timed(s, [&] {
+        const int rc = mi355_moe_flatmm(k, &a, s.stream_id_);
+        if(rc == MI355_MOE_E_UNSUPPORTED)
+        {
+            unsupported = true;
+            return 0;
+        }
+        detail::throw_on_error(rc, "moe_flatmm");
+        return rc;
+    });
+    return unsupported ? -1.f : ms;
+}
+
 // ------------------------------------------------------------------------------ moe_smoothquant
 // moe_smoothquant_traits / moe_smoothquant_args of CK's example/ck_tile/14_moe_smoothquant
 struct moe_smoothquant_traits

@@ -247,6 +247,53 @@ int mi355_moe_smoothquant(const mi355_moe_smoothquant_args* args, int32_t q_dtyp
 int mi355_moe_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
                               int32_t nw, int32_t kw, int32_t kv, int32_t inverse, void* stream);
 
+/* ------------------------------------------------------------------- stand-alone grouped GEMMs
+ * The two GEMMs as separate launches, for callers that keep sort / gemm1 / gemm2 apart.  Replaces
+ * ck_tile::MoeFlatmmKernel behind MoeFlatmmHostArgs (ops/flatmm/kernel/moe_flatmm_kernel.hpp:17-127, kinds
+ * :130-135); semantics as in host/reference/reference_moe_gemm.hpp:18-241:
+ *   gate+up: C[token * TopK + slot, n] = silu(A[token] . B[e, n]) * (A[token] . B[e, N/2 + n]),  n < N/2
+ *   down   : C[token, n] += sum over the token's slots of w * (A[token * TopK + slot] . B[e, n])
+ * with the per-row scale scale_m and the per-channel scale scale_n folded in.  Unlike ck_tile's atomic
+ * bf16 epilogue the down GEMM sums a token's slots in fp32, in slot order, and rounds once. */
+enum mi355_moe_flatmm_kind
+{
+    MI355_MOE_GEMM1_GATE_ONLY = 0, /* not implemented */
+    MI355_MOE_GEMM1_GATE_UP   = 1,
+    MI355_MOE_GEMM2           = 2
+};
+
+typedef struct mi355_moe_flatmm_args
+{
+    const void* p_sorted_token_ids;      /* as written by mi355_moe_sorting: token | slot << 24 */
+    const void* p_sorted_expert_weights; /* fp32 per sorted row (down GEMM) */
+    const void* p_sorted_expert_ids;
+    const void* p_max_token_id;          /* [1] int32: rows after padding (p_total_tokens_post_pad) */
+    const void* a_ptr;    /* gate+up: [NumTokens, stride_A]; down: [NumTokens * TopK, stride_A] */
+    const void* b_ptr;    /* [NumExperts, N, K], K contiguous (stride_B = K) */
+    void* c_ptr;          /* bf16; gate+up: [NumTokens * TopK, stride_C] (N/2 columns); down: [NumTokens, stride_C] */
+    const void* scale_m;  /* fp32 per row of A, or NULL (ScaleM) */
+    const void* scale_n;  /* fp32 [NumExperts, N], or NULL (ScaleN) */
+    const void* exp_bias; /* must be NULL */
+    void* ws_ptr;         /* mi355_moe_flatmm_workspace_size() bytes, 256-byte aligned */
+    size_t ws_bytes;
+    int32_t NumTokens;
+    int32_t NumExperts;
+    int32_t TopK;
+    int32_t k_batch;      /* 0 or 1 */
+    int32_t M;            /* length of the sorted id list (informational) */
+    int32_t N;
+    int32_t K;
+    int32_t stride_A;
+    int32_t stride_B;
+    int32_t stride_C;
+    int32_t prec_a;       /* mi355_moe_dtype of A: BF16, or INT8 for the gate+up GEMM with int8 weights */
+    int32_t prec_b;       /* mi355_moe_dtype of B: BF16 | INT8 */
+    int32_t block_m;      /* unit_size the sort was run with */
+} mi355_moe_flatmm_args;
+
+size_t mi355_moe_flatmm_workspace_size(int32_t kind, const mi355_moe_flatmm_args* args);
+int mi355_moe_flatmm(int32_t kind, const mi355_moe_flatmm_args* args, void* stream);
+
 /* ------------------------------------------------------------------------------ kernel timing
  * Counterpart of ck_tile::stream_config::time_kernel_ (host/stream_config.hpp:29-39,
  * host/kernel_launch.hpp:106-143): between _start and _stop every kernel the library launches is

@@ -236,6 +236,26 @@ def ck_moe_sorting(topk_ids, weights, experts, unit, local_expert_mask=None, ski
     return ids, w, eid, int(pp)
 
 
+# ------------------------------------------------------------------- unfused grouped GEMMs
+def moe_gemm(kind, sorted_ids, sorted_eid, sorted_w, post_pad, block_m, a, b, c, num_tokens, topk,
+             scale_a=None, scale_b=None):
+    """Oracle of ck_tile's unfused MoE GEMMs (kind 1 = gate+up with SiLU*up, 2 = down with weights, added to
+    c).  a, b fp32; c bf16 bits [rows, >= N or N/2], updated in place and returned."""
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    c = np.ascontiguousarray(c, dtype=np.uint16)
+    E, N, K = b.shape
+    ids, eid = _c(sorted_ids, np.int32), _c(sorted_eid, np.int32)
+    w = _c(sorted_w, np.float32)
+    f = lib().moe_oracle_moe_gemm
+    f.restype = C.c_int
+    rc = f(C.c_int(kind), _p(ids), _p(eid), _p(w), C.c_int32(int(post_pad)), C.c_int32(block_m), _p(a), _p(b), _p(c),
+           C.c_int32(num_tokens), C.c_int32(topk), C.c_int32(N), C.c_int32(K), C.c_int32(a.shape[1]),
+           C.c_int32(c.shape[1]), _p(_c(scale_a, np.float32)), _p(_c(scale_b, np.float32)))
+    if rc != 0:
+        raise ValueError(f"moe_oracle_moe_gemm failed ({rc})")
+    return c
+
+
 # ----------------------------------------------------------------------------- router
 def topk_softmax(logits, topk, sigmoid=False, renorm=False):
     """Oracle router: softmax (or sigmoid) over the last axis of fp32 `logits` [rows, experts], then the

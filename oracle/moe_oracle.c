@@ -16,6 +16,7 @@
  *   e4m3 (OCP) encode/decode  <- core/numeric/float8.hpp:600-660 (saturating RNE, +-448)
  *   row-wise quantisation     <- host/reference/reference_rowwise_quantization2d.hpp:12-31
  *   scale placement           <- host/reference/reference_moe_gemm.hpp:94-113,202-203
+ *   moe_oracle_moe_gemm       <- host/reference/reference_moe_gemm.hpp:18-241 (ck_tile's unfused grouped GEMMs)
  *   moe_oracle_topk_softmax   <- host/reference/reference_softmax.hpp:12-78 + host/reference/reference_topk.hpp:30-103
  *                                (sigmoid variant: ops/topk_softmax/pipeline/topk_softmax_warp_per_row_pipeline.hpp:88-92)
  *
@@ -30,6 +31,9 @@
  *   fused moe   - ck_tile's reference_fused_moe in oracle/_ref on the same inputs; an
  *                 independent dense (sorting-free) float64 formulation in numpy.
  *   bf16 / e4m3 - exhaustive comparison with torch's bfloat16 / float8_e4m3fn casts.
+ *   moe gemm    - ck_tile's reference for these is a device kernel and cannot run on the CPU: pinned by a
+ *                 dense float64 formulation that never sorts, by the composition gate+up -> down against
+ *                 moe_oracle_fused_moe (itself bit-exact with ck_tile), and by a triple loop on tiny shapes.
  *   topk softmax- ck_tile's reference_softmax + reference_topk in oracle/_ref; closed forms (equal
  *                 logits, shift invariance, weights of all experts sum to one), scipy's softmax and
  *                 numpy's argsort on random rows.
@@ -462,6 +466,77 @@ ORACLE_API int moe_oracle_fused_moe(const void* a, int a_dt, const float* a_scal
     if(!out_topk)
         free(part);
     return rc;
+}
+
+/* ---------------------------------------------------------------------- unfused grouped GEMMs
+ * reference_moe_gemm.hpp:41-241 with row-major A and C, B as [experts, N, K], one scale per row of A
+ * (scale_a, may be NULL) and per output channel (scale_b [experts, N], may be NULL), no expert bias.
+ *   kind 1 (gate+up): row r of the sorted list with token t, slot s: A row t, C row t*topk+s,
+ *       C[., n] = bf16( silu(acc_gate) * acc_up ), gate = B rows [0, N/2), up = B rows [N/2, N)
+ *   kind 2 (down)   : A row t*topk+s, C row t; ck_tile adds bf16(acc * w[r]) to C with packed bf16 atomics
+ *       (:214-238).  Here a token's slots are summed in fp32 in slot order on top of the bf16 value C holds
+ *       and rounded once: the same quantity without the order-dependent bf16 rounding of every partial sum.
+ * A and B are fp32 (the caller up-converts), C is bf16 bits. */
+ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const int32_t* sorted_eid, const float* sorted_w,
+                                   int32_t max_token_id, int32_t tokens_per_block, const float* A, const float* B,
+                                   uint16_t* C, int32_t num_tokens, int32_t topk, int32_t N, int32_t K, int32_t stride_a,
+                                   int32_t stride_c, const float* scale_a, const float* scale_b)
+{
+    if(kind != 1 && kind != 2)
+        return -1;
+    const int32_t pn = kind == 1 ? N / 2 : N;
+    float* acc2      = NULL; /* kind 2: fp32 sums [tokens, N], started from C */
+    if(kind == 2)
+    {
+        acc2 = (float*)malloc(sizeof(float) * (size_t)num_tokens * N);
+        if(!acc2)
+            return -2;
+        for(int64_t t = 0; t < num_tokens; t++)
+            for(int64_t n = 0; n < N; n++)
+                acc2[t * N + n] = moe_oracle_bf16_to_f32(C[t * stride_c + n]);
+    }
+    /* slot order inside a token = the order of the reference's reduction: walk slots, then rows */
+    for(int32_t s = 0; s < (kind == 2 ? topk : 1); s++)
+        for(int64_t r = 0; r < max_token_id; r++)
+        {
+            const int32_t id  = sorted_ids[r];
+            const int32_t tok = id & 0xffffff, slot = (int32_t)((uint32_t)id >> 24);
+            if(tok >= num_tokens || (kind == 2 && slot != s))
+                continue;
+            const int64_t e      = sorted_eid[r / tokens_per_block];
+            const int64_t a_row  = kind == 2 ? (int64_t)tok * topk + slot : tok;
+            const int64_t c_row  = kind == 2 ? tok : (int64_t)tok * topk + slot;
+            const float* a       = A + a_row * stride_a;
+            const float sa       = scale_a ? scale_a[a_row] : 1.0f;
+#pragma omp parallel for schedule(static)
+            for(int32_t n = 0; n < pn; n++)
+            {
+                const float* b = B + (e * N + n) * K;
+                float acc      = 0.f;
+                for(int32_t k = 0; k < K; k++)
+                    acc += a[k] * b[k];
+                acc *= sa * (scale_b ? scale_b[e * N + n] : 1.0f);
+                if(kind == 1)
+                {
+                    const float* bu = B + (e * N + n + pn) * K;
+                    float up        = 0.f;
+                    for(int32_t k = 0; k < K; k++)
+                        up += a[k] * bu[k];
+                    up *= sa * (scale_b ? scale_b[e * N + n + pn] : 1.0f);
+                    C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(silu_f32(acc) * up);
+                }
+                else
+                    acc2[c_row * N + n] += acc * sorted_w[r];
+            }
+        }
+    if(kind == 2)
+    {
+        for(int64_t t = 0; t < num_tokens; t++)
+            for(int64_t n = 0; n < N; n++)
+                C[t * stride_c + n] = moe_oracle_f32_to_bf16(acc2[t * N + n]);
+        free(acc2);
+    }
+    return 0;
 }
 
 /* ------------------------------------------------------------------------------ router

@@ -1,0 +1,88 @@
+"""GPU parity of the stand-alone grouped GEMMs (mi355_moe_flatmm) against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(t):
+    import torch
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def _rel(a, b):
+    a, b = a.astype(np.float64), b.astype(np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+# (tokens, experts, topk, hidden, inter, unit): decode kernel, 32-row tiles, 128-row tiles, large-tile kernel
+SHAPES = [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (130, 6, 2, 1152, 256, 64), (1024, 4, 2, 512, 384, 32)]
+
+
+@pytest.mark.parametrize("T,E,K,H,I,unit", SHAPES)
+@pytest.mark.parametrize("kind", ["bf16", "int8"])
+def test_gate_up_then_down(T, E, K, H, I, unit, kind):
+    import torch
+    import therock_amd as ta
+    from tests.gpu_util import run_sorting
+
+    rng = np.random.default_rng(T + H)
+    tol = 1e-2 if kind == "bf16" else 3e-2
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
+    w = rng.random((T, K), dtype=np.float32)
+    s_ids, s_w, s_eid, total = run_sorting(ids, w, E, unit, fill=True)
+    pp = int(total[0])
+    ref_sort = oracle.moe_sorting(ids, w, E, unit)
+    assert pp == ref_sort[3]
+    dev = lambda a: torch.from_numpy(a).cuda()
+    bf = lambda a: torch.from_numpy(a).cuda().to(torch.bfloat16)
+    x32 = rng.standard_normal((T, H)).astype(np.float32)
+    g32 = (rng.standard_normal((E, 2 * I, H)) * 0.05).astype(np.float32)
+    d32 = (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32)
+    d_ids, d_w, d_eid, d_tot = dev(s_ids), dev(s_w), dev(s_eid), dev(total.astype(np.int32))
+    if kind == "bf16":
+        x, g, d = bf(x32), bf(g32), bf(d32)
+        xr, gr, dr = x.float().cpu().numpy(), g.float().cpu().numpy(), d.float().cpu().numpy()
+        sa = sg = sd = None
+        d_sa = d_sg = d_sd = None
+    else:
+        xq, sa = oracle.rowwise_quant(x32, oracle.DT_I8, nearest=True)
+        gq, sg = oracle.rowwise_quant(g32.reshape(E * 2 * I, H), oracle.DT_I8, nearest=True)
+        dq, sd = oracle.rowwise_quant(d32.reshape(E * H, I), oracle.DT_I8, nearest=True)
+        x, g, d = dev(xq), dev(gq.reshape(E, 2 * I, H)), dev(dq.reshape(E, H, I))
+        xr, gr, dr = xq.astype(np.float32), gq.reshape(E, 2 * I, H).astype(np.float32), dq.reshape(E, H, I).astype(np.float32)
+        sg, sd = sg.reshape(E, 2 * I), sd.reshape(E, H)
+        d_sa, d_sg, d_sd = dev(sa), dev(sg), dev(sd)
+
+    # gate+up: every (token, slot) row written exactly, nothing else touched
+    y = torch.full((T * K + 3, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert ta.moe_flatmm(ta.GEMM1_GATE_UP, x, g, y, d_ids, d_eid, d_tot, T, K, unit, scale_m=d_sa, scale_n=d_sg) == 0.0
+    torch.cuda.synchronize()
+    y_ref = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, xr, gr, np.zeros((T * K, I), np.uint16), T, K, sa, sg)
+    yg = y.float().cpu().numpy()
+    assert np.isnan(yg[T * K:]).all() and not np.isnan(yg[:T * K]).any()
+    assert _rel(yg[:T * K], oracle.to_f32(y_ref, oracle.DT_BF16)) <= tol
+
+    # down: added to what c holds; a takes the reference's bf16 Y so that the two GEMMs are checked apart
+    y_in = torch.from_numpy(y_ref.view(np.int16)).cuda().view(torch.bfloat16)
+    c0 = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
+    c = bf(c0)
+    c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, oracle.to_f32(y_ref, oracle.DT_BF16), dr, _bits(c).copy(), T, K,
+                            None, sd)
+    assert ta.moe_flatmm(ta.GEMM2, y_in, d, c, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w, scale_n=d_sd) == 0.0
+    torch.cuda.synchronize()
+    assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, oracle.DT_BF16)) <= tol
+
+
+def test_unsupported_and_errors():
+    import torch
+    import therock_amd as ta
+
+    z = lambda *s, dt=torch.bfloat16: torch.zeros(s, dtype=dt, device="cuda")
+    ids, eid, tot = z(64, dt=torch.int32), z(2, dt=torch.int32), z(2, dt=torch.int32)
+    # gate-only and fp8 have no stand-alone kernel: -1 like ck_tile's dispatcher
+    assert ta.moe_flatmm(0, z(4, 64), z(2, 128, 64), z(8, 64), ids, eid, tot, 4, 2, 32) == -1.0
+    with pytest.raises(RuntimeError):
+        ta.moe_flatmm(ta.GEMM2, z(8, 64), z(2, 64, 64), z(4, 64), ids, eid, tot, 4, 2, 32)  # no sorted weights

@@ -69,6 +69,18 @@ class TopkSoftmaxTraits(C.Structure):
     ]
 
 
+class FlatmmArgs(C.Structure):
+    _fields_ = [
+        ("p_sorted_token_ids", C.c_void_p), ("p_sorted_expert_weights", C.c_void_p), ("p_sorted_expert_ids", C.c_void_p),
+        ("p_max_token_id", C.c_void_p), ("a_ptr", C.c_void_p), ("b_ptr", C.c_void_p), ("c_ptr", C.c_void_p),
+        ("scale_m", C.c_void_p), ("scale_n", C.c_void_p), ("exp_bias", C.c_void_p), ("ws_ptr", C.c_void_p),
+        ("ws_bytes", C.c_size_t), ("NumTokens", C.c_int32), ("NumExperts", C.c_int32), ("TopK", C.c_int32),
+        ("k_batch", C.c_int32), ("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("stride_A", C.c_int32),
+        ("stride_B", C.c_int32), ("stride_C", C.c_int32), ("prec_a", C.c_int32), ("prec_b", C.c_int32),
+        ("block_m", C.c_int32),
+    ]
+
+
 class SmoothquantArgs(C.Structure):
     _fields_ = [
         ("p_x", C.c_void_p), ("p_smscale", C.c_void_p), ("p_topk_ids", C.c_void_p), ("p_yscale", C.c_void_p),
@@ -88,6 +100,8 @@ PROTOTYPES = {
     "mi355_fused_moe_tile_rows": (C.c_int32, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
     "mi355_fused_moegemm": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeGemmArgs), C.c_void_p]),
     "mi355_fused_moe": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.c_void_p]),
+    "mi355_moe_flatmm_workspace_size": (C.c_size_t, [C.c_int32, C.POINTER(FlatmmArgs)]),
+    "mi355_moe_flatmm": (C.c_int, [C.c_int32, C.POINTER(FlatmmArgs), C.c_void_p]),
     "mi355_moe_permute_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int32] * 8 + [C.c_void_p]),
     "mi355_moe_smoothquant": (C.c_int, [C.POINTER(SmoothquantArgs), C.c_int32, C.c_void_p]),
     "mi355_moe_rowwise_quant": (C.c_int, [C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_int32, C.c_void_p,

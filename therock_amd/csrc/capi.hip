@@ -261,6 +261,19 @@ mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args
     return launch_fused_moegemm(*traits, g, static_cast<hipStream_t>(stream), /*prep_done=*/true);
 }
 
+__attribute__((visibility("default"))) size_t
+mi355_moe_flatmm_workspace_size(int32_t kind, const mi355_moe_flatmm_args* args)
+{
+    return args != nullptr ? moe_flatmm_workspace_bytes(kind, *args) : 0;
+}
+
+__attribute__((visibility("default"))) int mi355_moe_flatmm(int32_t kind, const mi355_moe_flatmm_args* args, void* stream)
+{
+    if(args == nullptr)
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: args is null");
+    return launch_moe_flatmm(kind, *args, static_cast<hipStream_t>(stream));
+}
+
 __attribute__((visibility("default"))) int
 mi355_moe_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
                           int32_t nw, int32_t kw, int32_t kv, int32_t inverse, void* stream)

@@ -86,8 +86,15 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
         }
         else
         {
-            xvalid[j] = r < nrows;
-            xptr[j]   = p.x + (int64_t)(row0 + (xvalid[j] ? r : 0)) * p.x_row_bytes + xchunk * 16;
+            xvalid[j]   = r < nrows;
+            int64_t src = row0 + (xvalid[j] ? r : 0);
+            if(p.slot_rows > 0)
+            {
+                const int sid = p.sorted_ids[src];
+                xvalid[j]     = xvalid[j] && (sid & 0xffffff) < p.tokens;
+                src           = xvalid[j] ? slot_row(sid, p.slot_rows) : 0;
+            }
+            xptr[j] = p.x + src * p.x_row_bytes + xchunk * 16;
         }
     }
 
@@ -342,13 +349,24 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
                                                            const int* __restrict__ inv,
                                                            const float* __restrict__ sorted_w,
                                                            unsigned char* __restrict__ out, int topk, int hidden,
-                                                           int64_t out_row_bytes)
+                                                           int64_t out_row_bytes, int accumulate)
 {
     const int t  = blockIdx.x;
     const int h0 = (blockIdx.y * 256 + threadIdx.x) * 8;
     if(h0 >= hidden)
         return;
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if(accumulate) // stand-alone down GEMM: add to what the output holds, as ck_tile's atomic epilogue does
+    {
+        const uint4 v = *reinterpret_cast<const uint4*>(out + (int64_t)t * out_row_bytes + (int64_t)h0 * 2);
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            acc[2 * i]     = __uint_as_float(d[i] << 16);
+            acc[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+        }
+    }
     for(int k = 0; k < topk; k++)
     {
         const int pos = inv[t * topk + k];
@@ -703,7 +721,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     KernelTimer timer(MI355_MOE_K_COMBINE, stream);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, inv,
                        static_cast<const float*>(a.sorted_weight_ptr), static_cast<unsigned char*>(a.o_ptr), K, H,
-                       (int64_t)a.stride_token * 2);
+                       (int64_t)a.stride_token * 2, 0);
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
@@ -760,6 +778,176 @@ int launch_permute_weights(const void* src, void* dst, int32_t experts, int32_t 
     else
         hipLaunchKernelGGL(permute_weights_kernel<uint32_t>, dim3(grid), dim3(256), 0, stream,
                            static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst), granules, n, kgran, nw, kw, inverse);
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stand-alone grouped GEMMs behind ck_tile's MoeFlatmmHostArgs: the same kernels as the fused path,
+// with the intermediate in ck_tile's [tokens * topk, .] layout instead of sorted-row order.
+namespace {
+struct FlatmmLayout
+{
+    size_t map_off, inv_off, p_off, total;
+    int64_t max_pad;
+    int32_t max_tiles;
+    int mblk, hidden, inter;
+    mi355_fused_moe_traits traits;
+};
+
+int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
+{
+    if(kind != MI355_MOE_GEMM1_GATE_UP && kind != MI355_MOE_GEMM2)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: kind %d (gate+up and down GEMMs are implemented)", kind);
+    const bool g1     = kind == MI355_MOE_GEMM1_GATE_UP;
+    const bool w8     = a.prec_b == MI355_MOE_INT8;
+    const bool ok_typ = (a.prec_b == MI355_MOE_BF16 && a.prec_a == MI355_MOE_BF16) ||
+                        (w8 && a.prec_a == (g1 ? MI355_MOE_INT8 : MI355_MOE_BF16));
+    if(!ok_typ)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: operand types a=%d b=%d (bf16 x bf16, int8 x int8 for the "
+                                             "gate+up GEMM, bf16 x int8 for the down GEMM)", a.prec_a, a.prec_b);
+    if(a.NumTokens < 0 || a.NumExperts <= 0 || a.NumExperts > 1024 || a.TopK <= 0 || a.TopK > 255 || a.N <= 0 || a.K <= 0 ||
+       a.block_m < 1 || a.block_m > 1024 || a.k_batch > 1 || (g1 && a.N % 2 != 0))
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: bad sizes (tokens=%d experts=%d topk=%d N=%d K=%d block_m=%d k_batch=%d)",
+                    a.NumTokens, a.NumExperts, a.TopK, a.N, a.K, a.block_m, a.k_batch);
+    L.hidden = g1 ? a.K : a.N;
+    L.inter  = g1 ? a.N / 2 : a.K;
+    if(L.hidden % 32 != 0 || L.inter % 32 != 0)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: N and K must give hidden and intermediate sizes that are "
+                                             "multiples of 32 (hidden=%d inter=%d)", L.hidden, L.inter);
+    const int prec = w8 ? MI355_MOE_INT8 : MI355_MOE_BF16;
+    L.traits       = mi355_fused_moe_traits{prec, prec, MI355_MOE_BF16, MI355_MOE_FP32, MI355_MOE_FP32, MI355_MOE_FP32,
+                                            MI355_MOE_FP32, a.block_m, 1, 0, 0, 0};
+    L.mblk         = pick_mblk(L.traits, a.NumTokens, a.TopK, a.NumExperts, L.hidden, L.inter);
+    L.max_pad      = (int64_t)a.TopK * a.NumTokens + (int64_t)a.NumExperts * a.block_m - a.TopK;
+    L.max_tiles    = (int32_t)(a.NumExperts + L.max_pad / (L.mblk * 32) + 1);
+    L.total        = 0;
+    auto bump      = [&](size_t bytes) {
+        const size_t off = L.total;
+        L.total += round_up<size_t>(bytes, 256);
+        return off;
+    };
+    L.map_off = bump(sizeof(int) * (kMapHdr + (size_t)kMapEnt * L.max_tiles));
+    L.inv_off = bump(sizeof(int) * (size_t)a.NumTokens * a.TopK);
+    L.p_off   = bump(g1 ? 0 : (size_t)L.max_pad * L.hidden * 2);
+    return MI355_MOE_OK;
+}
+} // namespace
+
+size_t moe_flatmm_workspace_bytes(int kind, const mi355_moe_flatmm_args& a)
+{
+    FlatmmLayout L{};
+    return flatmm_layout(kind, a, L) == MI355_MOE_OK ? L.total : 0;
+}
+
+int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stream)
+{
+    FlatmmLayout L{};
+    int rc = flatmm_layout(kind, a, L);
+    if(rc != MI355_MOE_OK)
+        return rc;
+    const bool g1 = kind == MI355_MOE_GEMM1_GATE_UP;
+    const bool w8 = a.prec_b == MI355_MOE_INT8;
+    if(!a.p_sorted_token_ids || !a.p_sorted_expert_ids || !a.p_max_token_id || !a.a_ptr || !a.b_ptr || !a.c_ptr ||
+       (!g1 && !a.p_sorted_expert_weights))
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: null pointer");
+    if(a.exp_bias != nullptr)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: expert bias is not implemented");
+    if(w8 && (!a.scale_n || (g1 && !a.scale_m)))
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: int8 weights need scale_n (and int8 activations scale_m)");
+    const int T = a.NumTokens, E = a.NumExperts, K = a.TopK, H = L.hidden, I = L.inter;
+    const int a_b = a.prec_a == MI355_MOE_INT8 ? 1 : 2, b_b = w8 ? 1 : 2;
+    if(a.stride_A < a.K || a.stride_B != a.K || a.stride_C < (g1 ? I : H) || ((int64_t)a.stride_A * a_b) % 16 != 0 ||
+       ((int64_t)a.stride_C * 2) % 16 != 0)
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: strides (A=%d B=%d C=%d): B must be [experts, N, K] with K "
+                                         "contiguous, rows of A and C 16-byte aligned", a.stride_A, a.stride_B, a.stride_C);
+    for(const void* ptr : {a.a_ptr, a.b_ptr, static_cast<const void*>(a.c_ptr)})
+        if(reinterpret_cast<uintptr_t>(ptr) % 16 != 0)
+            return fail(MI355_MOE_E_INVALID, "moe_flatmm: a, b and c must be 16-byte aligned");
+    if(T == 0)
+        return MI355_MOE_OK;
+    if(a.ws_ptr == nullptr || a.ws_bytes < L.total)
+        return fail(MI355_MOE_E_WORKSPACE, "moe_flatmm: workspace of %zu bytes needed, %zu given", L.total,
+                    a.ws_ptr ? a.ws_bytes : (size_t)0);
+    if(reinterpret_cast<uintptr_t>(a.ws_ptr) % 256 != 0)
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: workspace must be 256-byte aligned");
+    unsigned char* wsb = static_cast<unsigned char*>(a.ws_ptr);
+    int* tile_map      = reinterpret_cast<int*>(wsb + L.map_off);
+    int* inv           = reinterpret_cast<int*>(wsb + L.inv_off);
+    const int mblk     = L.mblk;
+    const int prec     = L.traits.prec_i;
+    {
+        KernelTimer timer(MI355_MOE_K_PREP, stream);
+        const int n_inv     = T * K;
+        const int prep_grid = 1 + std::min(ceil_div(n_inv, kPrepBlock * 4), 64);
+        hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
+                           static_cast<const int*>(a.p_sorted_expert_ids), static_cast<const int*>(a.p_max_token_id),
+                           a.block_m, E, mblk * 32, (int)ceil_div<int64_t>(L.max_pad, a.block_m), L.max_tiles, tile_map,
+                           inv, n_inv);
+        if(!g1)
+            hipLaunchKernelGGL(moe_inv_kernel, dim3(std::min<int>(ceil_div<int64_t>(L.max_pad, 256), 1024)), dim3(256), 0,
+                               stream, static_cast<const int*>(a.p_sorted_token_ids),
+                               static_cast<const int*>(a.p_max_token_id), (int)L.max_pad, T, K, inv);
+    }
+    MI355_HIP_TRY(hipGetLastError());
+
+    GemmParams p{};
+    p.sorted_ids     = static_cast<const int*>(a.p_sorted_token_ids);
+    p.tile_map       = tile_map;
+    p.tokens         = T;
+    p.slot_rows      = K;
+    p.x              = static_cast<const unsigned char*>(a.a_ptr);
+    p.x_row_bytes    = (int64_t)a.stride_A * a_b;
+    p.w              = static_cast<const unsigned char*>(a.b_ptr);
+    p.w_row_bytes    = (int64_t)a.K * b_b;
+    p.w_expert_bytes = (int64_t)a.N * a.K * b_b;
+    p.w_scale        = w8 ? static_cast<const float*>(a.scale_n) : nullptr;
+    p.k_bytes_x      = a.K * a_b;
+    p.k_bytes_w      = a.K * b_b;
+    const int64_t a_rows = g1 ? T : (int64_t)T * K;
+    if(a_rows * p.x_row_bytes >= ((int64_t)1 << 32) && mblk > 4)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: A of 4 GiB or more is not supported at this problem size");
+    const bool decode = mblk == 1 && decode_supported(a_rows * p.x_row_bytes, a_rows * p.x_row_bytes, p.w_expert_bytes);
+    if(g1)
+    {
+        p.x_scale       = w8 ? static_cast<const float*>(a.scale_m) : nullptr;
+        p.out           = static_cast<unsigned char*>(a.c_ptr);
+        p.out_row_bytes = (int64_t)a.stride_C * 2;
+        p.n_out         = I;
+        p.n_total       = 2 * I;
+        p.n_ntiles      = decode ? ceil_div(I, decode_tile_cols(true)) : ceil_div(I, 128);
+        if(decode)
+            rc = launch_gemm_decode(prec, true, p, L.max_tiles, stream);
+        else if(mblk > 4)
+            rc = launch_gemm_big(prec, true, p, L.max_tiles, stream);
+        else if(prec == MI355_MOE_BF16)
+            rc = launch_gemm<kBf16, true>(mblk, p, L.max_tiles, stream);
+        else
+            rc = launch_gemm<kI8, true>(mblk, p, L.max_tiles, stream);
+        return rc;
+    }
+    p.out           = wsb + L.p_off;
+    p.out_row_bytes = (int64_t)H * 2;
+    p.n_out         = H;
+    p.n_total       = H;
+    const bool decode1 = decode && (int64_t)std::min<int64_t>(E, (int64_t)T * K) * ceil_div(H, 256) < device_info().num_cu;
+    p.n_ntiles      = decode1 ? ceil_div(H, decode_tile_cols(false)) : ceil_div(H, 256);
+    if(decode1)
+        rc = launch_gemm_decode(prec, false, p, L.max_tiles, stream);
+    else if(mblk > 4)
+        rc = launch_gemm_big(prec, false, p, L.max_tiles, stream);
+    else if(prec == MI355_MOE_BF16)
+        rc = launch_gemm<kBf16, false>(mblk, p, L.max_tiles, stream);
+    else
+        rc = launch_gemm<kBf16W8, false>(mblk, p, L.max_tiles, stream);
+    if(rc != MI355_MOE_OK)
+        return rc;
+    {
+        KernelTimer timer(MI355_MOE_K_COMBINE, stream);
+        hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + L.p_off, inv,
+                           static_cast<const float*>(a.p_sorted_expert_weights), static_cast<unsigned char*>(a.c_ptr), K, H,
+                           (int64_t)a.stride_C * 2, 1);
+    }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }

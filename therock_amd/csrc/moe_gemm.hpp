@@ -50,6 +50,9 @@ int decode_tile_cols(bool gemm0);
 bool decode_supported(int64_t x_bytes, int64_t y_bytes, int64_t w_expert_bytes);
 int launch_gemm_decode(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream);
 
+size_t moe_flatmm_workspace_bytes(int kind, const mi355_moe_flatmm_args& a);
+int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stream);
+
 int launch_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
                            int32_t nw, int32_t kw, int32_t kv, int32_t inverse, hipStream_t stream);
 

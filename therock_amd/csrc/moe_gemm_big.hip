@@ -166,12 +166,13 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
         {
             const int lrow = (q4 + 4 * j) * 16 + lrow16;
             uint32_t src   = lrow < nrows ? row0 + lrow : row0;
-            if constexpr(GEMM0)
+            if(GEMM0 || p.slot_rows > 0)
             {
-                int tok = p.tokens;
+                int sid = p.tokens;
                 if(lrow < nrows)
-                    tok = p.sorted_ids[row0 + lrow] & 0xffffff;
-                src = tok < p.tokens ? tok : 0;
+                    sid = p.sorted_ids[row0 + lrow];
+                const bool ok = (sid & 0xffffff) < p.tokens;
+                src           = !ok ? 0u : GEMM0 ? (uint32_t)(sid & 0xffffff) : (uint32_t)slot_row(sid, p.slot_rows);
             }
             doff[j] = src * (uint32_t)p.x_row_bytes + cchunk * 16;
         }

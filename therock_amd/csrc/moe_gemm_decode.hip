@@ -81,8 +81,15 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
         }
         else
         {
-            xvalid[j] = r < nrows;
-            xoff[j]   = (uint32_t)(row0 + (xvalid[j] ? r : 0)) * (uint32_t)p.x_row_bytes + xchunk * 16;
+            xvalid[j]   = r < nrows;
+            int64_t src = row0 + (xvalid[j] ? r : 0);
+            if(p.slot_rows > 0)
+            {
+                const int sid = p.sorted_ids[src];
+                xvalid[j]     = xvalid[j] && (sid & 0xffffff) < p.tokens;
+                src           = xvalid[j] ? slot_row(sid, p.slot_rows) : 0;
+            }
+            xoff[j] = (uint32_t)src * (uint32_t)p.x_row_bytes + xchunk * 16;
         }
     }
     const int wchunk = tid % (kDecWKB / 16);

@@ -47,7 +47,17 @@ struct GemmParams
     int n_total;             // weight rows per expert (gemm0: 2*inter, gemm1: hidden)
     int n_ntiles;            // tiles along n
     int tokens;
+    // Row addressing of the stand-alone GEMM entry point (0 in the fused path, where Y and P are in
+    // sorted-row order): slot_rows = top-k count when gemm0's output rows, respectively gemm1's input
+    // rows, are token * topk + slot (ck_tile's MoeFlatmm convention, moe_flatmm_kernel.hpp:790-801)
+    int slot_rows;
 };
+
+// row of a [tokens * topk, .] buffer a sorted id refers to
+__device__ inline int64_t slot_row(int sid, int topk)
+{
+    return (int64_t)(sid & 0xffffff) * topk + static_cast<int>(static_cast<uint32_t>(sid) >> 24);
+}
 
 // Work item -> tile.  XCD x gets a contiguous range of the work list (workgroup ids are dealt
 // round-robin to the 8 XCDs); inside an expert the row tiles of one weight tile are adjacent.  One
@@ -330,18 +340,26 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
     load_channel_scales(sbase && b_ok ? sbase + (GEMM0 ? p.n_out + col_a : col_b) : nullptr, sc1);
     float sa[NBLK];
     bool real[NBLK];
+    int64_t orow[NBLK]; // output row
 #pragma unroll
     for(int i = 0; i < NBLK; i++)
     {
         sa[i]   = 1.0f;
         real[i] = true;
-        if((GEMM0 && p.x_scale != nullptr) || (!GEMM0 && SKIP_PAD))
+        orow[i] = row0 + first_row + i * row_step + r32;
+        if((GEMM0 && (p.x_scale != nullptr || p.slot_rows > 0)) || (!GEMM0 && SKIP_PAD))
         {
             const int r   = min(first_row + i * row_step + r32, nrows - 1); // clamped: always a valid cell
-            const int tok = p.sorted_ids[row0 + r] & 0xffffff;
+            const int sid = p.sorted_ids[row0 + r];
+            const int tok = sid & 0xffffff;
             real[i]       = tok < p.tokens;
             if constexpr(GEMM0)
-                sa[i] = real[i] ? p.x_scale[tok] : 0.0f;
+            {
+                if(p.x_scale != nullptr)
+                    sa[i] = real[i] ? p.x_scale[tok] : 0.0f;
+                if(p.slot_rows > 0)
+                    orow[i] = real[i] ? slot_row(sid, p.slot_rows) : 0;
+            }
         }
     }
     // every load above completes here, on every path: a load left pending on a path that does not use
@@ -352,7 +370,7 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
         asm volatile("" : "+v"(sc0[v]), "+v"(sc1[v]));
 #pragma unroll
     for(int i = 0; i < NBLK; i++)
-        asm volatile("" : "+v"(sa[i]));
+        asm volatile("" : "+v"(sa[i]), "+v"(orow[i]));
     // ---- apply
 #pragma unroll
     for(int i = 0; i < NBLK; i++)
@@ -364,7 +382,8 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
         if constexpr(GEMM0)
         {
             if(a_ok)
-                epilogue_gemm0<MODE>(p, acc[i][0], acc[i][1], sc0, sc1, sa[i], row0 + r, in_tile, col_a, kg);
+                epilogue_gemm0<MODE>(p, acc[i][0], acc[i][1], sc0, sc1, sa[i], orow[i],
+                                     in_tile && (p.slot_rows == 0 || real[i]), col_a, kg);
         }
         else
         {

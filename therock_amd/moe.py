@@ -203,6 +203,33 @@ def rowwise_quant(x, q_dtype: str, stream=None):
     return q, scale
 
 
+GEMM1_GATE_UP, GEMM2 = 1, 2
+
+
+def moe_flatmm(kind: int, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens: int, topk: int, block_m: int,
+               sorted_weights=None, scale_m=None, scale_n=None, stream=None):
+    """One grouped GEMM of the MoE layer as its own launch (ck_tile's MoeFlatmm conventions): kind
+    GEMM1_GATE_UP writes c[token * topk + slot, :N/2] = silu(gate) * up, kind GEMM2 adds the weighted
+    down projection of a[token * topk + slot] to c[token].  b is [experts, N, K]."""
+    import torch
+
+    experts, n, k = b.shape
+    dt = {torch.bfloat16: "bf16", torch.int8: "int8"}
+    args = _lib.FlatmmArgs(_ptr(sorted_ids), _ptr(sorted_weights), _ptr(sorted_eid), _ptr(max_token_id), _ptr(a), _ptr(b),
+                           _ptr(c), _ptr(scale_m), _ptr(scale_n), None, None, 0, num_tokens, experts, topk, 1,
+                           sorted_ids.numel(), n, k, a.stride(0), k, c.stride(0), _lib.DTYPES[dt[a.dtype]],
+                           _lib.DTYPES[dt[b.dtype]], block_m)
+    lib = _lib.load()
+    ws_bytes = int(lib.mi355_moe_flatmm_workspace_size(kind, C.byref(args)))
+    ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=a.device)
+    args.ws_ptr, args.ws_bytes = _ptr(ws), ws_bytes
+    rc = lib.mi355_moe_flatmm(kind, C.byref(args), _stream(stream))
+    if rc == _lib.E_UNSUPPORTED:
+        return -1.0
+    _check(rc, "moe_flatmm")
+    return 0.0
+
+
 def permute_weights(w, nw: int = 16, kw: int = 4, kv: int | None = None, inverse: bool = False, stream=None):
     """[experts, n, k] weights to (inverse=False) or from (inverse=True) ck_tile's pre-shuffled layout
     b_nr_kr_kw_nw_kv.  kv defaults to 16 bytes worth of elements (CK's example: 8 for bf16, 16 for 8-bit)."""
