@@ -74,6 +74,18 @@ def ck_ref():
     return _ref
 
 
+_ref_gpu = None
+
+
+def ck_ref_gpu():
+    """ck_tile's device reference (needs a GPU), or None when not built.  Load it only after the process
+    has initialised its own HIP runtime: the library carries device code."""
+    global _ref_gpu
+    if _ref_gpu is None:
+        _ref_gpu = _load(os.path.join(_HERE, "_ref", "libck_ref_gpu.so"))
+    return _ref_gpu
+
+
 def _p(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 
@@ -253,6 +265,28 @@ def moe_gemm(kind, sorted_ids, sorted_eid, sorted_w, post_pad, block_m, a, b, c,
            C.c_int32(c.shape[1]), _p(_c(scale_a, np.float32)), _p(_c(scale_b, np.float32)))
     if rc != 0:
         raise ValueError(f"moe_oracle_moe_gemm failed ({rc})")
+    return c
+
+
+def ck_moe_gemm_gpu(kind, sorted_ids, sorted_eid, sorted_w, post_pad, block_m, a_bf16, b_bf16, c_bf16, num_tokens, topk,
+                    scale_a=None, scale_b=None):
+    """ck_tile::reference_moe_gemm_gpu (a device kernel: needs a GPU) on bf16 operands given as bf16 bits.
+    c is updated in place (the down kind adds to it) and returned."""
+    r = ck_ref_gpu()
+    if r is None:
+        raise RuntimeError("oracle/_ref/libck_ref_gpu.so is not built")
+    a, b = _c(a_bf16, np.uint16), _c(b_bf16, np.uint16)
+    c = np.ascontiguousarray(c_bf16, dtype=np.uint16)
+    E, N, K = b.shape
+    ids, eid, w = _c(sorted_ids, np.int32), _c(sorted_eid, np.int32), _c(sorted_w, np.float32)
+    sa = _c(scale_a if scale_a is not None else np.ones(a.shape[0], np.float32), np.float32)
+    sb = _c(scale_b if scale_b is not None else np.ones((E, N), np.float32), np.float32)
+    r.ck_ref_moe_gemm_gpu.restype = C.c_int
+    rc = r.ck_ref_moe_gemm_gpu(C.c_int32(kind), _p(ids), _p(eid), C.c_int32(int(post_pad)), _p(a), _p(b), _p(c), _p(w),
+                               C.c_int32(num_tokens), C.c_int32(block_m), C.c_int32(topk), C.c_int32(ids.size),
+                               C.c_int32(E), C.c_int32(N), C.c_int32(K), _p(sa), _p(sb))
+    if rc != 0:
+        raise RuntimeError(f"ck_ref_moe_gemm_gpu failed ({rc})")
     return c
 
 

@@ -22,6 +22,7 @@
 #include "ck_tile/host/reference/reference_rowwise_quantization2d.hpp"
 #include "ck_tile/host/reference/reference_permute.hpp"
 
+
 using ck_tile::HostTensor;
 using ck_tile::index_t;
 

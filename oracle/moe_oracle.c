@@ -31,9 +31,9 @@
  *   fused moe   - ck_tile's reference_fused_moe in oracle/_ref on the same inputs; an
  *                 independent dense (sorting-free) float64 formulation in numpy.
  *   bf16 / e4m3 - exhaustive comparison with torch's bfloat16 / float8_e4m3fn casts.
- *   moe gemm    - ck_tile's reference for these is a device kernel and cannot run on the CPU: pinned by a
- *                 dense float64 formulation that never sorts, by the composition gate+up -> down against
- *                 moe_oracle_fused_moe (itself bit-exact with ck_tile), and by a triple loop on tiny shapes.
+ *   moe gemm    - a dense float64 formulation that never sorts, the composition gate+up -> down against
+ *                 moe_oracle_fused_moe (itself bit-exact with ck_tile); ck_tile's reference for these is a
+ *                 device kernel (oracle/_ref/libck_ref_gpu.so), compared in a GPU test.
  *   topk softmax- ck_tile's reference_softmax + reference_topk in oracle/_ref; closed forms (equal
  *                 logits, shift invariance, weights of all experts sum to one), scipy's softmax and
  *                 numpy's argsort on random rows.

@@ -86,3 +86,33 @@ def test_unsupported_and_errors():
     assert ta.moe_flatmm(0, z(4, 64), z(2, 128, 64), z(8, 64), ids, eid, tot, 4, 2, 32) == -1.0
     with pytest.raises(RuntimeError):
         ta.moe_flatmm(ta.GEMM2, z(8, 64), z(2, 64, 64), z(4, 64), ids, eid, tot, 4, 2, 32)  # no sorted weights
+
+
+@pytest.mark.parametrize("T,E,K,H,I,unit", [(40, 6, 3, 64, 96, 32), (130, 8, 2, 256, 128, 16)])
+def test_oracle_against_ck_tile_device_reference(T, E, K, H, I, unit):
+    """Pins moe_oracle_moe_gemm on ck_tile::reference_moe_gemm_gpu, which only runs on a GPU.  The gate+up
+    kind accumulates in the same order: equal up to the device's exp in SiLU (one bf16 ulp at most, rarely).
+    The down kind adds bf16 partial sums with atomics in ck_tile: compared to a bf16-rounding tolerance."""
+    import torch
+
+    torch.cuda.init()  # this process's HIP runtime first, then the reference library with its device code
+    if oracle.ck_ref_gpu() is None:
+        pytest.skip("oracle/_ref/libck_ref_gpu.so not built")
+    rng = np.random.default_rng(T)
+    bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
+    x, g, d = bf(rng.standard_normal((T, H))), bf(rng.standard_normal((E, 2 * I, H)) * 0.1), bf(rng.standard_normal((E, H, I)) * 0.1)
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
+    w = rng.random((T, K), dtype=np.float32)
+    s_ids, s_w, s_eid, pp = oracle.moe_sorting(ids, w, E, unit)
+    sa, sg = (0.5 + rng.random(T)).astype(np.float32), (0.5 + rng.random((E, 2 * I))).astype(np.float32)
+    f32 = lambda a: oracle.to_f32(a, oracle.DT_BF16)
+
+    y_ck = oracle.ck_moe_gemm_gpu(1, s_ids, s_eid, s_w, pp, unit, x, g, np.zeros((T * K, I), np.uint16), T, K, sa, sg)
+    y_or = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, f32(x), f32(g), np.zeros((T * K, I), np.uint16), T, K, sa, sg)
+    diff = np.abs(y_ck.astype(np.int32) - y_or.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 0.01
+
+    c0 = bf(rng.standard_normal((T, H)) * 0.1)
+    o_ck = oracle.ck_moe_gemm_gpu(2, s_ids, s_eid, s_w, pp, unit, y_or, d, c0.copy(), T, K)
+    o_or = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, f32(y_or), f32(d), c0.copy(), T, K)
+    assert _rel(f32(o_ck), f32(o_or)) < 8e-3
