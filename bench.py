@@ -28,6 +28,7 @@ if ROOT not in sys.path:
 
 METRIC = "fused-MoE TFLOP/s (prefill) + HBM GB/s (decode), % of MI355X roofline, 1 GPU"
 HEADLINE = "cfg3_dsv3_fp8"
+DOMINANT = "moe_gemm0_gate_up_silu"  # the kernel the roofline entry is about
 # published MI355X peaks: dense MFMA TFLOP/s (TOP/s for int8) and HBM GB/s
 PEAK_MFMA = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
 PEAK_HBM = 8000.0
@@ -38,8 +39,9 @@ def log(*a):
 
 
 def run_workload(cfg, steps, warmup, seed=0):
-    """Times `steps` passes of the path; per-kernel durations come from HIP events recorded by
-    the library on the launch stream inside the same timed region."""
+    """Times `steps` passes of the path.  The dominant kernel's duration comes from HIP events the
+    library records on the launch stream inside the timed region, the other kernels' from an untimed
+    pass just before it."""
     import torch
 
     import therock_amd as ta
@@ -55,13 +57,25 @@ def run_workload(cfg, steps, warmup, seed=0):
     for _ in range(warmup):
         assert ta.fused_moe(traits, args) == 0.0
     torch.cuda.synchronize()
+    # Per-kernel durations of every kernel: an untimed pass with an event pair around each launch.  Those
+    # records sit between the launches and lengthen a pass by a few microseconds each, so the timed region
+    # below keeps only the pair around the dominant kernel (the gate+up GEMM), which is what the roofline
+    # entry is computed from.
     _lib.profile_start()
+    for _ in range(max(3, min(steps, 10))):
+        ta.fused_moe(traits, args)
+    torch.cuda.synchronize()
+    kern = _lib.profile_stop()
+    _lib.profile_start(kinds=[DOMINANT])
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         ta.fused_moe(traits, args)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    kern = _lib.profile_stop()
+    dom = _lib.profile_stop()
+    if DOMINANT in dom:
+        kern[DOMINANT] = dom[DOMINANT]
     ms = (t1 - t0) * 1e3 / steps
     post_pad = int(buf.total[0])
     active = int(torch.unique(inp["topk_ids"]).numel())

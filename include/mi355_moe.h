@@ -315,6 +315,9 @@ enum mi355_moe_kernel_kind
     MI355_MOE_NUM_KERNELS    = 10
 };
 int mi355_moe_profile_start(void);
+/* same, timing only the kernel kinds whose bit (1 << kind) is set: every pair of event records sits between
+ * two launches and costs a few microseconds of the stream's time, which matters for the decode regime */
+int mi355_moe_profile_start_kinds(uint32_t kind_mask);
 int mi355_moe_profile_stop(double* ms, int32_t* launches);
 const char* mi355_moe_kernel_name(int32_t kind);
 

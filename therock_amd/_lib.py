@@ -107,6 +107,7 @@ PROTOTYPES = {
     "mi355_moe_rowwise_quant": (C.c_int, [C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_int32, C.c_void_p,
                                           C.c_void_p, C.c_void_p]),
     "mi355_moe_profile_start": (C.c_int, []),
+    "mi355_moe_profile_start_kinds": (C.c_int, [C.c_uint32]),
     "mi355_moe_profile_stop": (C.c_int, [C.POINTER(C.c_double), C.POINTER(C.c_int32)]),
     "mi355_moe_kernel_name": (C.c_char_p, [C.c_int32]),
     "mi355_moe_last_error": (C.c_char_p, []),
@@ -135,8 +136,17 @@ def load():
 NUM_KERNELS = 10
 
 
-def profile_start() -> None:
-    load().mi355_moe_profile_start()
+def profile_start(kinds=None) -> None:
+    """Starts per-kernel event timing; kinds = iterable of kernel names restricts it to those kernels."""
+    lib = load()
+    if kinds is None:
+        lib.mi355_moe_profile_start()
+        return
+    names = [lib.mi355_moe_kernel_name(k).decode() for k in range(NUM_KERNELS)]
+    mask = 0
+    for k in kinds:
+        mask |= 1 << names.index(k)
+    lib.mi355_moe_profile_start_kinds(C.c_uint32(mask))
 
 
 def profile_stop() -> dict:

@@ -43,7 +43,8 @@ const DeviceInfo& device_info()
 namespace {
 struct ProfileState
 {
-    bool enabled = false;
+    bool enabled  = false;
+    uint32_t mask = 0xffffffffu; // kernel kinds that are timed
     std::vector<hipEvent_t> pool; // events created so far
     size_t used = 0;
     struct Rec
@@ -68,7 +69,7 @@ struct ProfileState
 ProfileState g_prof;
 } // namespace
 
-bool profiling_enabled() { return g_prof.enabled; }
+bool profiling_enabled(int kind) { return g_prof.enabled && ((g_prof.mask >> kind) & 1u) != 0; }
 
 void profile_mark(int kind, hipStream_t stream, bool begin)
 {
@@ -105,8 +106,16 @@ __attribute__((visibility("default"))) const char* mi355_moe_kernel_name(int32_t
     return kind >= 0 && kind < MI355_MOE_NUM_KERNELS ? names[kind] : "?";
 }
 
+__attribute__((visibility("default"))) int mi355_moe_profile_start_kinds(uint32_t kind_mask);
+
 __attribute__((visibility("default"))) int mi355_moe_profile_start(void)
 {
+    return mi355_moe_profile_start_kinds(0xffffffffu);
+}
+
+__attribute__((visibility("default"))) int mi355_moe_profile_start_kinds(uint32_t kind_mask)
+{
+    g_prof.mask = kind_mask;
     g_prof.used = 0;
     g_prof.recs.clear();
     for(auto& p : g_prof.pending)

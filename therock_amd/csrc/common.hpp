@@ -52,7 +52,7 @@ struct DeviceInfo
 const DeviceInfo& device_info();
 
 // ---- optional per-kernel event timing (mi355_moe_profile_start / _stop)
-bool profiling_enabled();
+bool profiling_enabled(int kind);
 void profile_mark(int kind, hipStream_t stream, bool begin);
 
 // brackets one kernel launch with events while profiling is on
@@ -61,7 +61,7 @@ struct KernelTimer
     int kind;
     hipStream_t stream;
     bool on;
-    KernelTimer(int k, hipStream_t s) : kind(k), stream(s), on(profiling_enabled())
+    KernelTimer(int k, hipStream_t s) : kind(k), stream(s), on(profiling_enabled(k))
     {
         if(on)
             profile_mark(kind, stream, true);
