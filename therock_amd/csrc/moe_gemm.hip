@@ -565,7 +565,7 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
     w.sort_off       = bump(sorting_workspace_bytes(tokens, experts, topk));
     w.map_off        = bump(sizeof(int) * (kMapHdr + (size_t)kMapEnt * w.max_tiles));
     w.inv_off        = bump(sizeof(int) * (size_t)tokens * topk);
-    w.y_off          = bump((size_t)w.max_pad * inter * y_b);
+    w.y_off          = bump((size_t)round_up<int64_t>(w.max_pad, 16) * inter * y_b); // whole 16-row slabs
     w.ys_kb_stride   = round_up<int64_t>(w.max_pad, 256) + 512;
     w.ys_off         = bump(t.prec_i == MI355_MOE_FP8 ? (size_t)w.ys_kb_stride * (inter / 32) : 0);
     w.p_off          = bump((size_t)w.max_pad * hidden * 2);
@@ -671,6 +671,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     if(mblk > 4 && (int64_t)T * p.x_row_bytes >= ((int64_t)1 << 32))
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: a token buffer of 4 GiB or more (stride_token=%d) is not "
                                              "supported at this problem size", a.stride_token);
+    // the two large-tile GEMMs hand Y over in the slab-major layout
+    p.y_slab = (mblk > 4 && ((int64_t)I * y_b) % 64 == 0) ? (int)((int64_t)I * y_b / 64) : 0;
     if(decode)
         rc = launch_gemm_decode(t.prec_i, true, p, ws.max_tiles, stream);
     else if(mblk > 4)

@@ -175,12 +175,16 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 src           = !ok ? 0u : GEMM0 ? (uint32_t)(sid & 0xffffff) : (uint32_t)slot_row(sid, p.slot_rows);
             }
             doff[j] = src * (uint32_t)p.x_row_bytes + cchunk * 16;
+            if(!GEMM0 && p.y_slab > 0) // slab-major Y: whole slabs; slabs past the tile's rows read its first
+                doff[j] = (uint32_t)(((row0 >> 4) + ((q4 + 4 * j) * 16 < nrows ? q4 + 4 * j : 0)) * p.y_slab) * 1024u +
+                          lrow16 * 64 + cchunk * 16;
         }
         // scales: K block (q >> 1) of the step, rows (q & 1) * 256 .. + 255 (the rows are padded)
         doff[5] = (uint32_t)((q4 >> 1) * p.ys_kb_stride + row0 + (q4 & 1) * 256 + lane * 4);
         doff[6] = doff[7] = 0;
     }
     const int64_t ys_step = (kStepKB / 32) * p.ys_kb_stride;
+    const int x_step      = (!GEMM0 && p.y_slab > 0) ? 1024 : kStepKB; // bytes between token steps
 
     const uint32_t lds_base = lds_offset(lds);
     const int kt_count      = p.k_bytes_x / kStepKB; // compute steps = weight units (even)
@@ -201,7 +205,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
         if(x >= kt_count)
             return;
         const uint32_t sbase     = lds_base + kXOffset + (x % kXStages) * kXStageBytes + q4 * 1024;
-        const unsigned char* src = dbase + x * kStepKB;
+        const unsigned char* src = dbase + x * x_step;
 #pragma unroll
         for(int j = 0; j < 5; j++)
             dma16(src, doff[j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));

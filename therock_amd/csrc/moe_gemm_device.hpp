@@ -51,7 +51,18 @@ struct GemmParams
     // sorted-row order): slot_rows = top-k count when gemm0's output rows, respectively gemm1's input
     // rows, are token * topk + slot (ck_tile's MoeFlatmm convention, moe_flatmm_kernel.hpp:790-801)
     int slot_rows;
+    // Y layout between the two large-tile GEMMs: 0 = row-major; otherwise the number of 64-byte K
+    // segments of a row, and Y is stored slab-major: [row / 16][segment][row % 16][64 B], so that the
+    // 16 rows x 64 B one token DMA instruction of the down GEMM fetches are 1 KiB of consecutive memory
+    // (8 whole cache lines instead of 16 half lines)
+    int y_slab;
 };
+
+// byte offset of K byte kb of row `row` in the slab-major Y layout
+__device__ inline int64_t y_slab_offset(int64_t row, int kb, int segs)
+{
+    return (((row >> 4) * segs + (kb >> 6)) << 10) + ((row & 15) << 6) + (kb & 63);
+}
 
 // row of a [tokens * topk, .] buffer a sorted id refers to
 __device__ inline int64_t slot_row(int sid, int topk)
@@ -253,7 +264,9 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
         const float u = static_cast<float>(acc_up[v]) * (sa * us[v]);
         y[v]          = silu(g) * u;
     }
-    unsigned char* dst = p.out + grow * p.out_row_bytes;
+    constexpr int y_b  = MODE == kFp8 ? 1 : 2;
+    unsigned char* dst = p.y_slab > 0 ? p.out + y_slab_offset(grow, col0 * y_b, p.y_slab)
+                                      : p.out + grow * p.out_row_bytes + (int64_t)col0 * y_b;
     if constexpr(MODE == kFp8)
     {
         float amax = 0.f;
@@ -280,7 +293,7 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
         }
         if(store)
         {
-            *reinterpret_cast<uint4*>(dst + col0) = make_uint4(q[0], q[1], q[2], q[3]);
+            *reinterpret_cast<uint4*>(dst) = make_uint4(q[0], q[1], q[2], q[3]);
             if(kg == 0)
                 p.y_scale[(int64_t)(col0 >> 5) * p.ys_kb_stride + grow] = static_cast<unsigned char>(sb);
         }
@@ -292,7 +305,7 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
         o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
         o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
         o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
-        uint4* d4 = reinterpret_cast<uint4*>(dst + (int64_t)col0 * 2);
+        uint4* d4 = reinterpret_cast<uint4*>(dst);
         d4[0]     = o0;
         d4[1]     = o1;
     }
