@@ -124,8 +124,8 @@ typedef struct mi355_fused_moe_traits
     int32_t prec_sq; /* smooth-quant scale dtype: FP32 (unused) */
     int32_t prec_kw; /* top-k weight dtype: FP32 */
     int32_t block_m; /* rows per sorted tile = unit_size of the sort: 16, 32, 64 or 128 */
-    int32_t activation;  /* 0 = gelu (unsupported), 1 = silu */
-    int32_t gate_only;   /* 0 = gate and up ([e, 2*inter, hidden]), 1 = gate only (unsupported) */
+    int32_t activation;  /* 0 = gelu (erf form, ck_tile::element_wise::Gelu), 1 = silu */
+    int32_t gate_only;   /* 0 = gate and up (g [e, 2*inter, hidden]), 1 = gate only (g [e, inter, hidden], y = act(gate)) */
     int32_t fused_quant; /* 0 = none; quantised dtypes always take a_scale/g_scale/d_scale */
     int32_t local_expert_masking; /* 1 = apply local_expert_mask_ptr in the sort */
 } mi355_fused_moe_traits;
@@ -137,9 +137,9 @@ typedef struct mi355_fused_moegemm_args
 {
     const void* a_ptr;              /* [tokens, stride_token] activations */
     const void* a_scale_ptr;        /* [tokens] fp32 per-token scale (quantised dtypes) or NULL */
-    const void* g_ptr;              /* [experts, 2*inter, hidden] gate rows then up rows */
+    const void* g_ptr;              /* [experts, 2*inter, hidden] gate rows then up rows; gate_only: [experts, inter, hidden] */
     const void* d_ptr;              /* [experts, hidden, inter] */
-    const void* g_scale_ptr;        /* [experts, 2*inter] fp32 or NULL */
+    const void* g_scale_ptr;        /* [experts, 2*inter] ([experts, inter] when gate_only) fp32 or NULL */
     const void* d_scale_ptr;        /* [experts, hidden] fp32 or NULL */
     const void* y_smooth_scale_ptr; /* [experts, inter]; accepted, must be NULL */
     void* o_ptr;                    /* [tokens, stride_token] output, written (not accumulated) */
@@ -257,7 +257,7 @@ int mi355_moe_permute_weights(const void* src, void* dst, int32_t experts, int32
  * bf16 epilogue the down GEMM sums a token's slots in fp32, in slot order, and rounds once. */
 enum mi355_moe_flatmm_kind
 {
-    MI355_MOE_GEMM1_GATE_ONLY = 0, /* not implemented */
+    MI355_MOE_GEMM1_GATE_ONLY = 0, /* C = silu(A x B^T), B [experts, N, K] */
     MI355_MOE_GEMM1_GATE_UP   = 1,
     MI355_MOE_GEMM2           = 2
 };

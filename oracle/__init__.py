@@ -52,6 +52,8 @@ def lib():
         _lib.moe_oracle_f32_to_e4m3.argtypes = [C.c_float]
         _lib.moe_oracle_silu.restype = C.c_float
         _lib.moe_oracle_silu.argtypes = [C.c_float]
+        _lib.moe_oracle_gelu.restype = C.c_float
+        _lib.moe_oracle_gelu.argtypes = [C.c_float]
         _lib.moe_oracle_num_threads.restype = C.c_int
         _lib.moe_oracle_set_num_threads.argtypes = [C.c_int]
     return _lib
@@ -71,6 +73,8 @@ def ck_ref():
             _ref.ck_ref_fp8_to_f32.argtypes = [C.c_uint8]
             _ref.ck_ref_silu.restype = C.c_float
             _ref.ck_ref_silu.argtypes = [C.c_float]
+            _ref.ck_ref_gelu.restype = C.c_float
+            _ref.ck_ref_gelu.argtypes = [C.c_float]
     return _ref
 
 
@@ -323,7 +327,7 @@ def ck_topk_softmax(logits, topk):
 # ----------------------------------------------------------------------------- fused MoE
 def fused_moe(a, a_dt, g, g_dt, d, d_dt, sorted_ids, sorted_w, sorted_eid, post_pad, block_m,
               tokens, experts, hidden, inter, topk, a_scale=None, g_scale=None, d_scale=None,
-              gate_only=False, out_dt=DT_BF16, strict=False, want_partials=False):
+              gate_only=False, out_dt=DT_BF16, strict=False, want_partials=False, activation=1):
     """Oracle forward.  Operands are numpy arrays holding the raw storage type of their dtype
     code (uint16 for bf16, uint8 for e4m3, int8, float32).  Returns o[tokens, hidden] (uint16 bf16
     bits or float32) and, if asked, the fp32 per-slot partials [tokens, topk, hidden]."""
@@ -339,14 +343,14 @@ def fused_moe(a, a_dt, g, g_dt, d, d_dt, sorted_ids, sorted_w, sorted_eid, post_
     rc = lib().moe_oracle_fused_moe(_p(a), a_dt, _p(a_scale), _p(g), g_dt, _p(g_scale), _p(d), d_dt,
                                     _p(d_scale), _p(o), out_dt, _p(ids), _p(w), _p(eid),
                                     int(post_pad), block_m, tokens, experts, hidden, inter, topk,
-                                    int(bool(gate_only)), int(bool(strict)), _p(part))
+                                    int(bool(gate_only)), int(bool(strict)), _p(part), int(activation))
     if rc != 0:
         raise MemoryError("moe_oracle_fused_moe failed")
     return (o, part) if want_partials else o
 
 
 def ck_fused_moe(a, g, d, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, tokens, experts,
-                 hidden, inter, topk, gate_only=False, f32_inputs=False):
+                 hidden, inter, topk, gate_only=False, f32_inputs=False, activation=1):
     """ck_tile::reference_fused_moe on bf16 (uint16 bits) or float32 operands -> bf16 bits."""
     r = ck_ref()
     if r is None:
@@ -357,7 +361,7 @@ def ck_fused_moe(a, g, d, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, t
     fn = r.ck_ref_fused_moe_f32 if f32_inputs else r.ck_ref_fused_moe_bf16
     ids, w, eid = _c(sorted_ids, np.int32), _c(sorted_w, np.float32), _c(sorted_eid, np.int32)
     fn(_p(a), _p(g), _p(d), _p(o), _p(ids), _p(w), _p(eid), int(post_pad), block_m, tokens, experts,
-       hidden, inter, topk, int(bool(gate_only)))
+       hidden, inter, topk, int(bool(gate_only)), int(activation))
     return o
 
 

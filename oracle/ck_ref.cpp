@@ -37,7 +37,7 @@ HostTensor<T> make_tensor(std::vector<std::size_t> lens, const void* src)
     return t;
 }
 
-template <typename AT, typename GT, typename DT>
+template <typename AT, typename GT, typename DT, typename Act>
 int run_fused(const void* a, const void* g, const void* d, void* o_bf16,
               const int32_t* sorted_ids, const float* sorted_w, const int32_t* sorted_eid,
               int32_t post_pad, int32_t block_m, int32_t T, int32_t E, int32_t H, int32_t I,
@@ -64,7 +64,7 @@ int run_fused(const void* a, const void* g, const void* d, void* o_bf16,
     nst.mData[0] = post_pad;
     HostTensor<index_t> topk_ids({(std::size_t)T, (std::size_t)K}); // unused under MOCK_ID
 
-    ck_tile::reference_fused_moe<float, ck_tile::element_wise::Silu>(
+    ck_tile::reference_fused_moe<float, Act>(
         a_h, g_h, d_h, sa, sg, sd, sy, o_h, ids_h, w_h, eid_h, nst, topk_ids, block_m, T, E, H, I, K,
         gate_only);
     std::memcpy(o_bf16, o_h.data(), sizeof(uint16_t) * (std::size_t)T * H);
@@ -112,9 +112,13 @@ __attribute__((visibility("default"))) int
 ck_ref_fused_moe_bf16(const void* a, const void* g, const void* d, void* o, const int32_t* sorted_ids,
                       const float* sorted_w, const int32_t* sorted_eid, int32_t post_pad,
                       int32_t block_m, int32_t T, int32_t E, int32_t H, int32_t I, int32_t K,
-                      int32_t gate_only)
+                      int32_t gate_only, int32_t activation)
 {
-    return run_fused<ck_tile::bf16_t, ck_tile::bf16_t, ck_tile::bf16_t>(
+    // activation codes of the example's fused_moe_traits: 0 = gelu, 1 = silu
+    if(activation == 0)
+        return run_fused<ck_tile::bf16_t, ck_tile::bf16_t, ck_tile::bf16_t, ck_tile::element_wise::Gelu>(
+            a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, T, E, H, I, K, gate_only);
+    return run_fused<ck_tile::bf16_t, ck_tile::bf16_t, ck_tile::bf16_t, ck_tile::element_wise::Silu>(
         a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, T, E, H, I, K, gate_only);
 }
 
@@ -124,10 +128,13 @@ __attribute__((visibility("default"))) int
 ck_ref_fused_moe_f32(const void* a, const void* g, const void* d, void* o, const int32_t* sorted_ids,
                      const float* sorted_w, const int32_t* sorted_eid, int32_t post_pad,
                      int32_t block_m, int32_t T, int32_t E, int32_t H, int32_t I, int32_t K,
-                     int32_t gate_only)
+                     int32_t gate_only, int32_t activation)
 {
-    return run_fused<float, float, float>(a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad,
-                                          block_m, T, E, H, I, K, gate_only);
+    if(activation == 0)
+        return run_fused<float, float, float, ck_tile::element_wise::Gelu>(
+            a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, T, E, H, I, K, gate_only);
+    return run_fused<float, float, float, ck_tile::element_wise::Silu>(
+        a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, T, E, H, I, K, gate_only);
 }
 
 // router: reference_softmax over the experts of each row, then reference_topk (sorted, largest)
@@ -195,6 +202,12 @@ __attribute__((visibility("default"))) float ck_ref_silu(float x)
 {
     float y;
     ck_tile::element_wise::Silu{}(y, x);
+    return y;
+}
+__attribute__((visibility("default"))) float ck_ref_gelu(float x)
+{
+    float y;
+    ck_tile::element_wise::Gelu{}(y, x);
     return y;
 }
 }

@@ -91,6 +91,9 @@ ck_ref_moe_gemm_gpu(int32_t kind, const int32_t* ids, const int32_t* eid, int32_
                     const uint16_t* B, uint16_t* C, const float* w, int32_t T, int32_t block, int32_t topk, int32_t M,
                     int32_t E, int32_t N, int32_t K, const float* sa, const float* sb)
 {
+    if(kind == 0)
+        return run_moe_gemm_gpu<0>(ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, T, (int64_t)T * topk, N,
+                                   sa, sb);
     if(kind == 1)
         return run_moe_gemm_gpu<1>(ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, T, (int64_t)T * topk,
                                    N / 2, sa, sb);

@@ -141,8 +141,18 @@ ORACLE_API uint8_t moe_oracle_f32_to_e4m3(float f)
 }
 
 static inline float silu_f32(float x) { return x * (1.0f / (1.0f + expf(-x))); }
+/* ck_tile::element_wise::Gelu, the exact (erf) form: unary_element_wise_operation.hpp:975-986.  Its host
+ * expression `0.5f * x * (1.f + erf(float(0.70710678118f * x)))` picks the double erf, so the sum and the last
+ * product are evaluated in double and rounded to float once */
+static inline float gelu_f32(float x)
+{
+    return (float)((double)(0.5f * x) * (1.0 + erf((double)(0.70710678118f * x))));
+}
+/* activation codes of fused_moe_traits: 0 = gelu, 1 = silu */
+static inline float act_f32(float x, int activation) { return activation == 0 ? gelu_f32(x) : silu_f32(x); }
 
 ORACLE_API float moe_oracle_silu(float x) { return silu_f32(x); }
+ORACLE_API float moe_oracle_gelu(float x) { return gelu_f32(x); }
 
 /* -------------------------------------------------------------------------- quantisation */
 
@@ -372,7 +382,7 @@ ORACLE_API int moe_oracle_fused_moe(const void* a, int a_dt, const float* a_scal
                                     const int32_t* sorted_expert_ids, int32_t post_pad,
                                     int32_t block_m, int32_t tokens, int32_t experts,
                                     int32_t hidden, int32_t inter, int32_t topk, int32_t gate_only,
-                                    int32_t strict, float* out_topk)
+                                    int32_t strict, float* out_topk, int32_t activation)
 {
     (void)experts;
     const int64_t n0       = (int64_t)inter * (gate_only ? 1 : 2);
@@ -430,10 +440,10 @@ ORACLE_API int moe_oracle_fused_moe(const void* a, int a_dt, const float* a_scal
                     acc0[n] = dot_f32(x, gw + n * hidden, hidden, strict);
                 if(gate_only)
                     for(int64_t n = 0; n < inter; n++)
-                        y[n] = silu_f32(acc0[n]);
+                        y[n] = act_f32(acc0[n], activation);
                 else
                     for(int64_t n = 0; n < inter; n++) /* :156-161 */
-                        y[n] = silu_f32(acc0[n]) * acc0[n + inter];
+                        y[n] = act_f32(acc0[n], activation) * acc0[n + inter];
                 float* dst = part + ((int64_t)token * topk + slot) * hidden;
                 for(int64_t h = 0; h < hidden; h++) /* second gemm :166-174 */
                     dst[h] = dot_f32(y, dw + h * inter, inter, strict) * w;
@@ -473,6 +483,7 @@ ORACLE_API int moe_oracle_fused_moe(const void* a, int a_dt, const float* a_scal
  * (scale_a, may be NULL) and per output channel (scale_b [experts, N], may be NULL), no expert bias.
  *   kind 1 (gate+up): row r of the sorted list with token t, slot s: A row t, C row t*topk+s,
  *       C[., n] = bf16( silu(acc_gate) * acc_up ), gate = B rows [0, N/2), up = B rows [N/2, N)
+ *   kind 0 (gate only): the same rows, C[., n] = bf16( silu(acc) ) over all N rows of B (:216-219 with up = 1)
  *   kind 2 (down)   : A row t*topk+s, C row t; ck_tile adds bf16(acc * w[r]) to C with packed bf16 atomics
  *       (:214-238).  Here a token's slots are summed in fp32 in slot order on top of the bf16 value C holds
  *       and rounded once: the same quantity without the order-dependent bf16 rounding of every partial sum.
@@ -482,7 +493,7 @@ ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const in
                                    uint16_t* C, int32_t num_tokens, int32_t topk, int32_t N, int32_t K, int32_t stride_a,
                                    int32_t stride_c, const float* scale_a, const float* scale_b)
 {
-    if(kind != 1 && kind != 2)
+    if(kind < 0 || kind > 2)
         return -1;
     const int32_t pn = kind == 1 ? N / 2 : N;
     float* acc2      = NULL; /* kind 2: fp32 sums [tokens, N], started from C */
@@ -525,6 +536,8 @@ ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const in
                     up *= sa * (scale_b ? scale_b[e * N + n + pn] : 1.0f);
                     C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(silu_f32(acc) * up);
                 }
+                else if(kind == 0)
+                    C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(silu_f32(acc));
                 else
                     acc2[c_row * N + n] += acc * sorted_w[r];
             }

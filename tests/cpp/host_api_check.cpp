@@ -14,7 +14,7 @@ int moe_oracle_sorting(const int32_t*, const float*, const int32_t*, int32_t, in
                        int32_t*, float*, int32_t*, int32_t*);
 int moe_oracle_fused_moe(const void*, int, const float*, const void*, int, const float*, const void*, int,
                          const float*, void*, int, const int32_t*, const float*, const int32_t*, int32_t, int32_t,
-                         int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, float*);
+                         int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, float*, int32_t);
 uint16_t moe_oracle_f32_to_bf16(float);
 float moe_oracle_bf16_to_f32(uint16_t);
 }
@@ -69,7 +69,7 @@ int main()
     moe_oracle_sorting(ids.data(), w.data(), nullptr, T, K, E, U, 1, s_ids.data(), s_w.data(), s_eid.data(), &post_pad);
     std::vector<uint16_t> o_ref(T * H);
     moe_oracle_fused_moe(a.data(), 1, nullptr, g.data(), 1, nullptr, d.data(), 1, nullptr, o_ref.data(), 1, s_ids.data(),
-                         s_w.data(), s_eid.data(), post_pad, U, T, E, H, I, K, 0, 0, nullptr);
+                         s_w.data(), s_eid.data(), post_pad, U, T, E, H, I, K, 0, 0, nullptr, /*activation: silu*/ 1);
 
     // device path through the C++ API
     mi355::fused_moe_traits traits; // bf16, silu, block_m 32

@@ -39,11 +39,11 @@ def run_sorting(topk_ids, weights, experts, unit, mask=None, local_tokens=None, 
     return ids.cpu().numpy(), w.cpu().numpy(), eid.cpu().numpy(), total.cpu().numpy()
 
 
-def run_fused_moe(cfg, inp, mask=None, unfused=False, stride_pad=0):
+def run_fused_moe(cfg, inp, mask=None, unfused=False, stride_pad=0, activation=1, gate_only=0):
     """Runs mi355_fused_moe (or sorting + mi355_fused_moegemm) on numpy inputs of
     therock_amd.inputs.make_inputs_np.  Returns (out bf16 bits [T,H] numpy, buffers)."""
     traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit,
-                                 local_expert_masking=mask is not None)
+                                 local_expert_masking=mask is not None, activation=activation, gate_only=gate_only)
     buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, "cuda")
     view = TORCH_DT[cfg.dtype]
     a = dev(inp["a"]).view(view)

@@ -17,12 +17,12 @@ DT = {"bf16": oracle.DT_BF16, "fp8": oracle.DT_E4M3, "int8": oracle.DT_I8}
 TOL = {"bf16": 1e-2, "fp8": 3e-2, "int8": 3e-2}
 
 
-def oracle_out(cfg, inp, mask=None):
+def oracle_out(cfg, inp, mask=None, activation=1, gate_only=0):
     s = oracle.moe_sorting(inp["topk_ids"], inp["topk_weight"], cfg.experts, cfg.unit, local_expert_mask=mask)
     dt = DT[cfg.dtype]
     o = oracle.fused_moe(inp["a"], dt, inp["g"], dt, inp["d"], dt, *s, cfg.unit, cfg.tokens, inp["g"].shape[0],
                          cfg.hidden, cfg.inter, cfg.topk, a_scale=inp["a_scale"], g_scale=inp["g_scale"],
-                         d_scale=inp["d_scale"])
+                         d_scale=inp["d_scale"], activation=activation, gate_only=bool(gate_only))
     return oracle.bf16_to_f32(o), s
 
 
@@ -34,9 +34,13 @@ def check(cfg, seed=0, mask=None, **kw):
         for k in ("g", "d", "g_scale", "d_scale"):
             if inp[k] is not None:
                 inp[k] = inp[k][:nloc]
+    if kw.get("gate_only"):  # G holds the gate rows only
+        inp["g"] = np.ascontiguousarray(inp["g"][:, :cfg.inter])
+        if inp["g_scale"] is not None:
+            inp["g_scale"] = np.ascontiguousarray(inp["g_scale"][:, :cfg.inter])
     print(f"fused_moe {cfg} seed={seed} mask={mask is not None} {kw}", flush=True)
     got, buf = run_fused_moe(cfg, inp, mask=mask, **kw)
-    ref, s = oracle_out(cfg, inp, mask)
+    ref, s = oracle_out(cfg, inp, mask, kw.get("activation", 1), kw.get("gate_only", 0))
     pp = s[3]
     assert int(buf.total[0]) == pp
     assert np.array_equal(buf.sorted_ids[:pp].cpu().numpy(), s[0][:pp])
@@ -121,10 +125,23 @@ def test_decode_kernel_ragged(dtype):
     check(mi.MoeConfig("d", 40, 2080, 640, 64, 8, dtype, "sigmoid_renorm", unit=16), seed=3)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
+@pytest.mark.parametrize("activation,gate_only", [(0, 0), (1, 1), (0, 1)])
+def test_gelu_and_gate_only(dtype, activation, gate_only):
+    # the other activation of fused_moe_traits (gelu, erf form) and gate-only weights ([e, inter, hidden],
+    # y = act(gate)), through each of the three GEMM kernels: small tiles, decode tiles, 320-row tiles
+    kw = dict(activation=activation, gate_only=gate_only)
+    inter = 384 if dtype == "fp8" else 416  # not a multiple of the 256 columns a gate-only tile covers
+    check(mi.MoeConfig("a", 77, 320, inter, 12, 3, dtype, "softmax_renorm"), seed=3, **kw)
+    check(mi.MoeConfig("a", 24, 1056, 384 if dtype == "fp8" else 288, 16, 4, dtype, "softmax_renorm"), seed=1, **kw)
+    check(mi.MoeConfig("a", 700, 256, 384, 3, 2, dtype, "softmax_renorm"), seed=2, **kw)
+    check(mi.MoeConfig("a", 96, 256, 256, 10, 3, dtype, "softmax_renorm"), seed=4, unfused=True, **kw)
+
+
 def test_traits_without_kernel_return_minus_one():
     import torch
     import therock_amd as ta
-    for kw in (dict(prec_i="fp16", prec_w="fp16"), dict(activation=0), dict(gate_only=1), dict(prec_o="fp32")):
+    for kw in (dict(prec_i="fp16", prec_w="fp16"), dict(activation=2), dict(gate_only=2), dict(prec_o="fp32")):
         assert ta.fused_moe(ta.fused_moe_traits(**kw), ta.fused_moe_args()) == -1.0
     t = ta.fused_moe_traits()
     buf = ta.MoeBuffers(t, 4, 4, 2, 128, 128, "cuda")

@@ -65,6 +65,18 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     assert np.isnan(yg[T * K:]).all() and not np.isnan(yg[:T * K]).any()
     assert _rel(yg[:T * K], oracle.to_f32(y_ref, oracle.DT_BF16)) <= tol
 
+    # gate only: the gate half of the same weights on their own, c = silu(a b^T)
+    g_only = g[:, :I].contiguous()
+    yo = torch.full((T * K + 3, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert ta.moe_flatmm(ta.GEMM1_GATE_ONLY, x, g_only, yo, d_ids, d_eid, d_tot, T, K, unit, scale_m=d_sa,
+                         scale_n=None if d_sg is None else d_sg[:, :I].contiguous()) == 0.0
+    torch.cuda.synchronize()
+    yo_ref = oracle.moe_gemm(0, s_ids, s_eid, s_w, pp, unit, xr, np.ascontiguousarray(gr[:, :I]),
+                             np.zeros((T * K, I), np.uint16), T, K, sa, None if sg is None else np.ascontiguousarray(sg[:, :I]))
+    yog = yo.float().cpu().numpy()
+    assert np.isnan(yog[T * K:]).all() and not np.isnan(yog[:T * K]).any()
+    assert _rel(yog[:T * K], oracle.to_f32(yo_ref, oracle.DT_BF16)) <= tol
+
     # down: added to what c holds; a takes the reference's bf16 Y so that the two GEMMs are checked apart
     y_in = torch.from_numpy(y_ref.view(np.int16)).cuda().view(torch.bfloat16)
     c0 = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
@@ -82,8 +94,8 @@ def test_unsupported_and_errors():
 
     z = lambda *s, dt=torch.bfloat16: torch.zeros(s, dtype=dt, device="cuda")
     ids, eid, tot = z(64, dt=torch.int32), z(2, dt=torch.int32), z(2, dt=torch.int32)
-    # gate-only and fp8 have no stand-alone kernel: -1 like ck_tile's dispatcher
-    assert ta.moe_flatmm(0, z(4, 64), z(2, 128, 64), z(8, 64), ids, eid, tot, 4, 2, 32) == -1.0
+    # an unknown kind has no kernel: -1 like ck_tile's dispatcher
+    assert ta.moe_flatmm(3, z(4, 64), z(2, 128, 64), z(8, 64), ids, eid, tot, 4, 2, 32) == -1.0
     with pytest.raises(RuntimeError):
         ta.moe_flatmm(ta.GEMM2, z(8, 64), z(2, 64, 64), z(4, 64), ids, eid, tot, 4, 2, 32)  # no sorted weights
 
@@ -110,6 +122,13 @@ def test_oracle_against_ck_tile_device_reference(T, E, K, H, I, unit):
     y_ck = oracle.ck_moe_gemm_gpu(1, s_ids, s_eid, s_w, pp, unit, x, g, np.zeros((T * K, I), np.uint16), T, K, sa, sg)
     y_or = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, f32(x), f32(g), np.zeros((T * K, I), np.uint16), T, K, sa, sg)
     diff = np.abs(y_ck.astype(np.int32) - y_or.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 0.01
+
+    g1 = np.ascontiguousarray(g[:, :I])
+    s1 = np.ascontiguousarray(sg[:, :I])
+    z_ck = oracle.ck_moe_gemm_gpu(0, s_ids, s_eid, s_w, pp, unit, x, g1, np.zeros((T * K, I), np.uint16), T, K, sa, s1)
+    z_or = oracle.moe_gemm(0, s_ids, s_eid, s_w, pp, unit, f32(x), f32(g1), np.zeros((T * K, I), np.uint16), T, K, sa, s1)
+    diff = np.abs(z_ck.astype(np.int32) - z_or.astype(np.int32))
     assert diff.max() <= 1 and (diff != 0).mean() < 0.01
 
     c0 = bf(rng.standard_normal((T, H)) * 0.1)

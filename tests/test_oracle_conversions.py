@@ -80,6 +80,23 @@ def test_silu_closed_form_and_special_cases():
         assert l.moe_oracle_silu(float(x)) == pytest.approx(x / (1.0 + math.exp(-x)), rel=2e-6, abs=1e-9)
 
 
+def test_gelu_closed_form_and_special_cases():
+    from scipy.special import erf
+    l = oracle.lib()
+    assert l.moe_oracle_gelu(0.0) == 0.0
+    assert l.moe_oracle_gelu(20.0) == 20.0
+    assert l.moe_oracle_gelu(-20.0) == 0.0
+    for x in np.linspace(-6, 6, 97):
+        x = float(np.float32(x))
+        # x * Phi(x) in float64; and gelu(x) - gelu(-x) = x
+        assert l.moe_oracle_gelu(x) == pytest.approx(0.5 * x * (1.0 + erf(x / math.sqrt(2.0))), rel=3e-6, abs=1e-7)
+        assert l.moe_oracle_gelu(x) - l.moe_oracle_gelu(-x) == pytest.approx(x, rel=1e-6, abs=1e-7)
+    xs = torch.linspace(-5, 5, 1001)
+    want = torch.nn.functional.gelu(xs).numpy()
+    got = np.array([l.moe_oracle_gelu(float(v)) for v in xs.numpy()], dtype=np.float32)
+    assert np.allclose(got, want, rtol=2e-6, atol=1e-6)  # torch evaluates 1 + erf in fp32 (cancellation in the left tail)
+
+
 def test_rowwise_quant_matches_definition():
     rng = np.random.default_rng(3)
     x = (rng.standard_normal((9, 160)) * np.array([1e-3, 0.1, 1, 3, 10, 50, 0, 1, 1])[:, None]).astype(np.float32)
@@ -139,6 +156,7 @@ def test_conversions_match_ck_tile():
         assert r.ck_ref_f32_to_fp8(v) == l.moe_oracle_f32_to_e4m3(v)
         assert r.ck_ref_f32_to_bf16(v) == l.moe_oracle_f32_to_bf16(v)
         assert r.ck_ref_silu(v) == l.moe_oracle_silu(v)
+        assert r.ck_ref_gelu(v) == l.moe_oracle_gelu(v)
 
 
 @pytest.mark.parametrize("dtype,nw,kw,kv", [(np.uint16, 16, 4, 8), (np.uint8, 16, 4, 16), (np.uint16, 32, 2, 8), (np.int8, 32, 2, 16)])

@@ -86,6 +86,18 @@ def test_small_quantised_matches_golden_ck_output(key, golden_dir):
     assert np.array_equal(run_oracle(cfg, inp, strict=True), g[f"{key}_out_bf16"])
 
 
+@pytest.mark.parametrize("name", ["gelu", "silu_gate_only", "gelu_gate_only"])
+def test_activation_variants_match_golden_ck_output(name, golden_dir):
+    from tests.golden.make_golden import ACT_VARIANT_CFG as cfg, ACT_VARIANTS
+    g = np.load(os.path.join(golden_dir, "act_variants_ck_reference.npz"))
+    inp = mi.make_inputs_np(cfg, 11)
+    assert str(g["input_sha"]) == sha(inp["a"], inp["g"], inp["d"]), "input generator changed: regenerate tests/golden"
+    act, gate_only = ACT_VARIANTS[name]
+    if gate_only:
+        inp["g"] = np.ascontiguousarray(inp["g"][:, :cfg.inter])
+    assert np.array_equal(run_oracle(cfg, inp, strict=True, activation=act, gate_only=gate_only), g[name])
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 def test_matches_dense_float64_formulation(dtype):
     cfg = mi.MoeConfig("t", 37, 256, 192, 12, 3, dtype, "softmax_renorm", unit=16)
@@ -142,18 +154,25 @@ def test_tiny_triple_loop_and_partials():
 
 @pytest.mark.skipif(oracle.ck_ref() is None, reason="oracle/_ref not built")
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
-def test_bit_exact_with_ck_tile_reference(dtype):
+@pytest.mark.parametrize("activation,gate_only", [(1, False), (0, False), (1, True), (0, True)])
+def test_bit_exact_with_ck_tile_reference(dtype, activation, gate_only):
     cfg = mi.MoeConfig("t", 19, 128, 96, 6, 2, dtype, "softmax_renorm", unit=8)
     inp = mi.make_inputs_np(cfg, 11)
+    if gate_only:  # G holds the gate rows only
+        inp["g"] = np.ascontiguousarray(inp["g"][:, :cfg.inter])
+        if inp["g_scale"] is not None:
+            inp["g_scale"] = np.ascontiguousarray(inp["g_scale"][:, :cfg.inter])
     s = oracle.moe_sorting(inp["topk_ids"], inp["topk_weight"], cfg.experts, cfg.unit)
-    mine = run_oracle(cfg, inp, strict=True)
+    mine = run_oracle(cfg, inp, strict=True, activation=activation, gate_only=gate_only)
+    kw = dict(activation=activation, gate_only=gate_only)
     if dtype == "bf16":
         ck = oracle.ck_fused_moe(inp["a"], inp["g"], inp["d"], *s, cfg.unit, cfg.tokens, cfg.experts, cfg.hidden,
-                                 cfg.inter, cfg.topk)
+                                 cfg.inter, cfg.topk, **kw)
     else:
         dt = DT[dtype]
         ck = oracle.ck_fused_moe(oracle.to_f32(inp["a"], dt) * inp["a_scale"][:, None],
                                  oracle.to_f32(inp["g"], dt) * inp["g_scale"][:, :, None],
                                  oracle.to_f32(inp["d"], dt) * inp["d_scale"][:, :, None],
-                                 *s, cfg.unit, cfg.tokens, cfg.experts, cfg.hidden, cfg.inter, cfg.topk, f32_inputs=True)
+                                 *s, cfg.unit, cfg.tokens, cfg.experts, cfg.hidden, cfg.inter, cfg.topk, f32_inputs=True,
+                                 **kw)
     assert np.array_equal(mine, ck)

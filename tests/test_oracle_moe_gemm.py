@@ -33,6 +33,13 @@ def test_against_dense_float64(T, E, K, H, I, unit):
             e = ids[t, k]
             ref = _silu(x[t].astype(np.float64) @ g[e, :I].T.astype(np.float64)) * (x[t].astype(np.float64) @ g[e, I:].T)
             np.testing.assert_allclose(yf[t * K + k], ref, rtol=1.2e-2, atol=1e-6)  # one bf16 rounding
+    # gate only: silu(a b^T) over all rows of b; with b = the full gate+up matrix its first half is the gate part
+    z = oracle.to_f32(oracle.moe_gemm(0, s_ids, s_eid, s_w, pp, unit, x, g, np.zeros((T * K, 2 * I), np.uint16), T, K),
+                      oracle.DT_BF16)
+    for t in range(T):
+        for k in range(K):
+            ref = _silu(x[t].astype(np.float64) @ g[ids[t, k]].T.astype(np.float64))
+            np.testing.assert_allclose(z[t * K + k], ref, rtol=1.2e-2, atol=1e-6)
     c0 = oracle.f32_to_bf16(np.full((T, H), 0.25, np.float32))
     o = oracle.to_f32(oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, yf, d, c0.copy(), T, K), oracle.DT_BF16)
     for t in range(T):

@@ -100,7 +100,8 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
 
     const int wchunk = tid % kWChunks;
     const int wrow   = tid / kWChunks; // + kWRowsPerPass*j  (row of the LDS weight tile)
-    const int n_base = nt * (GEMM0 ? 128 : 256);
+    const bool paired = GEMM0 && !p.gate_only; // gate rows paired with up rows (see run_epilogue)
+    const int n_base  = nt * (paired ? 128 : 256);
     const unsigned char* wbase = p.w + (int64_t)expert * p.w_expert_bytes + wchunk * 16;
     int64_t woff[kWLoads];
 #pragma unroll
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
         const int blk  = lrow >> 5;
         const int c    = chan_of_row(lrow & 31);
         int grow;
-        if constexpr(GEMM0)
+        if(paired)
         {
             const int col = min(n_base + (blk >> 1) * 32 + c, p.n_out - 1);
             grow          = (blk & 1) * p.n_out + col;
@@ -532,10 +533,10 @@ int check_traits(const mi355_fused_moe_traits& t)
                     t.prec_o);
     if(t.prec_st != MI355_MOE_FP32 || t.prec_sw != MI355_MOE_FP32 || t.prec_kw != MI355_MOE_FP32)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: scales and top-k weights must be fp32");
-    if(t.activation != 1)
-        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: only activation=1 (silu) is implemented");
-    if(t.gate_only != 0)
-        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: gate_only is not implemented");
+    if(t.activation != 0 && t.activation != 1)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: activation=%d (0 = gelu, 1 = silu)", t.activation);
+    if(t.gate_only != 0 && t.gate_only != 1)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: gate_only=%d (0 or 1)", t.gate_only);
     if(t.fused_quant != 0)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: fused_quant=%d is not implemented", t.fused_quant);
     if(t.block_m < 1 || t.block_m > 1024)
@@ -656,18 +657,23 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.x_scale         = quant ? static_cast<const float*>(a.a_scale_ptr) : nullptr;
     p.w               = static_cast<const unsigned char*>(a.g_ptr);
     p.w_row_bytes     = (int64_t)H * eb;
-    p.w_expert_bytes  = (int64_t)2 * I * H * eb;
+    const int g_rows  = t.gate_only ? I : 2 * I; // weight rows per expert of the first GEMM
+    p.gate_only       = t.gate_only;
+    p.act             = t.activation;
+    p.w_expert_bytes  = (int64_t)g_rows * H * eb;
     p.w_scale         = quant ? static_cast<const float*>(a.g_scale_ptr) : nullptr;
     p.out             = wsb + ws.y_off;
     p.out_row_bytes   = (int64_t)I * y_b;
     p.k_bytes_x       = H * eb;
     p.k_bytes_w       = H * eb;
     p.n_out           = I;
-    p.n_total         = 2 * I;
+    p.n_total         = g_rows;
     // decode-sized problems (one 32-row block per tile) have their own kernel
     const bool decode = mblk == 1 && decode_supported((int64_t)T * a.stride_token * eb, ws.max_pad * (int64_t)I * y_b,
                                                       (int64_t)2 * I * H * eb);
-    p.n_ntiles        = decode ? ceil_div(I, decode_tile_cols(true)) : ceil_div(I, 128);
+    // Y columns per tile: the tile's weight rows, halved where gate and up rows share them
+    const int pair    = t.gate_only ? 1 : 2;
+    p.n_ntiles        = decode ? ceil_div(I, decode_tile_cols(false) / pair) : ceil_div(I, 256 / pair);
     if(mblk > 4 && (int64_t)T * p.x_row_bytes >= ((int64_t)1 << 32))
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: a token buffer of 4 GiB or more (stride_token=%d) is not "
                                              "supported at this problem size", a.stride_token);
@@ -690,6 +696,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.x              = wsb + ws.y_off;
     p.x_row_bytes    = (int64_t)I * y_b;
     p.x_scale        = nullptr;
+    p.gate_only      = 0;
     p.w              = static_cast<const unsigned char*>(a.d_ptr);
     p.w_row_bytes    = (int64_t)I * eb;
     p.w_expert_bytes = (int64_t)H * I * eb;
@@ -799,9 +806,10 @@ struct FlatmmLayout
 
 int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
 {
-    if(kind != MI355_MOE_GEMM1_GATE_UP && kind != MI355_MOE_GEMM2)
-        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: kind %d (gate+up and down GEMMs are implemented)", kind);
-    const bool g1     = kind == MI355_MOE_GEMM1_GATE_UP;
+    if(kind != MI355_MOE_GEMM1_GATE_ONLY && kind != MI355_MOE_GEMM1_GATE_UP && kind != MI355_MOE_GEMM2)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: kind %d (0 = gate only, 1 = gate+up, 2 = down)", kind);
+    const bool g1     = kind != MI355_MOE_GEMM2;
+    const bool go     = kind == MI355_MOE_GEMM1_GATE_ONLY;
     const bool w8     = a.prec_b == MI355_MOE_INT8;
     const bool ok_typ = (a.prec_b == MI355_MOE_BF16 && a.prec_a == MI355_MOE_BF16) ||
                         (w8 && a.prec_a == (g1 ? MI355_MOE_INT8 : MI355_MOE_BF16));
@@ -809,11 +817,11 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: operand types a=%d b=%d (bf16 x bf16, int8 x int8 for the "
                                              "gate+up GEMM, bf16 x int8 for the down GEMM)", a.prec_a, a.prec_b);
     if(a.NumTokens < 0 || a.NumExperts <= 0 || a.NumExperts > 1024 || a.TopK <= 0 || a.TopK > 255 || a.N <= 0 || a.K <= 0 ||
-       a.block_m < 1 || a.block_m > 1024 || a.k_batch > 1 || (g1 && a.N % 2 != 0))
+       a.block_m < 1 || a.block_m > 1024 || a.k_batch > 1 || (g1 && !go && a.N % 2 != 0))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: bad sizes (tokens=%d experts=%d topk=%d N=%d K=%d block_m=%d k_batch=%d)",
                     a.NumTokens, a.NumExperts, a.TopK, a.N, a.K, a.block_m, a.k_batch);
     L.hidden = g1 ? a.K : a.N;
-    L.inter  = g1 ? a.N / 2 : a.K;
+    L.inter  = g1 ? (go ? a.N : a.N / 2) : a.K;
     if(L.hidden % 32 != 0 || L.inter % 32 != 0)
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: N and K must give hidden and intermediate sizes that are "
                                              "multiples of 32 (hidden=%d inter=%d)", L.hidden, L.inter);
@@ -848,7 +856,8 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
     int rc = flatmm_layout(kind, a, L);
     if(rc != MI355_MOE_OK)
         return rc;
-    const bool g1 = kind == MI355_MOE_GEMM1_GATE_UP;
+    const bool g1 = kind != MI355_MOE_GEMM2;
+    const bool go = kind == MI355_MOE_GEMM1_GATE_ONLY;
     const bool w8 = a.prec_b == MI355_MOE_INT8;
     if(!a.p_sorted_token_ids || !a.p_sorted_expert_ids || !a.p_max_token_id || !a.a_ptr || !a.b_ptr || !a.c_ptr ||
        (!g1 && !a.p_sorted_expert_weights))
@@ -898,6 +907,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
     p.tile_map       = tile_map;
     p.tokens         = T;
     p.slot_rows      = K;
+    p.act            = 1; // silu, the activation of ck_tile's MoeFlatmmKernel instances
     p.x              = static_cast<const unsigned char*>(a.a_ptr);
     p.x_row_bytes    = (int64_t)a.stride_A * a_b;
     p.w              = static_cast<const unsigned char*>(a.b_ptr);
@@ -915,9 +925,11 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
         p.x_scale       = w8 ? static_cast<const float*>(a.scale_m) : nullptr;
         p.out           = static_cast<unsigned char*>(a.c_ptr);
         p.out_row_bytes = (int64_t)a.stride_C * 2;
+        const int pair  = go ? 1 : 2; // gate and up rows share the tile's Y columns
+        p.gate_only     = go;
         p.n_out         = I;
-        p.n_total       = 2 * I;
-        p.n_ntiles      = decode ? ceil_div(I, decode_tile_cols(true)) : ceil_div(I, 128);
+        p.n_total       = a.N;
+        p.n_ntiles      = decode ? ceil_div(I, decode_tile_cols(false) / pair) : ceil_div(I, 256 / pair);
         if(decode)
             rc = launch_gemm_decode(prec, true, p, L.max_tiles, stream);
         else if(mblk > 4)

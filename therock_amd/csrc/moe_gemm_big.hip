@@ -117,7 +117,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     const int nt     = tile.nt;
     const int nrows  = tile.nrows;
     const int nmb    = ceil_div(nrows, 32);
-    const int n_base = nt * (GEMM0 ? 128 : 256);
+    const bool paired = GEMM0 && !p.gate_only; // gate rows paired with up rows (see run_epilogue)
+    const int n_base  = nt * (paired ? 128 : 256);
 
     // ---- DMA assignments.
     // Loads of one wave return in order, so a wave that mixed the two streams would see its L2-hit
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 const int c      = chan_of_row(trow & 31);
                 const int cchunk = (lane & 7) ^ ((rih >> 1) & 7);
                 int grow;
-                if constexpr(GEMM0)
+                if(paired)
                     grow = (blk & 1) * p.n_out + min(n_base + (blk >> 1) * 32 + c, p.n_out - 1);
                 else
                     grow = min(n_base + blk * 32 + c, p.n_total - 1);

@@ -39,7 +39,6 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
     constexpr int kWRowsPerPass = kBlock / (kDecWKB / 16);        // 8
     constexpr int kXRowsPerPass = kBlock / (kXKB / 16);
     constexpr bool kMx     = MODE == kFp8 && !GEMM0;
-    constexpr int kNTile   = GEMM0 ? 32 : 64;
 
     extern __shared__ __align__(16) unsigned char lds[];
     unsigned char* lds_w = lds;
@@ -59,7 +58,8 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
     const int row0   = tile.row0;
     const int nt     = tile.nt;
     const int nrows  = min(tile.nrows, 32);
-    const int n_base = nt * kNTile;
+    const bool paired = GEMM0 && !p.gate_only; // gate rows paired with up rows (see run_epilogue)
+    const int n_base  = nt * (paired ? 32 : 64);
 
     // ---- global -> register staging assignments: 32 consecutive lanes fetch 512 contiguous bytes
     const int xchunk = tid % (kXKB / 16);
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
         const int blk  = lrow >> 5;
         const int c    = chan_of_row(lrow & 31);
         int grow;
-        if constexpr(GEMM0)
+        if(paired)
             grow = blk * p.n_out + min(n_base + c, p.n_out - 1);
         else
             grow = min(n_base + blk * 32 + c, p.n_total - 1);
@@ -238,7 +238,9 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
     __syncthreads();
     if(wave > 0)
         return;
-#pragma unroll
+    // one wave's 32 values at a time: fetching all 96 at once does not fit the register budget of three
+    // workgroups per compute unit
+#pragma nounroll
     for(int w = 0; w < 3; w++)
 #pragma unroll
         for(int b = 0; b < 2; b++)

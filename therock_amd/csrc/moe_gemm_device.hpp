@@ -56,6 +56,10 @@ struct GemmParams
     // 16 rows x 64 B one token DMA instruction of the down GEMM fetches are 1 KiB of consecutive memory
     // (8 whole cache lines instead of 16 half lines)
     int y_slab;
+    // gemm0 variants of ck_tile's fused_moe_traits: gate_only = the weights hold gate rows only ([experts,
+    // n_out, k]; a tile then covers twice the Y columns and y = act(gate)); act: 0 = gelu (erf form), 1 = silu
+    int gate_only;
+    int act;
 };
 
 // byte offset of K byte kb of row `row` in the slab-major Y layout
@@ -140,6 +144,17 @@ struct ModeTraits<kBf16W8>
 __device__ __host__ constexpr int chan_of_row(int m) { return 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3); }
 
 __device__ inline float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+// Gelu in the erf form of ck_tile::element_wise::Gelu (unary_element_wise_operation.hpp:975-986):
+// x * Phi(x) with erfc(z) = poly(t) * exp(-z^2), t = 1 / (1 + 0.3275911 z) (Abramowitz & Stegun 7.1.26,
+// absolute error of erf <= 1.5e-7), branch-free and free of cancellation in the negative tail
+__device__ inline float gelu(float x)
+{
+    const float z = fabsf(x) * 0.70710678118f;
+    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
+    const float q = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f)))) *
+                    __expf(-z * z); // erfc(z)
+    return x >= 0.f ? x * (1.0f - 0.5f * q) : 0.5f * x * q;
+}
 
 // 8 int8 (two dwords) -> 8 bf16 (exact: |v| <= 128 fits bf16's 8 significant bits)
 __device__ inline uint4 int8x8_to_bf16x8(uint2 v)
@@ -250,19 +265,32 @@ __device__ inline void load_channel_scales(const float* scale, float (&out)[16])
 // gemm0: y = silu(gate) * up with the per-token scale sa and the per-channel scales folded in;
 // stored as bf16 or (fp8 path) as e4m3 with one power-of-two scale per 32 columns.  Every lane of
 // the wave must call it (the fp8 path exchanges the block maximum with lane ^ 32); `store` masks
-// the writes.
+// the writes.  single: gate-only weights, y = act(gate) and the up operands are ignored.
 template <int MODE>
 __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc_gate,
                                       const typename ModeTraits<MODE>::Acc& acc_up, const float (&gs)[16],
-                                      const float (&us)[16], float sa, int64_t grow, bool store, int col0, int kg)
+                                      const float (&us)[16], float sa, int64_t grow, bool store, int col0, int kg,
+                                      bool single = false)
 {
     float y[16];
-#pragma unroll
-    for(int v = 0; v < 16; v++)
+    // p.act is uniform: one scalar branch
+    if(p.act == 0)
     {
-        const float g = static_cast<float>(acc_gate[v]) * (sa * gs[v]);
-        const float u = static_cast<float>(acc_up[v]) * (sa * us[v]);
-        y[v]          = silu(g) * u;
+#pragma unroll
+        for(int v = 0; v < 16; v++)
+            y[v] = gelu(static_cast<float>(acc_gate[v]) * (sa * gs[v]));
+    }
+    else
+    {
+#pragma unroll
+        for(int v = 0; v < 16; v++)
+            y[v] = silu(static_cast<float>(acc_gate[v]) * (sa * gs[v]));
+    }
+    if(!single)
+    {
+#pragma unroll
+        for(int v = 0; v < 16; v++)
+            y[v] *= static_cast<float>(acc_up[v]) * (sa * us[v]);
     }
     constexpr int y_b  = MODE == kFp8 ? 1 : 2;
     unsigned char* dst = p.y_slab > 0 ? p.out + y_slab_offset(grow, col0 * y_b, p.y_slab)
@@ -344,16 +372,19 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
 {
     // ---- one batch of loads
     float sc0[16], sc1[16];
-    const int col_a = GEMM0 ? n_base + wblk * 32 + 16 * kg : n_base + (wblk * 2) * 32 + 16 * kg;
-    const int col_b = GEMM0 ? col_a : col_a + 32;
-    const bool a_ok = (GEMM0 ? n_base + wblk * 32 : n_base + wblk * 64) < p.n_out;
-    const bool b_ok = GEMM0 ? a_ok : (n_base + wblk * 64 + 32) < p.n_out;
+    // gate+up tiles pair weight block 2w (gate) with 2w+1 (up) on the same 32 columns; every other kind of
+    // tile (down, gate-only) maps its blocks 2w and 2w+1 to consecutive groups of 32 columns
+    const bool paired = GEMM0 && !p.gate_only;
+    const int col_a = paired ? n_base + wblk * 32 + 16 * kg : n_base + (wblk * 2) * 32 + 16 * kg;
+    const int col_b = paired ? col_a : col_a + 32;
+    const bool a_ok = (paired ? n_base + wblk * 32 : n_base + wblk * 64) < p.n_out;
+    const bool b_ok = paired ? a_ok : (n_base + wblk * 64 + 32) < p.n_out;
     const float* sbase = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total : nullptr;
     load_channel_scales(sbase && a_ok ? sbase + col_a : nullptr, sc0);
-    load_channel_scales(sbase && b_ok ? sbase + (GEMM0 ? p.n_out + col_a : col_b) : nullptr, sc1);
+    load_channel_scales(sbase && b_ok ? sbase + (paired ? p.n_out + col_a : col_b) : nullptr, sc1);
     float sa[NBLK];
     bool real[NBLK];
-    int64_t orow[NBLK]; // output row
+    int orow[NBLK]; // output row (the launchers keep tokens * topk below 2^31)
 #pragma unroll
     for(int i = 0; i < NBLK; i++)
     {
@@ -371,7 +402,7 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
                 if(p.x_scale != nullptr)
                     sa[i] = real[i] ? p.x_scale[tok] : 0.0f;
                 if(p.slot_rows > 0)
-                    orow[i] = real[i] ? slot_row(sid, p.slot_rows) : 0;
+                    orow[i] = real[i] ? (int)slot_row(sid, p.slot_rows) : 0;
             }
         }
     }
@@ -385,21 +416,31 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
     for(int i = 0; i < NBLK; i++)
         asm volatile("" : "+v"(sa[i]), "+v"(orow[i]));
     // ---- apply
-#pragma unroll
-    for(int i = 0; i < NBLK; i++)
+    if constexpr(GEMM0)
     {
-        if(i >= nblk_live)
-            continue;
-        const int r        = first_row + i * row_step + r32;
-        const bool in_tile = r < nrows;
-        if constexpr(GEMM0)
+        // block by block, so that a block's accumulators are dead before the next block's temporaries
+        // are needed (the large-tile kernel has no registers to spare)
+#pragma unroll
+        for(int i = 0; i < NBLK; i++)
         {
+            if(i >= nblk_live)
+                continue;
+            const bool st = first_row + i * row_step + r32 < nrows && (p.slot_rows == 0 || real[i]);
             if(a_ok)
-                epilogue_gemm0<MODE>(p, acc[i][0], acc[i][1], sc0, sc1, sa[i], orow[i],
-                                     in_tile && (p.slot_rows == 0 || real[i]), col_a, kg);
+                epilogue_gemm0<MODE>(p, acc[i][0], acc[i][1], sc0, sc1, sa[i], orow[i], st, col_a, kg, !paired);
+            if(!paired && b_ok) // gate-only tile: the second accumulator holds the next 32 gate columns
+                epilogue_gemm0<MODE>(p, acc[i][1], acc[i][1], sc1, sc1, sa[i], orow[i], st, col_b, kg, true);
         }
-        else
+    }
+    else
+    {
+#pragma unroll
+        for(int i = 0; i < NBLK; i++)
         {
+            if(i >= nblk_live)
+                continue;
+            const int r        = first_row + i * row_step + r32;
+            const bool in_tile = r < nrows;
             if(a_ok)
                 epilogue_gemm1<MODE>(p, acc[i][0], sc0, row0 + r, in_tile && real[i], col_a);
             if(b_ok)

@@ -203,14 +203,14 @@ def rowwise_quant(x, q_dtype: str, stream=None):
     return q, scale
 
 
-GEMM1_GATE_UP, GEMM2 = 1, 2
+GEMM1_GATE_ONLY, GEMM1_GATE_UP, GEMM2 = 0, 1, 2
 
 
 def moe_flatmm(kind: int, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens: int, topk: int, block_m: int,
                sorted_weights=None, scale_m=None, scale_n=None, stream=None):
     """One grouped GEMM of the MoE layer as its own launch (ck_tile's MoeFlatmm conventions): kind
-    GEMM1_GATE_UP writes c[token * topk + slot, :N/2] = silu(gate) * up, kind GEMM2 adds the weighted
-    down projection of a[token * topk + slot] to c[token].  b is [experts, N, K]."""
+    GEMM1_GATE_UP writes c[token * topk + slot, :N/2] = silu(gate) * up, GEMM1_GATE_ONLY c[.., :N] = silu(a b^T),
+    kind GEMM2 adds the weighted down projection of a[token * topk + slot] to c[token].  b is [experts, N, K]."""
     import torch
 
     experts, n, k = b.shape
@@ -315,5 +315,5 @@ def make_args(traits: fused_moe_traits, buf: MoeBuffers, a, g, d, topk_ids, topk
         local_expert_mask_ptr=local_expert_mask, o_ptr=buf.out, ws_ptr=buf.ws, topk_ids_ptr=topk_ids,
         topk_weight_ptr=topk_weight, sorted_token_ids_ptr=buf.sorted_ids, sorted_weight_ptr=buf.sorted_w,
         sorted_expert_ids_ptr=buf.sorted_eid, num_sorted_tiles_ptr=buf.total, block_m=traits.block_m,
-        hidden_size=H, intermediate_size=n0 // 2, num_tokens=T, num_experts=E, topk=topk_ids.shape[1],
+        hidden_size=H, intermediate_size=n0 if traits.gate_only else n0 // 2, num_tokens=T, num_experts=E, topk=topk_ids.shape[1],
         stride_token=a.stride(0))
