@@ -368,19 +368,39 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
             acc[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
         }
     }
-    for(int k = 0; k < topk; k++)
+    // four slots at a time (eight measured the same): their rows are fetched together (read once: non-temporal), then added in slot order
+    constexpr int kSlotsPerPass = 4;
+    using u32x4 = __attribute__((ext_vector_type(4))) uint32_t;
+    for(int k0 = 0; k0 < topk; k0 += kSlotsPerPass)
     {
-        const int pos = inv[t * topk + k];
-        if(pos < 0)
-            continue;
-        const float w = sorted_w[pos];
-        const uint4 v = *reinterpret_cast<const uint4*>(part + ((int64_t)pos * hidden + h0) * 2);
-        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+        int pos[kSlotsPerPass];
+        float w[kSlotsPerPass];
+        u32x4 v[kSlotsPerPass];
 #pragma unroll
-        for(int i = 0; i < 4; i++)
+        for(int j = 0; j < kSlotsPerPass; j++)
+            pos[j] = k0 + j < topk ? __builtin_amdgcn_readfirstlane(inv[t * topk + k0 + j]) : -1;
+#pragma unroll
+        for(int j = 0; j < kSlotsPerPass; j++)
         {
-            acc[2 * i] += w * __uint_as_float(d[i] << 16);
-            acc[2 * i + 1] += w * __uint_as_float(d[i] & 0xffff0000u);
+            w[j] = 0.f;
+            v[j] = u32x4{0u, 0u, 0u, 0u};
+            if(pos[j] >= 0)
+            {
+                w[j] = sorted_w[pos[j]];
+                v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(part + ((int64_t)pos[j] * hidden + h0) * 2));
+            }
+        }
+#pragma unroll
+        for(int j = 0; j < kSlotsPerPass; j++)
+        {
+            if(pos[j] < 0)
+                continue;
+#pragma unroll
+            for(int i = 0; i < 4; i++)
+            {
+                acc[2 * i] += w[j] * __uint_as_float(v[j][i] << 16);
+                acc[2 * i + 1] += w[j] * __uint_as_float(v[j][i] & 0xffff0000u);
+            }
         }
     }
     uint4 o;
