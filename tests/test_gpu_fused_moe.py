@@ -125,6 +125,19 @@ def test_decode_kernel_ragged(dtype):
     check(mi.MoeConfig("d", 40, 2080, 640, 64, 8, dtype, "sigmoid_renorm", unit=16), seed=3)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+def test_large_tile_kernel_partial_tiles(dtype):
+    # from about 28 rows per expert on, and with enough tiles to fill the chip, the 320-row kernel runs with
+    # mostly empty tiles: it then fetches only the 64-row slab groups a tile has (1 to 5 per step)
+    import therock_amd as ta
+    for cfg, seed in ((mi.MoeConfig("p", 640, 256, 512, 64, 4, dtype, "softmax_renorm"), 1),
+                      (mi.MoeConfig("p", 1500, 256, 512, 64, 4, dtype, "zipf"), 2),
+                      (mi.MoeConfig("p", 4000, 384, 512, 64, 6, dtype, "zipf", unit=64), 3)):
+        traits = ta.fused_moe_traits(prec_i=dtype, prec_w=dtype, block_m=cfg.unit)
+        assert ta.fused_moe_tile_rows(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter) == 320
+        check(cfg, seed=seed)
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 @pytest.mark.parametrize("activation,gate_only", [(0, 0), (1, 1), (0, 1)])
 def test_gelu_and_gate_only(dtype, activation, gate_only):

@@ -503,18 +503,23 @@ __global__ __launch_bounds__(256) void moe_smoothquant_kernel(const uint16_t* __
 inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
 {
     const int64_t avg = tokens * topk / experts;
-    if(avg <= 32)
-        return 1;
-    if(avg <= 64)
-        return 2;
     const int eb  = t.prec_i == MI355_MOE_BF16 ? 2 : 1;
     const int y_b = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
     // the large-tile kernel addresses each operand as a base plus a 32-bit byte offset
     const int64_t lim     = (int64_t)1 << 32;
     const int64_t max_pad = topk * tokens + (int64_t)experts * t.block_m - topk;
     const bool fits = (int64_t)2 * inter * hidden * eb < lim && max_pad * inter * y_b < lim && tokens * hidden * eb < lim;
-    if(avg >= 160 && t.block_m % 4 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b))
+    // Measured crossovers (fp8, 256 experts; bf16, 8 experts): the decode kernel wins up to about 24 rows per
+    // expert, the large-tile kernel from about 28 on - it streams every weight tile once whatever the row
+    // count and fetches only the token slabs a tile has - provided its tiles fill the chip.
+    const int64_t big_tiles = (int64_t)experts * std::max<int64_t>(1, ceil_div<int64_t>(avg, big_tile_rows())) * ceil_div(inter, 128);
+    const bool big_ok = t.block_m % 4 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b);
+    if(big_ok && (avg >= 160 || (avg >= 28 && big_tiles >= device_info().num_cu)))
         return big_tile_rows() / 32;
+    if(avg <= 32)
+        return 1;
+    if(avg <= 64)
+        return 2;
     return 4;
 }
 

@@ -126,8 +126,10 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     // waves: waves 0..3 the weights, waves 4..7 the tokens (and, on the fp8 down-GEMM, the e8m0 scales).
     // Weights: unit u = rows (u & 1) * 128 .. + 127 of the tile, K bytes [128 * (u >> 1), + 128).  One unit
     // is 16 instructions of 8 rows x 128 B (full cache lines); wave w issues instructions w, w+4, w+8, w+12.
-    // Tokens: step x = all 320 rows, K bytes [64 x, + 64), 20 slabs of 16 rows x 64 B; wave 4+q fills slabs
-    // q, q+4, .. q+16 and fetches 256 scale bytes.
+    // Tokens: step x = the tile's rows, K bytes [64 x, + 64), up to 20 slabs of 16 rows x 64 B; wave 4+q fills
+    // slabs q, q+4, .. as far as the tile has rows (one instruction per 64 rows of the tile) and fetches 256
+    // scale bytes.  The count is a template argument of the K loop: selecting the instructions and the
+    // matching wait with scalar branches inside the loop cost 5 % of the kernel's time.
     // Every source address is a wave-uniform base (operand base + K offset of the unit, kept in
     // scalar registers) plus a per-lane 32-bit row offset doff[] that never changes: weights
     // doff[4 * half + j]; tokens doff[0..4], scales doff[5].  Token rows that do not exist (padding
@@ -202,20 +204,24 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             dma16(src, doff[H * 4 + j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));
     };
     // token role: step x -> ring stage x % 3
-    auto issue_x = [&](int x) __attribute__((always_inline)) {
+    auto issue_x = [&](int x, int groups) __attribute__((always_inline)) {
         if(x >= kt_count)
             return;
         const uint32_t sbase     = lds_base + kXOffset + (x % kXStages) * kXStageBytes + q4 * 1024;
         const unsigned char* src = dbase + x * x_step;
 #pragma unroll
         for(int j = 0; j < 5; j++)
-            dma16(src, doff[j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));
+            if(j < groups)
+                dma16(src, doff[j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));
         if constexpr(kMx)
             dma4(p.y_scale + x * ys_step, doff[5],
                  __builtin_amdgcn_readfirstlane(lds_base + kYsOffset + (x % kXStages) * kYsStageBytes +
                                                 (q4 >> 1) * kYsRows + (q4 & 1) * 256));
     };
-    constexpr int kXInstr = kMx ? 6 : 5; // token-role DMA instructions per step
+
+    // token blocks of this wave (blocks wt, wt + 2, ..) and 64-row slab groups that hold rows of the tile
+    const int nb_w     = __builtin_amdgcn_readfirstlane(max(0, min(kMaxNB, (nmb - wt + 1) / 2)));
+    const int x_groups = __builtin_amdgcn_readfirstlane(max(1, (nmb + 1) / 2));
 
     Acc acc[kMaxNB][2];
 #pragma unroll
@@ -238,8 +244,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     }
     else
     {
-        issue_x(0);
-        issue_x(1);
+        issue_x(0, x_groups);
+        issue_x(1, x_groups);
     }
 
     // per-lane LDS read offsets (swizzled chunk positions are per-lane constants)
@@ -249,8 +255,10 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     const int w_h   = ww >> 1;
     const int x_off = kXOffset + (wt * 32 + r32) * kStepKB;
 
-    auto k_loop = [&](auto nb_tag) {
+    // NB: token blocks of this wave; XG: slab groups a token-role wave issues per step (0 in a weight-role wave)
+    auto k_loop = [&](auto nb_tag, auto xg_tag) {
         constexpr int NB = decltype(nb_tag)::value;
+        constexpr int XG = decltype(xg_tag)::value;
         constexpr int NF = NB > 0 ? NB : 1;
         // one compute step; PAR = k & 1
         auto step = [&](int k, auto par_tag) __attribute__((always_inline)) {
@@ -262,7 +270,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 if(w_role)
                     wait_vmcnt<PAR ? 12 : 8>();
                 else
-                    wait_vmcnt<kXInstr>();
+                    wait_vmcnt<XG + (kMx ? 1 : 0)>(); // token-role instructions of one step
             }
             else
                 wait_vmcnt<0>();
@@ -275,7 +283,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             if(w_role)
                 issue_w(k + 4, par_tag);
             else
-                issue_x(k + 2);
+                issue_x(k + 2, XG);
 
             const unsigned char* wst = lds + (((k & ~1) + w_h) % kWSlots) * kWUnitBytes + w_off;
             const unsigned char* xst = lds + x_off + (k % kXStages) * kXStageBytes;
@@ -333,15 +341,26 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             step(k + 1, H1{});
         }
     };
-    const int nb_w = max(0, min(kMaxNB, (nmb - wt + 1) / 2));
+    // weight-role waves own blocks 0, 2, .. (ceil(nmb / 2) of them), token-role waves blocks 1, 3, ..
+    // (floor(nmb / 2)) and issue ceil(nmb / 2) slab groups: the same count, or one more when nmb is odd
+    using I0 = std::integral_constant<int, 0>;
+    auto run = [&](auto nb_tag) {
+        constexpr int NB = decltype(nb_tag)::value;
+        if(w_role)
+            k_loop(nb_tag, I0{});
+        else if(x_groups == NB)
+            k_loop(nb_tag, std::integral_constant<int, (NB > 0 ? NB : 1)>{});
+        else
+            k_loop(nb_tag, std::integral_constant<int, (NB < kMaxNB ? NB + 1 : kMaxNB)>{});
+    };
     switch(nb_w)
     {
-    case 5: k_loop(std::integral_constant<int, 5>{}); break;
-    case 4: k_loop(std::integral_constant<int, 4>{}); break;
-    case 3: k_loop(std::integral_constant<int, 3>{}); break;
-    case 2: k_loop(std::integral_constant<int, 2>{}); break;
-    case 1: k_loop(std::integral_constant<int, 1>{}); break;
-    default: k_loop(std::integral_constant<int, 0>{}); break;
+    case 5: run(std::integral_constant<int, 5>{}); break;
+    case 4: run(std::integral_constant<int, 4>{}); break;
+    case 3: run(std::integral_constant<int, 3>{}); break;
+    case 2: run(std::integral_constant<int, 2>{}); break;
+    case 1: run(std::integral_constant<int, 1>{}); break;
+    default: run(std::integral_constant<int, 0>{}); break;
     }
 
     // ---- epilogue
