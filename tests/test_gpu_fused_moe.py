@@ -126,6 +126,18 @@ def test_decode_kernel_ragged(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+def test_many_rows_per_expert_with_small_sort_units(dtype):
+    # hundreds of rows per expert, but expert boundaries on multiples of 8 or 24 rows only: the 320-row kernel
+    # (whose tiles start on whole 16-row slabs of the intermediate buffer) must not be chosen for unit 8 or 24
+    import therock_amd as ta
+    for unit, rows in ((8, 128), (24, 128), (16, 320), (48, 320)):
+        cfg = mi.MoeConfig("u", 700, 256, 384, 3, 2, dtype, "softmax_renorm", unit=unit)
+        traits = ta.fused_moe_traits(prec_i=dtype, prec_w=dtype, block_m=unit)
+        assert ta.fused_moe_tile_rows(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter) == rows
+        check(cfg, seed=unit)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
 def test_large_tile_kernel_partial_tiles(dtype):
     # from about 28 rows per expert on, and with enough tiles to fill the chip, the 320-row kernel runs with
     # mostly empty tiles: it then fetches only the 64-row slab groups a tile has (1 to 5 per step)

@@ -513,7 +513,8 @@ inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, 
     // expert, the large-tile kernel from about 28 on - it streams every weight tile once whatever the row
     // count and fetches only the token slabs a tile has - provided its tiles fill the chip.
     const int64_t big_tiles = (int64_t)experts * std::max<int64_t>(1, ceil_div<int64_t>(avg, big_tile_rows())) * ceil_div(inter, 128);
-    const bool big_ok = t.block_m % 4 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b);
+    // (its tiles start on whole 16-row slabs of Y: the sort unit must be a multiple of 16)
+    const bool big_ok = t.block_m % 16 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b);
     if(big_ok && (avg >= 160 || (avg >= 28 && big_tiles >= device_info().num_cu)))
         return big_tile_rows() / 32;
     if(avg <= 32)
