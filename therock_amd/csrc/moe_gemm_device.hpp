@@ -80,6 +80,7 @@ __device__ inline int64_t slot_row(int sid, int topk)
 struct TileRef
 {
     int expert, row0, nrows, nt; // nt: column tile
+    int expert_tiles;            // row tiles of this expert (each of them re-reads the same weight tiles)
     bool ok;
 };
 __device__ inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_ntiles, int block)
@@ -98,6 +99,7 @@ __device__ inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_nt
     t.nt              = rel / max(b.x, 1);
     const int j       = rel - t.nt * b.x;
     t.expert          = a.x;
+    t.expert_tiles    = b.x;
     t.row0            = b.y + j * b.w;
     t.nrows           = min(b.w, b.z - j * b.w);
     return t;
