@@ -411,93 +411,6 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
     *reinterpret_cast<uint4*>(out + (int64_t)t * out_row_bytes + (int64_t)h0 * 2) = o;
 }
 
-// per-row dynamic quantisation bf16 -> e4m3 / int8
-template <bool FP8>
-__global__ __launch_bounds__(256) void rowwise_quant_kernel(const uint16_t* __restrict__ x, int cols,
-                                                             int64_t stride_x, unsigned char* __restrict__ q,
-                                                             float* __restrict__ scale)
-{
-    __shared__ float s_red[4];
-    const int64_t row  = blockIdx.x;
-    const uint16_t* xr = x + row * stride_x;
-    float amax         = 0.f;
-    for(int c = threadIdx.x; c < cols; c += 256)
-        amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c])));
-#pragma unroll
-    for(int d = 32; d > 0; d >>= 1)
-        amax = fmaxf(amax, __shfl_xor(amax, d));
-    if((threadIdx.x & 63) == 0)
-        s_red[threadIdx.x >> 6] = amax;
-    __syncthreads();
-    amax            = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    const float qmx = FP8 ? 448.0f : 127.0f;
-    const float s   = amax > 0.f ? amax / qmx : 1.0f;
-    if(threadIdx.x == 0)
-        scale[row] = s;
-    for(int c = threadIdx.x; c < cols; c += 256)
-    {
-        const float v = bf16_bits_to_float(xr[c]) / s;
-        if constexpr(FP8)
-        {
-            const float cl = fminf(fmaxf(v, -448.f), 448.f);
-            q[row * cols + c] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
-        }
-        else
-        {
-            // ck_tile's float -> int8 conversion is a static_cast: truncation toward zero
-            const float cl = fminf(fmaxf(v, -128.f), 127.f);
-            q[row * cols + c] = static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
-        }
-    }
-}
-
-// MoE smooth-quant: row (slot k, token t) = x[t, :] * smscale[expert(t, k), :], per-row dynamic quantisation
-template <bool FP8>
-__global__ __launch_bounds__(256) void moe_smoothquant_kernel(const uint16_t* __restrict__ x,
-                                                               const float* __restrict__ smscale,
-                                                               const int* __restrict__ topk_ids, int tokens, int hidden,
-                                                               int experts, int topk, int64_t x_stride, int64_t y_stride,
-                                                               unsigned char* __restrict__ qy, float* __restrict__ yscale)
-{
-    __shared__ float s_red[4];
-    const int t = blockIdx.x;
-    const int k = blockIdx.y;
-    int e       = topk_ids[(int64_t)t * topk + k];
-    e           = min(max(e, 0), experts - 1);
-    const uint16_t* xr = x + (int64_t)t * x_stride;
-    const float* sr    = smscale + (int64_t)e * hidden;
-    float amax         = 0.f;
-    for(int c = threadIdx.x; c < hidden; c += 256)
-        amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c]) * sr[c]));
-#pragma unroll
-    for(int d = 32; d > 0; d >>= 1)
-        amax = fmaxf(amax, __shfl_xor(amax, d));
-    if((threadIdx.x & 63) == 0)
-        s_red[threadIdx.x >> 6] = amax;
-    __syncthreads();
-    amax            = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    const float qmx = FP8 ? 448.0f : 127.0f;
-    const float ys  = amax / qmx;
-    const int64_t r = (int64_t)k * tokens + t;
-    if(threadIdx.x == 0)
-        yscale[r] = ys;
-    unsigned char* qr = qy + r * y_stride;
-    for(int c = threadIdx.x; c < hidden; c += 256)
-    {
-        const float v = (bf16_bits_to_float(xr[c]) * sr[c]) / ys;
-        if constexpr(FP8)
-        {
-            const float cl = fminf(fmaxf(v, -448.f), 448.f);
-            qr[c] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
-        }
-        else
-        {
-            const float cl = fminf(fmaxf(v, -128.f), 127.f);
-            qr[c] = static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
-        }
-    }
-}
-
 // 32-row blocks per M tile, from the expected rows per expert; big_tile_rows()/32 selects the
 // large-tile kernel
 inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
@@ -546,6 +459,32 @@ int launch_gemm(int mblk, const GemmParams& p, int max_tiles, hipStream_t stream
 #undef MI355_LAUNCH
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
+}
+
+// One grouped GEMM over the tile list: sets the column-tile count for the kernel family that runs this
+// tile size and launches it.  use_decode: the caller found the decode kernel applicable (one 32-row block per
+// tile, 32-bit offsets suffice).  The down GEMM of the int8 path multiplies bf16 Y by int8 weights.
+int launch_grouped_gemm(int prec, bool gemm0, int mblk, bool use_decode, GemmParams& p, int max_tiles, hipStream_t stream)
+{
+    // output columns per tile: the tile's weight rows, halved where gate and up rows share them
+    const int pair = gemm0 && !p.gate_only ? 2 : 1;
+    p.n_ntiles     = ceil_div(p.n_out, (use_decode ? decode_tile_cols(false) : 256) / pair);
+    if(use_decode)
+        return launch_gemm_decode(prec, gemm0, p, max_tiles, stream);
+    if(mblk > 4)
+        return launch_gemm_big(prec, gemm0, p, max_tiles, stream);
+    if(prec == MI355_MOE_BF16)
+        return gemm0 ? launch_gemm<kBf16, true>(mblk, p, max_tiles, stream) : launch_gemm<kBf16, false>(mblk, p, max_tiles, stream);
+    if(prec == MI355_MOE_FP8)
+        return gemm0 ? launch_gemm<kFp8, true>(mblk, p, max_tiles, stream) : launch_gemm<kFp8, false>(mblk, p, max_tiles, stream);
+    return gemm0 ? launch_gemm<kI8, true>(mblk, p, max_tiles, stream) : launch_gemm<kBf16W8, false>(mblk, p, max_tiles, stream);
+}
+
+// the narrow decode tiles re-read the input rows once per 64 output columns: for the down GEMM they pay off
+// only where the 256-column tiles would leave most compute units without a workgroup
+bool down_gemm_wants_decode(int experts, int64_t entries, int hidden)
+{
+    return std::min<int64_t>(experts, entries) * ceil_div(hidden, 256) < device_info().num_cu;
 }
 
 } // namespace
@@ -697,24 +636,12 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     // decode-sized problems (one 32-row block per tile) have their own kernel
     const bool decode = mblk == 1 && decode_supported((int64_t)T * a.stride_token * eb, ws.max_pad * (int64_t)I * y_b,
                                                       (int64_t)2 * I * H * eb);
-    // Y columns per tile: the tile's weight rows, halved where gate and up rows share them
-    const int pair    = t.gate_only ? 1 : 2;
-    p.n_ntiles        = decode ? ceil_div(I, decode_tile_cols(false) / pair) : ceil_div(I, 256 / pair);
     if(mblk > 4 && (int64_t)T * p.x_row_bytes >= ((int64_t)1 << 32))
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: a token buffer of 4 GiB or more (stride_token=%d) is not "
                                              "supported at this problem size", a.stride_token);
     // the two large-tile GEMMs hand Y over in the slab-major layout
     p.y_slab = (mblk > 4 && ((int64_t)I * y_b) % 64 == 0) ? (int)((int64_t)I * y_b / 64) : 0;
-    if(decode)
-        rc = launch_gemm_decode(t.prec_i, true, p, ws.max_tiles, stream);
-    else if(mblk > 4)
-        rc = launch_gemm_big(t.prec_i, true, p, ws.max_tiles, stream);
-    else if(t.prec_i == MI355_MOE_BF16)
-        rc = launch_gemm<kBf16, true>(mblk, p, ws.max_tiles, stream);
-    else if(t.prec_i == MI355_MOE_FP8)
-        rc = launch_gemm<kFp8, true>(mblk, p, ws.max_tiles, stream);
-    else
-        rc = launch_gemm<kI8, true>(mblk, p, ws.max_tiles, stream);
+    rc       = launch_grouped_gemm(t.prec_i, true, mblk, decode, p, ws.max_tiles, stream);
     if(rc != MI355_MOE_OK)
         return rc;
 
@@ -733,21 +660,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.k_bytes_w      = I * eb;
     p.n_out          = H;
     p.n_total        = H;
-    // down GEMM: rows of I bytes are short enough for the 256-row tiles to stream well, and the narrow
-    // decode tiles re-read Y once per 64 output columns; they pay off only where the wide tiles would
-    // leave most compute units without a workgroup
-    const bool decode1 = decode && (int64_t)std::min<int64_t>(E, (int64_t)T * K) * ceil_div(H, 256) < device_info().num_cu;
-    p.n_ntiles       = decode1 ? ceil_div(H, decode_tile_cols(false)) : ceil_div(H, 256);
-    if(decode1)
-        rc = launch_gemm_decode(t.prec_i, false, p, ws.max_tiles, stream);
-    else if(mblk > 4)
-        rc = launch_gemm_big(t.prec_i, false, p, ws.max_tiles, stream);
-    else if(t.prec_i == MI355_MOE_BF16)
-        rc = launch_gemm<kBf16, false>(mblk, p, ws.max_tiles, stream);
-    else if(t.prec_i == MI355_MOE_FP8)
-        rc = launch_gemm<kFp8, false>(mblk, p, ws.max_tiles, stream);
-    else
-        rc = launch_gemm<kBf16W8, false>(mblk, p, ws.max_tiles, stream);
+    rc = launch_grouped_gemm(t.prec_i, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p, ws.max_tiles,
+                             stream);
     if(rc != MI355_MOE_OK)
         return rc;
 
@@ -758,61 +672,6 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
                        static_cast<const float*>(a.sorted_weight_ptr), static_cast<unsigned char*>(a.o_ptr), K, H,
                        (int64_t)a.stride_token * 2, 0);
     }
-    MI355_HIP_TRY(hipGetLastError());
-    return MI355_MOE_OK;
-}
-
-// ck_tile's pre-shuffled weight layout b_nr_kr_kw_nw_kv: the row-major [e, n, k] tensor viewed as
-// [e, nr, nw, kr, kw, kv] and permuted to [e, nr, kr, kw, nw, kv].  One thread moves one kv granule.
-template <typename G>
-__global__ __launch_bounds__(256) void permute_weights_kernel(const G* __restrict__ src, G* __restrict__ dst,
-                                                               int64_t granules, int n, int kgran, int nw, int kw,
-                                                               int inverse)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if(i >= granules)
-        return;
-    // i enumerates the permuted layout: (e, nr, kr, kw, nw)
-    const int kr_n = kgran / kw;
-    int64_t r      = i;
-    const int a_nw = (int)(r % nw);
-    r /= nw;
-    const int a_kw = (int)(r % kw);
-    r /= kw;
-    const int a_kr = (int)(r % kr_n);
-    r /= kr_n;
-    const int a_nr = (int)(r % (n / nw));
-    const int64_t e = r / (n / nw);
-    const int64_t row_major = (e * n + (int64_t)a_nr * nw + a_nw) * kgran + (int64_t)a_kr * kw + a_kw;
-    if(inverse)
-        dst[row_major] = src[i];
-    else
-        dst[i] = src[row_major];
-}
-
-int launch_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
-                           int32_t nw, int32_t kw, int32_t kv, int32_t inverse, hipStream_t stream)
-{
-    if(!src || !dst || src == dst || experts <= 0 || n <= 0 || k <= 0 || nw <= 0 || kw <= 0 || kv <= 0 ||
-       (elem_bytes != 1 && elem_bytes != 2))
-        return fail(MI355_MOE_E_INVALID, "permute_weights: bad arguments");
-    const int gran = kv * elem_bytes;
-    if(n % nw != 0 || k % (kw * kv) != 0 || (gran != 4 && gran != 8 && gran != 16))
-        return fail(MI355_MOE_E_UNSUPPORTED,
-                    "permute_weights: n %% nw, k %% (kw*kv) must be 0 and kv*elem_bytes 4, 8 or 16 (n=%d k=%d nw=%d kw=%d kv=%d)",
-                    n, k, nw, kw, kv);
-    const int kgran        = k / kv;
-    const int64_t granules = (int64_t)experts * n * kgran;
-    const unsigned grid    = (unsigned)ceil_div<int64_t>(granules, 256);
-    if(gran == 16)
-        hipLaunchKernelGGL(permute_weights_kernel<uint4>, dim3(grid), dim3(256), 0, stream, static_cast<const uint4*>(src),
-                           static_cast<uint4*>(dst), granules, n, kgran, nw, kw, inverse);
-    else if(gran == 8)
-        hipLaunchKernelGGL(permute_weights_kernel<uint2>, dim3(grid), dim3(256), 0, stream, static_cast<const uint2*>(src),
-                           static_cast<uint2*>(dst), granules, n, kgran, nw, kw, inverse);
-    else
-        hipLaunchKernelGGL(permute_weights_kernel<uint32_t>, dim3(grid), dim3(256), 0, stream,
-                           static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst), granules, n, kgran, nw, kw, inverse);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }
@@ -951,35 +810,16 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
         p.x_scale       = w8 ? static_cast<const float*>(a.scale_m) : nullptr;
         p.out           = static_cast<unsigned char*>(a.c_ptr);
         p.out_row_bytes = (int64_t)a.stride_C * 2;
-        const int pair  = go ? 1 : 2; // gate and up rows share the tile's Y columns
         p.gate_only     = go;
         p.n_out         = I;
         p.n_total       = a.N;
-        p.n_ntiles      = decode ? ceil_div(I, decode_tile_cols(false) / pair) : ceil_div(I, 256 / pair);
-        if(decode)
-            rc = launch_gemm_decode(prec, true, p, L.max_tiles, stream);
-        else if(mblk > 4)
-            rc = launch_gemm_big(prec, true, p, L.max_tiles, stream);
-        else if(prec == MI355_MOE_BF16)
-            rc = launch_gemm<kBf16, true>(mblk, p, L.max_tiles, stream);
-        else
-            rc = launch_gemm<kI8, true>(mblk, p, L.max_tiles, stream);
-        return rc;
+        return launch_grouped_gemm(prec, true, mblk, decode, p, L.max_tiles, stream);
     }
     p.out           = wsb + L.p_off;
     p.out_row_bytes = (int64_t)H * 2;
     p.n_out         = H;
     p.n_total       = H;
-    const bool decode1 = decode && (int64_t)std::min<int64_t>(E, (int64_t)T * K) * ceil_div(H, 256) < device_info().num_cu;
-    p.n_ntiles      = decode1 ? ceil_div(H, decode_tile_cols(false)) : ceil_div(H, 256);
-    if(decode1)
-        rc = launch_gemm_decode(prec, false, p, L.max_tiles, stream);
-    else if(mblk > 4)
-        rc = launch_gemm_big(prec, false, p, L.max_tiles, stream);
-    else if(prec == MI355_MOE_BF16)
-        rc = launch_gemm<kBf16, false>(mblk, p, L.max_tiles, stream);
-    else
-        rc = launch_gemm<kBf16W8, false>(mblk, p, L.max_tiles, stream);
+    rc = launch_grouped_gemm(prec, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p, L.max_tiles, stream);
     if(rc != MI355_MOE_OK)
         return rc;
     {
@@ -988,58 +828,6 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
                            static_cast<const float*>(a.p_sorted_expert_weights), static_cast<unsigned char*>(a.c_ptr), K, H,
                            (int64_t)a.stride_C * 2, 1);
     }
-    MI355_HIP_TRY(hipGetLastError());
-    return MI355_MOE_OK;
-}
-
-int launch_moe_smoothquant(const mi355_moe_smoothquant_args& a, int32_t q_dtype, hipStream_t stream)
-{
-    if(q_dtype != MI355_MOE_FP8 && q_dtype != MI355_MOE_INT8)
-        return fail(MI355_MOE_E_UNSUPPORTED, "moe_smoothquant: q_dtype must be fp8 or int8");
-    if(a.tokens < 0 || a.hidden_size <= 0 || a.experts <= 0 || a.topk <= 0 || a.topk > 65535 || a.x_stride < a.hidden_size ||
-       a.y_stride < a.hidden_size)
-        return fail(MI355_MOE_E_INVALID, "moe_smoothquant: bad sizes (tokens=%d hidden=%d experts=%d topk=%d strides=%d,%d)",
-                    a.tokens, a.hidden_size, a.experts, a.topk, a.x_stride, a.y_stride);
-    if(a.tokens == 0)
-        return MI355_MOE_OK;
-    if(!a.p_x || !a.p_smscale || !a.p_topk_ids || !a.p_yscale || !a.p_qy)
-        return fail(MI355_MOE_E_INVALID, "moe_smoothquant: null pointer");
-    KernelTimer timer(MI355_MOE_K_QUANT, stream);
-    const dim3 grid((unsigned)a.tokens, (unsigned)a.topk);
-    if(q_dtype == MI355_MOE_FP8)
-        hipLaunchKernelGGL(moe_smoothquant_kernel<true>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
-                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
-                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
-                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
-    else
-        hipLaunchKernelGGL(moe_smoothquant_kernel<false>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
-                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
-                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
-                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
-    MI355_HIP_TRY(hipGetLastError());
-    return MI355_MOE_OK;
-}
-
-int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype, void* q,
-                         void* scale, hipStream_t stream)
-{
-    if(!x || !q || !scale || rows < 0 || cols <= 0 || stride_x < cols)
-        return fail(MI355_MOE_E_INVALID, "rowwise_quant: bad arguments");
-    if(q_dtype != MI355_MOE_FP8 && q_dtype != MI355_MOE_INT8)
-        return fail(MI355_MOE_E_UNSUPPORTED, "rowwise_quant: q_dtype must be fp8 or int8");
-    if(rows == 0)
-        return MI355_MOE_OK;
-    if(rows > 0x7fffffff)
-        return fail(MI355_MOE_E_INVALID, "rowwise_quant: too many rows");
-    KernelTimer timer(MI355_MOE_K_QUANT, stream);
-    if(q_dtype == MI355_MOE_FP8)
-        hipLaunchKernelGGL(rowwise_quant_kernel<true>, dim3((unsigned)rows), dim3(256), 0, stream,
-                           static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),
-                           static_cast<float*>(scale));
-    else
-        hipLaunchKernelGGL(rowwise_quant_kernel<false>, dim3((unsigned)rows), dim3(256), 0, stream,
-                           static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),
-                           static_cast<float*>(scale));
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }

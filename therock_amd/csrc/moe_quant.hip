@@ -1,0 +1,208 @@
+// Data-preparation kernels around the fused-MoE GEMMs for gfx950: per-row dynamic quantisation, ck_tile's
+// MoE smooth-quant, and the conversion to and from ck_tile's pre-shuffled weight layout.  All of them are
+// HBM-bound byte movers: one pass over the input, coalesced 16-byte accesses, no LDS beyond the row reductions.
+#include "moe_gemm_device.hpp"
+
+#include <algorithm>
+
+namespace mi355 {
+using namespace gemm;
+namespace {
+
+// per-row dynamic quantisation bf16 -> e4m3 / int8
+template <bool FP8>
+__global__ __launch_bounds__(256) void rowwise_quant_kernel(const uint16_t* __restrict__ x, int cols,
+                                                             int64_t stride_x, unsigned char* __restrict__ q,
+                                                             float* __restrict__ scale)
+{
+    __shared__ float s_red[4];
+    const int64_t row  = blockIdx.x;
+    const uint16_t* xr = x + row * stride_x;
+    float amax         = 0.f;
+    for(int c = threadIdx.x; c < cols; c += 256)
+        amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c])));
+#pragma unroll
+    for(int d = 32; d > 0; d >>= 1)
+        amax = fmaxf(amax, __shfl_xor(amax, d));
+    if((threadIdx.x & 63) == 0)
+        s_red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax            = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    const float qmx = FP8 ? 448.0f : 127.0f;
+    const float s   = amax > 0.f ? amax / qmx : 1.0f;
+    if(threadIdx.x == 0)
+        scale[row] = s;
+    for(int c = threadIdx.x; c < cols; c += 256)
+    {
+        const float v = bf16_bits_to_float(xr[c]) / s;
+        if constexpr(FP8)
+        {
+            const float cl = fminf(fmaxf(v, -448.f), 448.f);
+            q[row * cols + c] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
+        }
+        else
+        {
+            // ck_tile's float -> int8 conversion is a static_cast: truncation toward zero
+            const float cl = fminf(fmaxf(v, -128.f), 127.f);
+            q[row * cols + c] = static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
+        }
+    }
+}
+
+// MoE smooth-quant: row (slot k, token t) = x[t, :] * smscale[expert(t, k), :], per-row dynamic quantisation
+template <bool FP8>
+__global__ __launch_bounds__(256) void moe_smoothquant_kernel(const uint16_t* __restrict__ x,
+                                                               const float* __restrict__ smscale,
+                                                               const int* __restrict__ topk_ids, int tokens, int hidden,
+                                                               int experts, int topk, int64_t x_stride, int64_t y_stride,
+                                                               unsigned char* __restrict__ qy, float* __restrict__ yscale)
+{
+    __shared__ float s_red[4];
+    const int t = blockIdx.x;
+    const int k = blockIdx.y;
+    int e       = topk_ids[(int64_t)t * topk + k];
+    e           = min(max(e, 0), experts - 1);
+    const uint16_t* xr = x + (int64_t)t * x_stride;
+    const float* sr    = smscale + (int64_t)e * hidden;
+    float amax         = 0.f;
+    for(int c = threadIdx.x; c < hidden; c += 256)
+        amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c]) * sr[c]));
+#pragma unroll
+    for(int d = 32; d > 0; d >>= 1)
+        amax = fmaxf(amax, __shfl_xor(amax, d));
+    if((threadIdx.x & 63) == 0)
+        s_red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax            = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    const float qmx = FP8 ? 448.0f : 127.0f;
+    const float ys  = amax / qmx;
+    const int64_t r = (int64_t)k * tokens + t;
+    if(threadIdx.x == 0)
+        yscale[r] = ys;
+    unsigned char* qr = qy + r * y_stride;
+    for(int c = threadIdx.x; c < hidden; c += 256)
+    {
+        const float v = (bf16_bits_to_float(xr[c]) * sr[c]) / ys;
+        if constexpr(FP8)
+        {
+            const float cl = fminf(fmaxf(v, -448.f), 448.f);
+            qr[c] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
+        }
+        else
+        {
+            const float cl = fminf(fmaxf(v, -128.f), 127.f);
+            qr[c] = static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
+        }
+    }
+}
+
+// ck_tile's pre-shuffled weight layout b_nr_kr_kw_nw_kv: the row-major [e, n, k] tensor viewed as
+// [e, nr, nw, kr, kw, kv] and permuted to [e, nr, kr, kw, nw, kv].  One thread moves one kv granule.
+template <typename G>
+__global__ __launch_bounds__(256) void permute_weights_kernel(const G* __restrict__ src, G* __restrict__ dst,
+                                                               int64_t granules, int n, int kgran, int nw, int kw,
+                                                               int inverse)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if(i >= granules)
+        return;
+    // i enumerates the permuted layout: (e, nr, kr, kw, nw)
+    const int kr_n = kgran / kw;
+    int64_t r      = i;
+    const int a_nw = (int)(r % nw);
+    r /= nw;
+    const int a_kw = (int)(r % kw);
+    r /= kw;
+    const int a_kr = (int)(r % kr_n);
+    r /= kr_n;
+    const int a_nr = (int)(r % (n / nw));
+    const int64_t e = r / (n / nw);
+    const int64_t row_major = (e * n + (int64_t)a_nr * nw + a_nw) * kgran + (int64_t)a_kr * kw + a_kw;
+    if(inverse)
+        dst[row_major] = src[i];
+    else
+        dst[i] = src[row_major];
+}
+
+} // namespace
+
+int launch_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
+                           int32_t nw, int32_t kw, int32_t kv, int32_t inverse, hipStream_t stream)
+{
+    if(!src || !dst || src == dst || experts <= 0 || n <= 0 || k <= 0 || nw <= 0 || kw <= 0 || kv <= 0 ||
+       (elem_bytes != 1 && elem_bytes != 2))
+        return fail(MI355_MOE_E_INVALID, "permute_weights: bad arguments");
+    const int gran = kv * elem_bytes;
+    if(n % nw != 0 || k % (kw * kv) != 0 || (gran != 4 && gran != 8 && gran != 16))
+        return fail(MI355_MOE_E_UNSUPPORTED,
+                    "permute_weights: n %% nw, k %% (kw*kv) must be 0 and kv*elem_bytes 4, 8 or 16 (n=%d k=%d nw=%d kw=%d kv=%d)",
+                    n, k, nw, kw, kv);
+    const int kgran        = k / kv;
+    const int64_t granules = (int64_t)experts * n * kgran;
+    const unsigned grid    = (unsigned)ceil_div<int64_t>(granules, 256);
+    if(gran == 16)
+        hipLaunchKernelGGL(permute_weights_kernel<uint4>, dim3(grid), dim3(256), 0, stream, static_cast<const uint4*>(src),
+                           static_cast<uint4*>(dst), granules, n, kgran, nw, kw, inverse);
+    else if(gran == 8)
+        hipLaunchKernelGGL(permute_weights_kernel<uint2>, dim3(grid), dim3(256), 0, stream, static_cast<const uint2*>(src),
+                           static_cast<uint2*>(dst), granules, n, kgran, nw, kw, inverse);
+    else
+        hipLaunchKernelGGL(permute_weights_kernel<uint32_t>, dim3(grid), dim3(256), 0, stream,
+                           static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst), granules, n, kgran, nw, kw, inverse);
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+int launch_moe_smoothquant(const mi355_moe_smoothquant_args& a, int32_t q_dtype, hipStream_t stream)
+{
+    if(q_dtype != MI355_MOE_FP8 && q_dtype != MI355_MOE_INT8)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_smoothquant: q_dtype must be fp8 or int8");
+    if(a.tokens < 0 || a.hidden_size <= 0 || a.experts <= 0 || a.topk <= 0 || a.topk > 65535 || a.x_stride < a.hidden_size ||
+       a.y_stride < a.hidden_size)
+        return fail(MI355_MOE_E_INVALID, "moe_smoothquant: bad sizes (tokens=%d hidden=%d experts=%d topk=%d strides=%d,%d)",
+                    a.tokens, a.hidden_size, a.experts, a.topk, a.x_stride, a.y_stride);
+    if(a.tokens == 0)
+        return MI355_MOE_OK;
+    if(!a.p_x || !a.p_smscale || !a.p_topk_ids || !a.p_yscale || !a.p_qy)
+        return fail(MI355_MOE_E_INVALID, "moe_smoothquant: null pointer");
+    KernelTimer timer(MI355_MOE_K_QUANT, stream);
+    const dim3 grid((unsigned)a.tokens, (unsigned)a.topk);
+    if(q_dtype == MI355_MOE_FP8)
+        hipLaunchKernelGGL(moe_smoothquant_kernel<true>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
+                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
+                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
+                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
+    else
+        hipLaunchKernelGGL(moe_smoothquant_kernel<false>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
+                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
+                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
+                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype, void* q,
+                         void* scale, hipStream_t stream)
+{
+    if(!x || !q || !scale || rows < 0 || cols <= 0 || stride_x < cols)
+        return fail(MI355_MOE_E_INVALID, "rowwise_quant: bad arguments");
+    if(q_dtype != MI355_MOE_FP8 && q_dtype != MI355_MOE_INT8)
+        return fail(MI355_MOE_E_UNSUPPORTED, "rowwise_quant: q_dtype must be fp8 or int8");
+    if(rows == 0)
+        return MI355_MOE_OK;
+    if(rows > 0x7fffffff)
+        return fail(MI355_MOE_E_INVALID, "rowwise_quant: too many rows");
+    KernelTimer timer(MI355_MOE_K_QUANT, stream);
+    if(q_dtype == MI355_MOE_FP8)
+        hipLaunchKernelGGL(rowwise_quant_kernel<true>, dim3((unsigned)rows), dim3(256), 0, stream,
+                           static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),
+                           static_cast<float*>(scale));
+    else
+        hipLaunchKernelGGL(rowwise_quant_kernel<false>, dim3((unsigned)rows), dim3(256), 0, stream,
+                           static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),
+                           static_cast<float*>(scale));
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+} // namespace mi355
