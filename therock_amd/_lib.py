@@ -125,6 +125,12 @@ def load():
             raise RuntimeError(
                 f"{LIB_PATH} is missing: build it with `python -m therock_amd.build` (needs hipcc); "
                 "there is no CPU fallback")
+        # PyTorch ships its own HIP runtime under the same soname as ROCm's.  Whichever is loaded first serves
+        # the whole process, and initialising ROCm's copy from this library before torch initialises left the
+        # process without a visible device.  torch owns the device memory and the streams here, so its runtime
+        # is loaded first and this library binds to it.
+        import torch  # noqa: F401
+
         lib = C.CDLL(LIB_PATH)
         for name, (res, args) in PROTOTYPES.items():
             fn = getattr(lib, name)
