@@ -30,7 +30,9 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_struct_layouts_match_the_header(tmp_path):
     structs = {"mi355_moe_sorting_args": _lib.SortingArgs, "mi355_fused_moe_traits": _lib.FusedMoeTraits,
-               "mi355_fused_moegemm_args": _lib.FusedMoeGemmArgs, "mi355_fused_moe_args": _lib.FusedMoeArgs}
+               "mi355_fused_moegemm_args": _lib.FusedMoeGemmArgs, "mi355_fused_moe_args": _lib.FusedMoeArgs,
+               "mi355_topk_softmax_args": _lib.TopkSoftmaxArgs, "mi355_topk_softmax_traits": _lib.TopkSoftmaxTraits,
+               "mi355_moe_flatmm_args": _lib.FlatmmArgs, "mi355_moe_smoothquant_args": _lib.SmoothquantArgs}
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void){"]
     for cname, ct in structs.items():
         lines.append(f'printf("{cname} %zu\\n", sizeof({cname}));')
@@ -63,6 +65,18 @@ def test_host_only_entry_points():
     assert lib.mi355_fused_moe_workspace_size(C.byref(bad), 128, 8, 2, 1024, 1024) == 0
     assert lib.mi355_moe_sorting(None, None) == _lib.E_INVALID and b"null" in lib.mi355_moe_last_error()
     assert lib.mi355_fused_moe(None, None, None) == _lib.E_INVALID
+    # traits of the reference's example API: both activations and both weight layouts have kernels
+    for act, gate_only, ok in ((0, 0, 1), (1, 1, 1), (0, 1, 1), (2, 0, 0), (1, 2, 0)):
+        t = _lib.FusedMoeTraits(0, 0, 0, 3, 3, 3, 3, 32, act, gate_only, 0, 0)
+        assert lib.mi355_fused_moe_supported(C.byref(t)) == ok
+    # rows per GEMM workgroup: decode tiles, small tiles, 320-row tiles (bf16 / fp8 only, sort unit a multiple of 16)
+    rows = lambda prec, unit, *shape: lib.mi355_fused_moe_tile_rows(
+        C.byref(_lib.FusedMoeTraits(prec, prec, 0, 3, 3, 3, 3, unit, 1, 0, 0, 0)), *shape)
+    assert rows(2, 32, 64, 128, 8, 4096, 1536) == 32
+    assert rows(1, 32, 8192, 256, 8, 7168, 2048) == 320
+    assert rows(1, 32, 1024, 256, 8, 7168, 2048) == 320 and rows(1, 32, 512, 256, 8, 7168, 2048) == 32
+    assert rows(1, 8, 8192, 256, 8, 7168, 2048) == 128
+    assert rows(2, 32, 8192, 128, 8, 4096, 1536) == 128
 
 
 def test_python_mirror_rejects_unknown_traits_without_touching_the_gpu():
