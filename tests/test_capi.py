@@ -69,14 +69,14 @@ def test_host_only_entry_points():
     for act, gate_only, ok in ((0, 0, 1), (1, 1, 1), (0, 1, 1), (2, 0, 0), (1, 2, 0)):
         t = _lib.FusedMoeTraits(0, 0, 0, 3, 3, 3, 3, 32, act, gate_only, 0, 0)
         assert lib.mi355_fused_moe_supported(C.byref(t)) == ok
-    # rows per GEMM workgroup: decode tiles, small tiles, 320-row tiles (bf16 / fp8 only, sort unit a multiple of 16)
+    # rows per GEMM workgroup: decode tiles, small tiles, 320-row tiles (sort unit a multiple of 16)
     rows = lambda prec, unit, *shape: lib.mi355_fused_moe_tile_rows(
         C.byref(_lib.FusedMoeTraits(prec, prec, 0, 3, 3, 3, 3, unit, 1, 0, 0, 0)), *shape)
     assert rows(2, 32, 64, 128, 8, 4096, 1536) == 32
     assert rows(1, 32, 8192, 256, 8, 7168, 2048) == 320
     assert rows(1, 32, 1024, 256, 8, 7168, 2048) == 320 and rows(1, 32, 512, 256, 8, 7168, 2048) == 32
     assert rows(1, 8, 8192, 256, 8, 7168, 2048) == 128
-    assert rows(2, 32, 8192, 128, 8, 4096, 1536) == 128
+    assert rows(2, 32, 8192, 128, 8, 4096, 1536) == 320 and rows(2, 32, 8192, 128, 8, 4096, 1504) == 128
 
 
 def test_python_mirror_rejects_unknown_traits_without_touching_the_gpu():

@@ -125,7 +125,7 @@ def test_decode_kernel_ragged(dtype):
     check(mi.MoeConfig("d", 40, 2080, 640, 64, 8, dtype, "sigmoid_renorm", unit=16), seed=3)
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 def test_many_rows_per_expert_with_small_sort_units(dtype):
     # hundreds of rows per expert, but expert boundaries on multiples of 8 or 24 rows only: the 320-row kernel
     # (whose tiles start on whole 16-row slabs of the intermediate buffer) must not be chosen for unit 8 or 24
@@ -137,7 +137,7 @@ def test_many_rows_per_expert_with_small_sort_units(dtype):
         check(cfg, seed=unit)
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 def test_large_tile_kernel_partial_tiles(dtype):
     # from about 28 rows per expert on, and with enough tiles to fill the chip, the 320-row kernel runs with
     # mostly empty tiles: it then fetches only the 64-row slab groups a tile has (1 to 5 per step)

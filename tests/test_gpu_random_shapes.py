@@ -36,10 +36,10 @@ def draw_many_rows(rng, dtype):
     return mi.MoeConfig("rnd", tokens, hidden, inter, experts, topk, dtype, str(rng.choice(ROUTERS)), unit=unit)
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 def test_random_shapes_many_rows_per_expert(dtype):
     import therock_amd as ta
-    rng = np.random.default_rng({"bf16": 11, "fp8": 22}[dtype])
+    rng = np.random.default_rng({"bf16": 11, "fp8": 22, "int8": 33}[dtype])
     for case in range(10):
         cfg = draw_many_rows(rng, dtype)
         traits = ta.fused_moe_traits(prec_i=dtype, prec_w=dtype, block_m=cfg.unit)

@@ -98,8 +98,11 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     using Acc = typename MT::Acc;
     constexpr int kOpB   = MT::kOpB;
     constexpr int kSteps = kStepKB / (2 * kOpB); // MFMAs along K per compute step: 1 (fp8) or 2 (bf16, i8)
+    // int8 weights against bf16 tokens (down GEMM of the int8 path): a 64-byte token step is 32 elements = 32
+    // weight bytes, so the 128-byte lines of a weight unit last four steps instead of two
+    constexpr bool kW8 = MODE == kBf16W8;
     constexpr bool kMx   = MODE == kFp8 && !GEMM0;
-    static_assert(MODE == kBf16 || MODE == kFp8 || MODE == kI8, "no large-tile kernel for this mode");
+    static_assert(MODE == kBf16 || MODE == kFp8 || (MODE == kI8 && GEMM0) || (MODE == kBf16W8 && !GEMM0), "no large-tile kernel for this mode");
 
     extern __shared__ __align__(16) unsigned char lds[];
 
@@ -195,7 +198,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     const int x_step      = (!GEMM0 && p.y_slab > 0) ? 1024 : kStepKB; // bytes between token steps
 
     const uint32_t lds_base = lds_offset(lds);
-    const int kt_count      = p.k_bytes_x / kStepKB; // compute steps = weight units (even)
+    const int kt_count      = p.k_bytes_x / kStepKB; // compute steps (even; a multiple of four with int8 weights)
+    const int n_wunits      = kW8 ? kt_count / 2 : kt_count; // two units (row halves) per 128 bytes of weight K
 
     // weight role: unit u (half u & 1) -> ring slot u % 6
     // Weights no other row tile re-reads (the expert has a single one) are fetched non-temporal: measured
@@ -206,17 +210,22 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     auto issue_w = [&](int u, auto half_tag, auto nt_tag) __attribute__((always_inline)) {
         constexpr int H = decltype(half_tag)::value;
         constexpr bool NT = decltype(nt_tag)::value;
-        if(u >= kt_count)
+        if(u >= n_wunits)
             return;
         const uint32_t sbase     = lds_base + (u % kWSlots) * kWUnitBytes + q4 * 1024;
         const unsigned char* src = dbase + (u >> 1) * (2 * kStepKB);
 #pragma unroll
         for(int j = 0; j < 4; j++)
         {
+            // H < 0: the row half is not known at compile time (int8 weights: one unit every other step); the
+            // choice is spelled as arithmetic, a select between two elements of doff[] turns the array into an
+            // indexed one in scratch memory
+            const uint32_t off = H >= 0 ? doff[(H >= 0 ? H : 0) * 4 + j]
+                                        : doff[j] ^ ((doff[j] ^ doff[4 + j]) & (0u - (uint32_t)(u & 1)));
             if constexpr(NT)
-                dma16nt(src, doff[H * 4 + j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));
+                dma16nt(src, off, __builtin_amdgcn_readfirstlane(sbase + j * 4096));
             else
-                dma16(src, doff[H * 4 + j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));
+                dma16(src, off, __builtin_amdgcn_readfirstlane(sbase + j * 4096));
         }
     };
     // token role: step x -> ring stage x % 3
@@ -307,11 +316,18 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             if(w_role)
-                issue_w(k + 4, par_tag, nt_tag);
+            {
+                if constexpr(!kW8)
+                    issue_w(k + 4, par_tag, nt_tag);
+                else if constexpr(PAR == 0)
+                    issue_w((k >> 1) + 4, std::integral_constant<int, -1>{}, nt_tag);
+            }
             else
                 issue_x(k + 2, XG);
 
-            const unsigned char* wst = lds + (((k & ~1) + w_h) % kWSlots) * kWUnitBytes + w_off;
+            // first unit of the pair that holds this step's weight bytes
+            const int pair0          = kW8 ? (k >> 2) << 1 : (k & ~1);
+            const unsigned char* wst = lds + ((pair0 + w_h) % kWSlots) * kWUnitBytes + w_off;
             const unsigned char* xst = lds + x_off + (k % kXStages) * kXStageBytes;
             [[maybe_unused]] const unsigned char* ysl =
                 lds + kYsOffset + (k % kXStages) * kYsStageBytes + kg * kYsRows + wt * 32 + r32;
@@ -330,9 +346,18 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 for(int b = 0; b < 2; b++)
                 {
                     const unsigned char* wp = wst + b * 32 * (2 * kStepKB);
-                    wf[b].lo                = *reinterpret_cast<const uint4*>(wp + cw_lo);
-                    if constexpr(kOpB == 32)
-                        wf[b].hi = *reinterpret_cast<const uint4*>(wp + cw_hi);
+                    if constexpr(kW8)
+                    {
+                        // 8 int8 of this lane's K group: 16-byte chunk (k & 3) * 2 + s of the row, half kg
+                        const int c8 = ((((k & 3) << 1) + s) ^ sw_w) * 16 + kg * 8;
+                        wf[b].lo     = int8x8_to_bf16x8(*reinterpret_cast<const uint2*>(wp + c8));
+                    }
+                    else
+                    {
+                        wf[b].lo = *reinterpret_cast<const uint4*>(wp + cw_lo);
+                        if constexpr(kOpB == 32)
+                            wf[b].hi = *reinterpret_cast<const uint4*>(wp + cw_hi);
+                    }
                 }
 #pragma unroll
                 for(int i = 0; i < NB; i++)
@@ -422,6 +447,9 @@ int big_tile_rows() { return kBigXRows; }
 
 bool big_tile_supported(int prec, int k_bytes0, int k_bytes1)
 {
+    // K in whole pairs of 64-byte steps; the int8 path's down GEMM (bf16 Y against int8 weights) in fours
+    if(prec == MI355_MOE_INT8)
+        return k_bytes0 % (2 * kStepKB) == 0 && k_bytes1 % (4 * kStepKB) == 0;
     return (prec == MI355_MOE_BF16 || prec == MI355_MOE_FP8) && k_bytes0 % (2 * kStepKB) == 0 && k_bytes1 % (2 * kStepKB) == 0;
 }
 
@@ -431,6 +459,8 @@ int launch_gemm_big(int prec, bool gemm0, const GemmParams& p, int max_tiles, hi
         return gemm0 ? launch_big_t<kBf16, true>(p, max_tiles, stream) : launch_big_t<kBf16, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_FP8)
         return gemm0 ? launch_big_t<kFp8, true>(p, max_tiles, stream) : launch_big_t<kFp8, false>(p, max_tiles, stream);
+    if(prec == MI355_MOE_INT8)
+        return gemm0 ? launch_big_t<kI8, true>(p, max_tiles, stream) : launch_big_t<kBf16W8, false>(p, max_tiles, stream);
     return fail(MI355_MOE_E_UNSUPPORTED, "no large-tile kernel for precision %d", prec);
 }
 
