@@ -286,8 +286,8 @@ typedef struct mi355_moe_flatmm_args
     int32_t stride_A;
     int32_t stride_B;
     int32_t stride_C;
-    int32_t prec_a;       /* mi355_moe_dtype of A: BF16, or INT8 for the gate+up GEMM with int8 weights */
-    int32_t prec_b;       /* mi355_moe_dtype of B: BF16 | INT8 */
+    int32_t prec_a;       /* mi355_moe_dtype of A: BF16, FP8 (with FP8 weights), or INT8 for the gate+up GEMM with int8 weights */
+    int32_t prec_b;       /* mi355_moe_dtype of B: BF16 | FP8 | INT8 */
     int32_t block_m;      /* unit_size the sort was run with */
 } mi355_moe_flatmm_args;
 

@@ -22,7 +22,7 @@ SHAPES = [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (130, 6, 2, 1152
 
 
 @pytest.mark.parametrize("T,E,K,H,I,unit", SHAPES)
-@pytest.mark.parametrize("kind", ["bf16", "int8"])
+@pytest.mark.parametrize("kind", ["bf16", "int8", "fp8"])
 def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     import torch
     import therock_amd as ta
@@ -48,11 +48,14 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
         sa = sg = sd = None
         d_sa = d_sg = d_sd = None
     else:
-        xq, sa = oracle.rowwise_quant(x32, oracle.DT_I8, nearest=True)
-        gq, sg = oracle.rowwise_quant(g32.reshape(E * 2 * I, H), oracle.DT_I8, nearest=True)
-        dq, sd = oracle.rowwise_quant(d32.reshape(E * H, I), oracle.DT_I8, nearest=True)
+        qdt = oracle.DT_I8 if kind == "int8" else oracle.DT_E4M3
+        kw = dict(nearest=True) if kind == "int8" else {}
+        xq, sa = oracle.rowwise_quant(x32, qdt, **kw)
+        gq, sg = oracle.rowwise_quant(g32.reshape(E * 2 * I, H), qdt, **kw)
+        dq, sd = oracle.rowwise_quant(d32.reshape(E * H, I), qdt, **kw)
         x, g, d = dev(xq), dev(gq.reshape(E, 2 * I, H)), dev(dq.reshape(E, H, I))
-        xr, gr, dr = xq.astype(np.float32), gq.reshape(E, 2 * I, H).astype(np.float32), dq.reshape(E, H, I).astype(np.float32)
+        xr, gr, dr = (oracle.to_f32(xq, qdt), oracle.to_f32(gq.reshape(E, 2 * I, H), qdt),
+                      oracle.to_f32(dq.reshape(E, H, I), qdt))
         sg, sd = sg.reshape(E, 2 * I), sd.reshape(E, H)
         d_sa, d_sg, d_sd = dev(sa), dev(sg), dev(sd)
 
@@ -78,12 +81,18 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     assert _rel(yog[:T * K], oracle.to_f32(yo_ref, oracle.DT_BF16)) <= tol
 
     # down: added to what c holds; a takes the reference's bf16 Y so that the two GEMMs are checked apart
-    y_in = torch.from_numpy(y_ref.view(np.int16)).cuda().view(torch.bfloat16)
+    # (fp8: that Y quantised per row, the row scales going in as scale_m)
+    y_f32 = oracle.to_f32(y_ref, oracle.DT_BF16)
+    if kind == "fp8":
+        yq, sy = oracle.rowwise_quant(y_f32, oracle.DT_E4M3)
+        y_in, a_ref, s_m, d_sm = dev(yq), oracle.to_f32(yq, oracle.DT_E4M3), sy, dev(sy)
+    else:
+        y_in, a_ref, s_m, d_sm = torch.from_numpy(y_ref.view(np.int16)).cuda().view(torch.bfloat16), y_f32, None, None
     c0 = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
     c = bf(c0)
-    c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, oracle.to_f32(y_ref, oracle.DT_BF16), dr, _bits(c).copy(), T, K,
-                            None, sd)
-    assert ta.moe_flatmm(ta.GEMM2, y_in, d, c, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w, scale_n=d_sd) == 0.0
+    c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, a_ref, dr, _bits(c).copy(), T, K, s_m, sd)
+    assert ta.moe_flatmm(ta.GEMM2, y_in, d, c, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w, scale_m=d_sm,
+                         scale_n=d_sd) == 0.0
     torch.cuda.synchronize()
     assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, oracle.DT_BF16)) <= tol
 

@@ -345,12 +345,20 @@ __global__ __launch_bounds__(256) void moe_inv_kernel(const int* __restrict__ so
     }
 }
 
+// 16-byte fill (a kernel, not a memset node: the path may be captured in a graph)
+__global__ __launch_bounds__(256) void fill_u32x4_kernel(uint4* __restrict__ dst, int64_t n, uint32_t v)
+{
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+        dst[i] = make_uint4(v, v, v, v);
+}
+
 // O[t, h] = sum over slots (in slot order) of top-k weight * bf16 partial, fp32 accumulate, one rounding
 __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* __restrict__ part,
                                                            const int* __restrict__ inv,
                                                            const float* __restrict__ sorted_w,
                                                            unsigned char* __restrict__ out, int topk, int hidden,
-                                                           int64_t out_row_bytes, int accumulate)
+                                                           int64_t out_row_bytes, int accumulate,
+                                                           const float* __restrict__ slot_scale)
 {
     const int t  = blockIdx.x;
     const int h0 = (blockIdx.y * 256 + threadIdx.x) * 8;
@@ -387,6 +395,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
             if(pos[j] >= 0)
             {
                 w[j] = sorted_w[pos[j]];
+                if(slot_scale) // per-row scale of the stand-alone down GEMM's quantised input, row = token * topk + slot
+                    w[j] *= slot_scale[t * topk + k0 + j];
                 v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(part + ((int64_t)pos[j] * hidden + h0) * 2));
             }
         }
@@ -670,7 +680,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     KernelTimer timer(MI355_MOE_K_COMBINE, stream);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, inv,
                        static_cast<const float*>(a.sorted_weight_ptr), static_cast<unsigned char*>(a.o_ptr), K, H,
-                       (int64_t)a.stride_token * 2, 0);
+                       (int64_t)a.stride_token * 2, 0, static_cast<const float*>(nullptr));
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
@@ -682,8 +692,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
 namespace {
 struct FlatmmLayout
 {
-    size_t map_off, inv_off, p_off, total;
-    int64_t max_pad;
+    size_t map_off, inv_off, p_off, ys_off, total;
+    int64_t max_pad, ys_kb_stride;
     int32_t max_tiles;
     int mblk, hidden, inter;
     mi355_fused_moe_traits traits;
@@ -696,21 +706,23 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
     const bool g1     = kind != MI355_MOE_GEMM2;
     const bool go     = kind == MI355_MOE_GEMM1_GATE_ONLY;
     const bool w8     = a.prec_b == MI355_MOE_INT8;
-    const bool ok_typ = (a.prec_b == MI355_MOE_BF16 && a.prec_a == MI355_MOE_BF16) ||
+    const bool f8     = a.prec_b == MI355_MOE_FP8;
+    const bool ok_typ = (a.prec_b == MI355_MOE_BF16 && a.prec_a == MI355_MOE_BF16) || (f8 && a.prec_a == MI355_MOE_FP8) ||
                         (w8 && a.prec_a == (g1 ? MI355_MOE_INT8 : MI355_MOE_BF16));
     if(!ok_typ)
-        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: operand types a=%d b=%d (bf16 x bf16, int8 x int8 for the "
-                                             "gate+up GEMM, bf16 x int8 for the down GEMM)", a.prec_a, a.prec_b);
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: operand types a=%d b=%d (bf16 x bf16, fp8 x fp8, int8 x int8 for "
+                                             "the gate+up GEMM, bf16 x int8 for the down GEMM)", a.prec_a, a.prec_b);
     if(a.NumTokens < 0 || a.NumExperts <= 0 || a.NumExperts > 1024 || a.TopK <= 0 || a.TopK > 255 || a.N <= 0 || a.K <= 0 ||
        a.block_m < 1 || a.block_m > 1024 || a.k_batch > 1 || (g1 && !go && a.N % 2 != 0))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: bad sizes (tokens=%d experts=%d topk=%d N=%d K=%d block_m=%d k_batch=%d)",
                     a.NumTokens, a.NumExperts, a.TopK, a.N, a.K, a.block_m, a.k_batch);
     L.hidden = g1 ? a.K : a.N;
     L.inter  = g1 ? (go ? a.N : a.N / 2) : a.K;
-    if(L.hidden % 32 != 0 || L.inter % 32 != 0)
+    if(L.hidden % 32 != 0 || L.inter % 32 != 0 || (f8 && !g1 && L.inter % 128 != 0))
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: N and K must give hidden and intermediate sizes that are "
-                                             "multiples of 32 (hidden=%d inter=%d)", L.hidden, L.inter);
-    const int prec = w8 ? MI355_MOE_INT8 : MI355_MOE_BF16;
+                                             "multiples of 32, K of the fp8 down GEMM of 128 (hidden=%d inter=%d)", L.hidden,
+                    L.inter);
+    const int prec = w8 ? MI355_MOE_INT8 : f8 ? MI355_MOE_FP8 : MI355_MOE_BF16;
     L.traits       = mi355_fused_moe_traits{prec, prec, MI355_MOE_BF16, MI355_MOE_FP32, MI355_MOE_FP32, MI355_MOE_FP32,
                                             MI355_MOE_FP32, a.block_m, 1, 0, 0, 0};
     L.mblk         = pick_mblk(L.traits, a.NumTokens, a.TopK, a.NumExperts, L.hidden, L.inter);
@@ -725,6 +737,9 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
     L.map_off = bump(sizeof(int) * (kMapHdr + (size_t)kMapEnt * L.max_tiles));
     L.inv_off = bump(sizeof(int) * (size_t)a.NumTokens * a.TopK);
     L.p_off   = bump(g1 ? 0 : (size_t)L.max_pad * L.hidden * 2);
+    // the fp8 down GEMM runs the block-scaled MFMA: its input carries one scale per row, so every block scale is 2^0
+    L.ys_kb_stride = round_up<int64_t>(L.max_pad, 256) + 512;
+    L.ys_off       = bump(f8 && !g1 ? (size_t)L.ys_kb_stride * (L.inter / 32) : 0);
     return MI355_MOE_OK;
 }
 } // namespace
@@ -744,15 +759,16 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
     const bool g1 = kind != MI355_MOE_GEMM2;
     const bool go = kind == MI355_MOE_GEMM1_GATE_ONLY;
     const bool w8 = a.prec_b == MI355_MOE_INT8;
+    const bool f8 = a.prec_b == MI355_MOE_FP8;
     if(!a.p_sorted_token_ids || !a.p_sorted_expert_ids || !a.p_max_token_id || !a.a_ptr || !a.b_ptr || !a.c_ptr ||
        (!g1 && !a.p_sorted_expert_weights))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: null pointer");
     if(a.exp_bias != nullptr)
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: expert bias is not implemented");
-    if(w8 && (!a.scale_n || (g1 && !a.scale_m)))
-        return fail(MI355_MOE_E_INVALID, "moe_flatmm: int8 weights need scale_n (and int8 activations scale_m)");
+    if((w8 || f8) && (!a.scale_n || ((g1 || f8) && !a.scale_m)))
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: quantised weights need scale_n, quantised activations scale_m");
     const int T = a.NumTokens, E = a.NumExperts, K = a.TopK, H = L.hidden, I = L.inter;
-    const int a_b = a.prec_a == MI355_MOE_INT8 ? 1 : 2, b_b = w8 ? 1 : 2;
+    const int a_b = a.prec_a == MI355_MOE_BF16 ? 2 : 1, b_b = (w8 || f8) ? 1 : 2;
     if(a.stride_A < a.K || a.stride_B != a.K || a.stride_C < (g1 ? I : H) || ((int64_t)a.stride_A * a_b) % 16 != 0 ||
        ((int64_t)a.stride_C * 2) % 16 != 0)
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: strides (A=%d B=%d C=%d): B must be [experts, N, K] with K "
@@ -798,7 +814,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
     p.w              = static_cast<const unsigned char*>(a.b_ptr);
     p.w_row_bytes    = (int64_t)a.K * b_b;
     p.w_expert_bytes = (int64_t)a.N * a.K * b_b;
-    p.w_scale        = w8 ? static_cast<const float*>(a.scale_n) : nullptr;
+    p.w_scale        = (w8 || f8) ? static_cast<const float*>(a.scale_n) : nullptr;
     p.k_bytes_x      = a.K * a_b;
     p.k_bytes_w      = a.K * b_b;
     const int64_t a_rows = g1 ? T : (int64_t)T * K;
@@ -807,7 +823,8 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
     const bool decode = mblk == 1 && decode_supported(a_rows * p.x_row_bytes, a_rows * p.x_row_bytes, p.w_expert_bytes);
     if(g1)
     {
-        p.x_scale       = w8 ? static_cast<const float*>(a.scale_m) : nullptr;
+        p.x_scale       = (w8 || f8) ? static_cast<const float*>(a.scale_m) : nullptr;
+        p.y_bf16        = 1; // C is bf16 whatever the operand type
         p.out           = static_cast<unsigned char*>(a.c_ptr);
         p.out_row_bytes = (int64_t)a.stride_C * 2;
         p.gate_only     = go;
@@ -819,6 +836,14 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
     p.out_row_bytes = (int64_t)H * 2;
     p.n_out         = H;
     p.n_total       = H;
+    if(f8)
+    {
+        p.y_scale      = wsb + L.ys_off;
+        p.ys_kb_stride = L.ys_kb_stride;
+        const int64_t n16 = (L.ys_kb_stride * (I / 32) + 15) / 16; // the buffer is a multiple of 256 bytes
+        hipLaunchKernelGGL(fill_u32x4_kernel, dim3((unsigned)std::min<int64_t>(ceil_div<int64_t>(n16, 256), 4096)), dim3(256), 0,
+                           stream, reinterpret_cast<uint4*>(p.y_scale), n16, 0x7f7f7f7fu);
+    }
     rc = launch_grouped_gemm(prec, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p, L.max_tiles, stream);
     if(rc != MI355_MOE_OK)
         return rc;
@@ -826,7 +851,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
         KernelTimer timer(MI355_MOE_K_COMBINE, stream);
         hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + L.p_off, inv,
                            static_cast<const float*>(a.p_sorted_expert_weights), static_cast<unsigned char*>(a.c_ptr), K, H,
-                           (int64_t)a.stride_C * 2, 1);
+                           (int64_t)a.stride_C * 2, 1, f8 ? static_cast<const float*>(a.scale_m) : nullptr);
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;

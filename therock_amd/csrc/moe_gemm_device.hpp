@@ -60,6 +60,8 @@ struct GemmParams
     // n_out, k]; a tile then covers twice the Y columns and y = act(gate)); act: 0 = gelu (erf form), 1 = silu
     int gate_only;
     int act;
+    // fp8 gate+up GEMM of the stand-alone entry point: write bf16 instead of e4m3 with block scales
+    int y_bf16;
 };
 
 // byte offset of K byte kb of row `row` in the slab-major Y layout
@@ -294,10 +296,11 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
         for(int v = 0; v < 16; v++)
             y[v] *= static_cast<float>(acc_up[v]) * (sa * us[v]);
     }
-    constexpr int y_b  = MODE == kFp8 ? 1 : 2;
+    const bool as_fp8  = MODE == kFp8 && !p.y_bf16;
+    const int y_b      = as_fp8 ? 1 : 2;
     unsigned char* dst = p.y_slab > 0 ? p.out + y_slab_offset(grow, col0 * y_b, p.y_slab)
                                       : p.out + grow * p.out_row_bytes + (int64_t)col0 * y_b;
-    if constexpr(MODE == kFp8)
+    if(as_fp8)
     {
         float amax = 0.f;
 #pragma unroll
