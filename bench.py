@@ -164,6 +164,61 @@ def run_router(cfg, steps, warmup):
             "GBps": byt / ms / 1e6 if ms > 0 else None}
 
 
+def run_neighbours(cfg, inp, buf, steps):
+    """The callers and data formats either side of the path, on the headline workload's shapes: per-token
+    activation quantisation, MoE smooth-quant, the weight pre-shuffle (a slice of the experts), and the gate+up /
+    down GEMMs as stand-alone launches on the sorted arrays the path has just produced.  Wall time per call from
+    events on the launch stream; bytes are the algorithmic ones of each step."""
+    import torch
+
+    import therock_amd as ta
+
+    T, H, I, E, K = cfg.tokens, cfg.hidden, cfg.inter, cfg.experts, cfg.topk
+    qd = "fp8" if cfg.dtype == "fp8" else "int8"
+    out = {}
+
+    def timed(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn((T, H), device="cuda", generator=g).to(torch.bfloat16)
+    ms = timed(lambda: ta.rowwise_quant(x, qd), steps)
+    out["rowwise_quant"] = {"ms": ms, "GBps": T * H * 3 / ms / 1e6, "what": f"[{T}, {H}] bf16 -> {qd} + scale"}
+    sm = torch.rand((E, H), device="cuda", generator=g) + 0.5
+    ms = timed(lambda: ta.moe_smoothquant(x, sm, inp["topk_ids"], qd), max(2, steps // 4))
+    out["moe_smoothquant"] = {"ms": ms, "GBps": (T * H * 2 + K * T * H) / ms / 1e6,
+                              "what": f"[{T}, {H}] bf16 -> [{K}, {T}, {H}] {qd} + scales"}
+    del sm
+    ne = min(E, 32)
+    w = inp["d"][:ne]
+    ms = timed(lambda: ta.permute_weights(w), 3)
+    out["permute_weights"] = {"ms": ms, "GBps": 2 * w.numel() * w.element_size() / ms / 1e6,
+                              "what": f"{ne} experts of d [{H}, {I}] to ck_tile's pre-shuffled layout"}
+    if cfg.dtype in ("bf16", "fp8"):
+        y = torch.empty((T * K, I), dtype=torch.bfloat16, device="cuda")
+        ms = timed(lambda: ta.moe_flatmm(ta.GEMM1_GATE_UP, inp["a"], inp["g"], y, buf.sorted_ids, buf.sorted_eid, buf.total,
+                                         T, K, cfg.unit, scale_m=inp["a_scale"], scale_n=inp["g_scale"]), max(2, steps // 4))
+        out["flatmm_gate_up"] = {"ms": ms, "tflops": 4.0 * T * K * H * I / ms / 1e9, "what": "stand-alone gate+up GEMM, bf16 C"}
+        if cfg.dtype == "fp8":
+            yq, ys = ta.rowwise_quant(y, "fp8")
+        else:
+            yq, ys = y, None
+        c = torch.zeros((T, H), dtype=torch.bfloat16, device="cuda")
+        ms = timed(lambda: ta.moe_flatmm(ta.GEMM2, yq, inp["d"], c, buf.sorted_ids, buf.sorted_eid, buf.total, T, K, cfg.unit,
+                                         sorted_weights=buf.sorted_w, scale_m=ys, scale_n=inp["d_scale"]), max(2, steps // 4))
+        out["flatmm_down"] = {"ms": ms, "tflops": 2.0 * T * K * H * I / ms / 1e9,
+                              "what": "stand-alone down GEMM + combine, added to bf16 C"}
+    return out
+
+
 def cpu_baseline(cfg, inp, max_rows=256):
     """ck_tile's own host reference (oracle/_ref) timed on this machine's cores on a bounded
     sample of the workload: every row routed to one expert (T'=rows, E'=1, K'=1), operands
@@ -250,6 +305,11 @@ def main():
             log(f"[bench] cpu baseline: {cpu}")
         except Exception as e:  # the baseline is a report, never a reason to lose the measurement
             log(f"[bench] cpu baseline failed: {e!r}")
+    try:
+        neighbours = run_neighbours(cfg, inp, buf, a.steps)
+        log(f"[bench] neighbours: {neighbours}")
+    except Exception as e:
+        neighbours = {"error": repr(e)}
     del inp, buf
     torch.cuda.empty_cache()
     try:
@@ -286,7 +346,7 @@ def main():
                    "path": "moe_sorting + gemm0(gate,up,SiLU*up) + gemm1(down) + combine, one stream"},
         "frac_of_mfma_peak": res["frac_mfma_peak"], "tokens_per_s": res["tokens_per_s"],
         "hbm_GBps": res["hbm_GBps"], "kernel_avg_ms": res["kernel_avg_ms"], "gemm0_tflops": res["gemm0_tflops"],
-        "gemm1_tflops": res["gemm1_tflops"], "roofline": roof, "cpu_baseline": cpu, "router": router, "workloads": others,
+        "gemm1_tflops": res["gemm1_tflops"], "roofline": roof, "cpu_baseline": cpu, "router": router, "neighbours": neighbours, "workloads": others,
     }
     print(json.dumps(line), flush=True)
 

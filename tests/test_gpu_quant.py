@@ -19,7 +19,8 @@ def _raw(t):
     return t.view(torch.uint8).cpu().numpy() if t.element_size() == 1 and t.dtype != torch.int8 else t.cpu().numpy()
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 32), (64, 4096), (513, 7168), (7, 1000)])
+# 7168: 16-byte pieces kept in registers; 12288: more pieces than the register cache holds; 1004, 100: scalar path
+@pytest.mark.parametrize("rows,cols", [(1, 32), (64, 4096), (513, 7168), (7, 1000), (33, 12288), (5, 1004), (3, 100)])
 @pytest.mark.parametrize("kind", ["int8", "fp8"])
 def test_rowwise_quant(rows, cols, kind):
     import torch
@@ -27,15 +28,25 @@ def test_rowwise_quant(rows, cols, kind):
 
     rng = np.random.default_rng(rows + cols)
     x = _bf16((rng.standard_normal((rows, cols)) * rng.choice([1e-2, 1, 30], size=(rows, 1))).astype(np.float32))
+    x[rows // 2] = 0  # an all-zero row: scale 1, zeros
     q, s = ta.rowwise_quant(x, kind)
     torch.cuda.synchronize()
     dt = oracle.DT_I8 if kind == "int8" else oracle.DT_E4M3
     rq, rs = oracle.rowwise_quant(x.float().cpu().numpy(), dt)
     assert np.array_equal(s.cpu().numpy(), rs)
     assert np.array_equal(_raw(q), rq)
+    # the same rows 2 bytes off a 16-byte boundary: the scalar path
+    flat = torch.zeros((rows * cols + 8,), dtype=torch.bfloat16, device="cuda")
+    shifted = flat[1:1 + rows * cols].view(rows, cols)
+    shifted.copy_(x)
+    assert shifted.data_ptr() % 16 == 2
+    q2, s2 = ta.rowwise_quant(shifted, kind)
+    torch.cuda.synchronize()
+    assert np.array_equal(s2.cpu().numpy(), rs) and np.array_equal(_raw(q2), rq)
 
 
-@pytest.mark.parametrize("tokens,hidden,experts,topk", [(1, 64, 4, 2), (64, 4096, 128, 8), (300, 1024, 8, 2), (17, 7168, 256, 8)])
+@pytest.mark.parametrize("tokens,hidden,experts,topk", [(1, 64, 4, 2), (64, 4096, 128, 8), (300, 1024, 8, 2), (17, 7168, 256, 8),
+                                                         (9, 10240, 4, 3), (5, 100, 3, 2)])
 @pytest.mark.parametrize("kind", ["int8", "fp8"])
 def test_moe_smoothquant(tokens, hidden, experts, topk, kind):
     import torch

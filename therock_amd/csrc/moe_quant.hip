@@ -9,47 +9,140 @@ namespace mi355 {
 using namespace gemm;
 namespace {
 
-// per-row dynamic quantisation bf16 -> e4m3 / int8
+// one value -> e4m3 (round to nearest even, saturating) or int8 (saturate, then ck_tile's float -> int8
+// static_cast: truncation toward zero)
 template <bool FP8>
+__device__ inline unsigned char quantise_one(float v)
+{
+    if constexpr(FP8)
+    {
+        const float cl = fminf(fmaxf(v, -448.f), 448.f);
+        return static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
+    }
+    else
+    {
+        const float cl = fminf(fmaxf(v, -128.f), 127.f);
+        return static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
+    }
+}
+
+__device__ inline float block_max_256(float v, float* s_red)
+{
+#pragma unroll
+    for(int d = 32; d > 0; d >>= 1)
+        v = fmaxf(v, __shfl_xor(v, d));
+    if((threadIdx.x & 63) == 0)
+        s_red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+}
+
+// Per-row dynamic quantisation of one row by one 256-thread workgroup: xr bf16 (times sr fp32 when SMOOTH),
+// scale = amax / qmax, q = quantise(value / scale).  With VEC the row is walked in 16-byte pieces of 8 elements
+// (cols % 8 == 0, 16-byte aligned rows); the first kCache pieces of every thread stay in registers between the
+// two passes, so rows of up to 8192 columns are read once.  Returns the row's amax to every thread.
+constexpr int kQuantCache = 4;
+template <bool FP8, bool SMOOTH, bool VEC>
+__device__ inline float quantise_row(const uint16_t* __restrict__ xr, const float* __restrict__ sr, int cols,
+                                     unsigned char* __restrict__ qr, float* s_red, bool unit_scale_when_zero, float* scale_out)
+{
+    const float qmx = FP8 ? 448.0f : 127.0f;
+    if constexpr(VEC)
+    {
+        const int chunks = cols >> 3;
+        float v[kQuantCache][8];
+        auto load = [&](int c, float (&o)[8]) {
+            const uint4 r = *reinterpret_cast<const uint4*>(xr + c * 8);
+            const uint32_t d[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+            for(int i = 0; i < 4; i++)
+            {
+                o[2 * i]     = __uint_as_float(d[i] << 16);
+                o[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+            }
+            if constexpr(SMOOTH)
+            {
+                const float4 s0 = *reinterpret_cast<const float4*>(sr + c * 8);
+                const float4 s1 = *reinterpret_cast<const float4*>(sr + c * 8 + 4);
+                o[0] *= s0.x; o[1] *= s0.y; o[2] *= s0.z; o[3] *= s0.w;
+                o[4] *= s1.x; o[5] *= s1.y; o[6] *= s1.z; o[7] *= s1.w;
+            }
+        };
+        float amax = 0.f;
+#pragma unroll
+        for(int j = 0; j < kQuantCache; j++)
+        {
+            const int c = threadIdx.x + 256 * j;
+            if(c < chunks)
+            {
+                load(c, v[j]);
+#pragma unroll
+                for(int i = 0; i < 8; i++)
+                    amax = fmaxf(amax, fabsf(v[j][i]));
+            }
+        }
+        for(int c = threadIdx.x + 256 * kQuantCache; c < chunks; c += 256)
+        {
+            float t[8];
+            load(c, t);
+#pragma unroll
+            for(int i = 0; i < 8; i++)
+                amax = fmaxf(amax, fabsf(t[i]));
+        }
+        amax          = block_max_256(amax, s_red);
+        const float s = (amax > 0.f || !unit_scale_when_zero) ? amax / qmx : 1.0f;
+        if(threadIdx.x == 0)
+            *scale_out = s;
+        auto store = [&](int c, const float (&o)[8]) {
+            uint32_t w[2] = {0u, 0u};
+#pragma unroll
+            for(int i = 0; i < 8; i++)
+                w[i >> 2] |= static_cast<uint32_t>(quantise_one<FP8>(o[i] / s)) << (8 * (i & 3));
+            *reinterpret_cast<uint2*>(qr + c * 8) = make_uint2(w[0], w[1]);
+        };
+#pragma unroll
+        for(int j = 0; j < kQuantCache; j++)
+        {
+            const int c = threadIdx.x + 256 * j;
+            if(c < chunks)
+                store(c, v[j]);
+        }
+        for(int c = threadIdx.x + 256 * kQuantCache; c < chunks; c += 256)
+        {
+            float t[8];
+            load(c, t);
+            store(c, t);
+        }
+        return amax;
+    }
+    else
+    {
+        float amax = 0.f;
+        for(int c = threadIdx.x; c < cols; c += 256)
+            amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c]) * (SMOOTH ? sr[c] : 1.0f)));
+        amax          = block_max_256(amax, s_red);
+        const float s = (amax > 0.f || !unit_scale_when_zero) ? amax / qmx : 1.0f;
+        if(threadIdx.x == 0)
+            *scale_out = s;
+        for(int c = threadIdx.x; c < cols; c += 256)
+            qr[c] = quantise_one<FP8>((bf16_bits_to_float(xr[c]) * (SMOOTH ? sr[c] : 1.0f)) / s);
+        return amax;
+    }
+}
+
+// per-row dynamic quantisation bf16 -> e4m3 / int8
+template <bool FP8, bool VEC>
 __global__ __launch_bounds__(256) void rowwise_quant_kernel(const uint16_t* __restrict__ x, int cols,
                                                              int64_t stride_x, unsigned char* __restrict__ q,
                                                              float* __restrict__ scale)
 {
     __shared__ float s_red[4];
-    const int64_t row  = blockIdx.x;
-    const uint16_t* xr = x + row * stride_x;
-    float amax         = 0.f;
-    for(int c = threadIdx.x; c < cols; c += 256)
-        amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c])));
-#pragma unroll
-    for(int d = 32; d > 0; d >>= 1)
-        amax = fmaxf(amax, __shfl_xor(amax, d));
-    if((threadIdx.x & 63) == 0)
-        s_red[threadIdx.x >> 6] = amax;
-    __syncthreads();
-    amax            = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    const float qmx = FP8 ? 448.0f : 127.0f;
-    const float s   = amax > 0.f ? amax / qmx : 1.0f;
-    if(threadIdx.x == 0)
-        scale[row] = s;
-    for(int c = threadIdx.x; c < cols; c += 256)
-    {
-        const float v = bf16_bits_to_float(xr[c]) / s;
-        if constexpr(FP8)
-        {
-            const float cl = fminf(fmaxf(v, -448.f), 448.f);
-            q[row * cols + c] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
-        }
-        else
-        {
-            // ck_tile's float -> int8 conversion is a static_cast: truncation toward zero
-            const float cl = fminf(fmaxf(v, -128.f), 127.f);
-            q[row * cols + c] = static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
-        }
-    }
+    const int64_t row = blockIdx.x;
+    quantise_row<FP8, false, VEC>(x + row * stride_x, nullptr, cols, q + row * cols, s_red, true, scale + row);
 }
 
-// MoE smooth-quant: row (slot k, token t) = x[t, :] * smscale[expert(t, k), :], per-row dynamic quantisation
+// MoE smooth-quant: row (slot k, token t) = x[t, :] * smscale[expert(t, k), :], per-row dynamic quantisation.
+// Scalar form: one workgroup per (token, slot).
 template <bool FP8>
 __global__ __launch_bounds__(256) void moe_smoothquant_kernel(const uint16_t* __restrict__ x,
                                                                const float* __restrict__ smscale,
@@ -62,36 +155,99 @@ __global__ __launch_bounds__(256) void moe_smoothquant_kernel(const uint16_t* __
     const int k = blockIdx.y;
     int e       = topk_ids[(int64_t)t * topk + k];
     e           = min(max(e, 0), experts - 1);
-    const uint16_t* xr = x + (int64_t)t * x_stride;
-    const float* sr    = smscale + (int64_t)e * hidden;
-    float amax         = 0.f;
-    for(int c = threadIdx.x; c < hidden; c += 256)
-        amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c]) * sr[c]));
-#pragma unroll
-    for(int d = 32; d > 0; d >>= 1)
-        amax = fmaxf(amax, __shfl_xor(amax, d));
-    if((threadIdx.x & 63) == 0)
-        s_red[threadIdx.x >> 6] = amax;
-    __syncthreads();
-    amax            = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    const float qmx = FP8 ? 448.0f : 127.0f;
-    const float ys  = amax / qmx;
     const int64_t r = (int64_t)k * tokens + t;
-    if(threadIdx.x == 0)
-        yscale[r] = ys;
-    unsigned char* qr = qy + r * y_stride;
-    for(int c = threadIdx.x; c < hidden; c += 256)
-    {
-        const float v = (bf16_bits_to_float(xr[c]) * sr[c]) / ys;
-        if constexpr(FP8)
+    quantise_row<FP8, true, false>(x + (int64_t)t * x_stride, smscale + (int64_t)e * hidden, hidden, qy + r * y_stride, s_red,
+                                   false, yscale + r);
+}
+
+// Vector form (hidden % 8 == 0, aligned rows): one workgroup per token walks its slots, so the token's row is
+// read once (its first kQuantCache pieces per thread stay in registers) and only the experts' smooth scales and
+// the quantised rows move per slot.
+template <bool FP8>
+__global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t* __restrict__ x,
+                                                                   const float* __restrict__ smscale,
+                                                                   const int* __restrict__ topk_ids, int tokens,
+                                                                   int hidden, int experts, int topk, int64_t x_stride,
+                                                                   int64_t y_stride, unsigned char* __restrict__ qy,
+                                                                   float* __restrict__ yscale)
+{
+    __shared__ float s_red[2][4];
+    const int t        = blockIdx.x;
+    const uint16_t* xr = x + (int64_t)t * x_stride;
+    const int chunks   = hidden >> 3;
+    const float qmx    = FP8 ? 448.0f : 127.0f;
+    auto load_x = [&](int c, float (&o)[8]) {
+        const uint4 r = *reinterpret_cast<const uint4*>(xr + c * 8);
+        const uint32_t d[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for(int i = 0; i < 4; i++)
         {
-            const float cl = fminf(fmaxf(v, -448.f), 448.f);
-            qr[c] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(cl, cl, 0, false) & 0xff);
+            o[2 * i]     = __uint_as_float(d[i] << 16);
+            o[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
         }
-        else
+    };
+    auto times_sm = [&](const float* sr, int c, const float (&in)[8], float (&o)[8]) {
+        const float4 s0 = *reinterpret_cast<const float4*>(sr + c * 8);
+        const float4 s1 = *reinterpret_cast<const float4*>(sr + c * 8 + 4);
+        o[0] = in[0] * s0.x; o[1] = in[1] * s0.y; o[2] = in[2] * s0.z; o[3] = in[3] * s0.w;
+        o[4] = in[4] * s1.x; o[5] = in[5] * s1.y; o[6] = in[6] * s1.z; o[7] = in[7] * s1.w;
+    };
+    float xv[kQuantCache][8];
+#pragma unroll
+    for(int j = 0; j < kQuantCache; j++)
+        if(threadIdx.x + 256 * j < chunks)
+            load_x(threadIdx.x + 256 * j, xv[j]);
+    for(int k = 0; k < topk; k++)
+    {
+        int e = topk_ids[(int64_t)t * topk + k];
+        e     = min(max(e, 0), experts - 1);
+        const float* sr = smscale + (int64_t)e * hidden;
+        float v[kQuantCache][8];
+        float amax = 0.f;
+#pragma unroll
+        for(int j = 0; j < kQuantCache; j++)
         {
-            const float cl = fminf(fmaxf(v, -128.f), 127.f);
-            qr[c] = static_cast<unsigned char>(static_cast<signed char>(static_cast<int>(cl)));
+            const int c = threadIdx.x + 256 * j;
+            if(c < chunks)
+            {
+                times_sm(sr, c, xv[j], v[j]);
+#pragma unroll
+                for(int i = 0; i < 8; i++)
+                    amax = fmaxf(amax, fabsf(v[j][i]));
+            }
+        }
+        for(int c = threadIdx.x + 256 * kQuantCache; c < chunks; c += 256)
+        {
+            float a[8], b[8];
+            load_x(c, a);
+            times_sm(sr, c, a, b);
+#pragma unroll
+            for(int i = 0; i < 8; i++)
+                amax = fmaxf(amax, fabsf(b[i]));
+        }
+        amax            = block_max_256(amax, s_red[k & 1]); // two buffers: one barrier per slot suffices
+        const float ys  = amax / qmx;
+        const int64_t r = (int64_t)k * tokens + t;
+        if(threadIdx.x == 0)
+            yscale[r] = ys;
+        unsigned char* qr = qy + r * y_stride;
+        auto store = [&](int c, const float (&o)[8]) {
+            uint32_t w[2] = {0u, 0u};
+#pragma unroll
+            for(int i = 0; i < 8; i++)
+                w[i >> 2] |= static_cast<uint32_t>(quantise_one<FP8>(o[i] / ys)) << (8 * (i & 3));
+            *reinterpret_cast<uint2*>(qr + c * 8) = make_uint2(w[0], w[1]);
+        };
+#pragma unroll
+        for(int j = 0; j < kQuantCache; j++)
+            if(threadIdx.x + 256 * j < chunks)
+                store(threadIdx.x + 256 * j, v[j]);
+        for(int c = threadIdx.x + 256 * kQuantCache; c < chunks; c += 256)
+        {
+            float a[8], b[8];
+            load_x(c, a);
+            times_sm(sr, c, a, b);
+            store(c, b);
         }
     }
 }
@@ -166,17 +322,21 @@ int launch_moe_smoothquant(const mi355_moe_smoothquant_args& a, int32_t q_dtype,
     if(!a.p_x || !a.p_smscale || !a.p_topk_ids || !a.p_yscale || !a.p_qy)
         return fail(MI355_MOE_E_INVALID, "moe_smoothquant: null pointer");
     KernelTimer timer(MI355_MOE_K_QUANT, stream);
-    const dim3 grid((unsigned)a.tokens, (unsigned)a.topk);
+    // 16-byte pieces of 8 elements when every row starts on a 16-byte (output: 8-byte) boundary
+    const bool vec = a.hidden_size % 8 == 0 && a.x_stride % 8 == 0 && a.y_stride % 8 == 0 &&
+                     reinterpret_cast<uintptr_t>(a.p_x) % 16 == 0 && reinterpret_cast<uintptr_t>(a.p_smscale) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(a.p_qy) % 8 == 0;
+    auto launch = [&](auto kernel, dim3 grid) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
+                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
+                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
+                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
+    };
+    const dim3 per_token((unsigned)a.tokens), per_row((unsigned)a.tokens, (unsigned)a.topk);
     if(q_dtype == MI355_MOE_FP8)
-        hipLaunchKernelGGL(moe_smoothquant_kernel<true>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
-                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
-                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
-                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
+        vec ? launch(moe_smoothquant_vec_kernel<true>, per_token) : launch(moe_smoothquant_kernel<true>, per_row);
     else
-        hipLaunchKernelGGL(moe_smoothquant_kernel<false>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(a.p_x),
-                           static_cast<const float*>(a.p_smscale), static_cast<const int*>(a.p_topk_ids), a.tokens,
-                           a.hidden_size, a.experts, a.topk, (int64_t)a.x_stride, (int64_t)a.y_stride,
-                           static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
+        vec ? launch(moe_smoothquant_vec_kernel<false>, per_token) : launch(moe_smoothquant_kernel<false>, per_row);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }
@@ -193,14 +353,16 @@ int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stri
     if(rows > 0x7fffffff)
         return fail(MI355_MOE_E_INVALID, "rowwise_quant: too many rows");
     KernelTimer timer(MI355_MOE_K_QUANT, stream);
+    const bool vec = cols % 8 == 0 && stride_x % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(q) % 8 == 0;
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)rows), dim3(256), 0, stream, static_cast<const uint16_t*>(x), cols,
+                           stride_x, static_cast<unsigned char*>(q), static_cast<float*>(scale));
+    };
     if(q_dtype == MI355_MOE_FP8)
-        hipLaunchKernelGGL(rowwise_quant_kernel<true>, dim3((unsigned)rows), dim3(256), 0, stream,
-                           static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),
-                           static_cast<float*>(scale));
+        vec ? launch(rowwise_quant_kernel<true, true>) : launch(rowwise_quant_kernel<true, false>);
     else
-        hipLaunchKernelGGL(rowwise_quant_kernel<false>, dim3((unsigned)rows), dim3(256), 0, stream,
-                           static_cast<const uint16_t*>(x), cols, stride_x, static_cast<unsigned char*>(q),
-                           static_cast<float*>(scale));
+        vec ? launch(rowwise_quant_kernel<false, true>) : launch(rowwise_quant_kernel<false, false>);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }
