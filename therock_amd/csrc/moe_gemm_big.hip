@@ -425,12 +425,16 @@ int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
 {
     constexpr bool kMx  = MODE == kFp8 && !GEMM0;
     const size_t lds    = kMx ? kLdsBytes : kYsOffset;
-    static bool attr_ok = false; // the limit is a per-function attribute; setting it again is harmless
-    if(!attr_ok)
+    // the dynamic LDS limit is an attribute of the function on one device: set once per device
+    static bool attr_ok[64] = {};
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if(dev < 0 || dev >= 64 || !attr_ok[dev])
     {
         MI355_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_big_kernel<MODE, GEMM0>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_ok = true;
+        if(dev >= 0 && dev < 64)
+            attr_ok[dev] = true;
     }
     const int grid = round_up(max_tiles * p.n_ntiles, 8);
     if(grid <= 0)
