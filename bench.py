@@ -277,8 +277,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py: this build measures one GPU only; run with --gpus 1 (the path is single-GPU, "
-                 "how it would shard across GPUs is described in DESIGN.md)")
+        sys.exit("bench.py: this build measures one GPU only; run with --gpus 1 (the path is single-GPU: across "
+                 "GPUs the experts would be sharded with the sort's local-expert mask, which is not built here)")
     import torch
 
     from therock_amd import inputs as mi

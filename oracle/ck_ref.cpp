@@ -107,7 +107,7 @@ ck_ref_moe_sorting(const int32_t* topk_ids, const float* weights, const int32_t*
     return cnt;
 }
 
-// bf16 activations and weights, bf16 output (BASELINE configs 1, 2, 5)
+// bf16 activations and weights, bf16 output (the bf16 benchmark configurations)
 __attribute__((visibility("default"))) int
 ck_ref_fused_moe_bf16(const void* a, const void* g, const void* d, void* o, const int32_t* sorted_ids,
                       const float* sorted_w, const int32_t* sorted_eid, int32_t post_pad,
