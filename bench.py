@@ -305,11 +305,13 @@ def main():
             log(f"[bench] cpu baseline: {cpu}")
         except Exception as e:  # the baseline is a report, never a reason to lose the measurement
             log(f"[bench] cpu baseline failed: {e!r}")
-    try:
-        neighbours = run_neighbours(cfg, inp, buf, a.steps)
-        log(f"[bench] neighbours: {neighbours}")
-    except Exception as e:
-        neighbours = {"error": repr(e)}
+    neighbours = None
+    if not a.headline_only:  # (a profiled --headline-only run holds launches of the path and the router only)
+        try:
+            neighbours = run_neighbours(cfg, inp, buf, a.steps)
+            log(f"[bench] neighbours: {neighbours}")
+        except Exception as e:
+            neighbours = {"error": repr(e)}
     del inp, buf
     torch.cuda.empty_cache()
     try:
