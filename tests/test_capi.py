@@ -84,3 +84,19 @@ def test_python_mirror_rejects_unknown_traits_without_touching_the_gpu():
     assert ta.fused_moe(ta.fused_moe_traits(prec_i="fp16", prec_w="fp16"), ta.fused_moe_args()) == -1.0
     with pytest.raises(ValueError):
         ta.fused_moe_traits(prec_i="fp4").pod()
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """There is no CPU fallback: without the built HIP library every entry point of the Python mirror raises."""
+    import therock_amd as ta
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmi355_moe.so"))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ta.moe_sorting_get_workspace_size(64, 8, 2)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ta.fused_moe(ta.fused_moe_traits(), ta.fused_moe_args())
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run(["python", os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU only" in r.stderr
