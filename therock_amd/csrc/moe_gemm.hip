@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
 
     // ---- work item: XCD x gets a contiguous range of the work list (workgroup ids are dealt
     // round-robin to the 8 XCDs), and inside an expert the M tiles of one weight tile are adjacent
-    const TileRef tile = lookup_tile(p.tile_map, p.n_ntiles, blockIdx.x);
+    const TileRef tile = lookup_tile(p.tile_map, p.n_ntiles, p.max_tiles, blockIdx.x);
     if(!tile.ok)
         return;
     const int expert = tile.expert;
@@ -478,6 +478,7 @@ int launch_grouped_gemm(int prec, bool gemm0, int mblk, bool use_decode, GemmPar
 {
     // output columns per tile: the tile's weight rows, halved where gate and up rows share them
     const int pair = gemm0 && !p.gate_only ? 2 : 1;
+    p.max_tiles    = max_tiles;
     p.n_ntiles     = ceil_div(p.n_out, (use_decode ? decode_tile_cols(false) : 256) / pair);
     if(use_decode)
         return launch_gemm_decode(prec, gemm0, p, max_tiles, stream);

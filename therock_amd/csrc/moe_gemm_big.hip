@@ -117,7 +117,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     const int ww   = wave & 3;  // weight-row quarter
 
     // ---- work item (same XCD-aware order as moe_gemm_kernel)
-    const TileRef tile = lookup_tile(p.tile_map, p.n_ntiles, blockIdx.x);
+    const TileRef tile = lookup_tile<true>(p.tile_map, p.n_ntiles, p.max_tiles, blockIdx.x);
     if(!tile.ok)
         return;
     const int expert = tile.expert;
@@ -436,7 +436,7 @@ int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
         if(dev >= 0 && dev < 64)
             attr_ok[dev] = true;
     }
-    const int grid = round_up(max_tiles * p.n_ntiles, 8);
+    const int grid = round_up(max_tiles * p.n_ntiles, 256); // whole rounds of 32-item chunks over the 8 XCDs
     if(grid <= 0)
         return MI355_MOE_OK;
     KernelTimer timer(GEMM0 ? MI355_MOE_K_GEMM0 : MI355_MOE_K_GEMM1, stream);

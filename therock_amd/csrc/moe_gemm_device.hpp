@@ -62,6 +62,7 @@ struct GemmParams
     int act;
     // fp8 gate+up GEMM of the stand-alone entry point: write bf16 instead of e4m3 with block scales
     int y_bf16;
+    int max_tiles; // entries the tile list has room for (upper bound of live tiles)
 };
 
 // byte offset of K byte kb of row `row` in the slab-major Y layout
@@ -76,27 +77,46 @@ __device__ inline int64_t slot_row(int sid, int topk)
     return (int64_t)(sid & 0xffffff) * topk + static_cast<int>(static_cast<uint32_t>(sid) >> 24);
 }
 
-// Work item -> tile.  XCD x gets a contiguous range of the work list (workgroup ids are dealt
-// round-robin to the 8 XCDs); inside an expert the row tiles of one weight tile are adjacent.  One
-// entry of the list describes the whole expert, so a single load resolves any of its tiles.
+// Work item -> tile.  Workgroup ids are dealt round-robin to the 8 XCDs; inside an expert the row tiles of one
+// weight tile are adjacent.  One entry of the list describes the whole expert, so a single load resolves any of
+// its tiles.  Two orders: XCD x takes a contiguous eighth of the work list (the weight-streaming kernels: every
+// XCD walks its own region of the weights), or chunks of 32 consecutive work items go round-robin to the XCDs (the
+// large-tile kernel: tiles of hot and cold experts cost very different amounts, and chunks spread them - 5 % on
+// the Zipf-routed workload; the position then does not depend on the live tile count, so that count and the
+// tile's entry are fetched together instead of one after the other).
 struct TileRef
 {
     int expert, row0, nrows, nt; // nt: column tile
     int expert_tiles;            // row tiles of this expert (each of them re-reads the same weight tiles)
     bool ok;
 };
-__device__ inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_ntiles, int block)
+template <bool CHUNKED = false>
+__device__ inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_ntiles, int max_tiles, int block)
 {
     TileRef t;
-    const int total   = tile_map[0] * n_ntiles;
-    const int per_xcd = ceil_div(total, 8);
-    const int slot    = block >> 3;
-    const int work    = (block & 7) * per_xcd + slot;
-    t.ok              = slot < per_xcd && work < total;
-    const int t0      = t.ok ? work / n_ntiles : 0;
-    const int4* e     = reinterpret_cast<const int4*>(tile_map + kMapHdr + t0 * kMapEnt);
-    const int4 a      = e[0]; // expert, row0, nrows, first tile of the expert
-    const int4 b      = e[1]; // tiles of the expert, its first row, its rows, rows per tile
+    const int slot = block >> 3;
+    int work, total;
+    if constexpr(CHUNKED)
+    {
+        work  = ((((slot >> 5) << 3) + (block & 7)) << 5) + (slot & 31);
+        t.ok  = true;
+    }
+    else
+    {
+        total             = tile_map[0] * n_ntiles;
+        const int per_xcd = ceil_div(total, 8);
+        work              = (block & 7) * per_xcd + slot;
+        t.ok              = slot < per_xcd && work < total;
+    }
+    // (chunked: the entry is fetched before the item is known to be live, so the index is kept inside the list)
+    const int t0  = CHUNKED ? min(work / n_ntiles, max_tiles - 1) : (t.ok ? work / n_ntiles : 0);
+    const int4* e = reinterpret_cast<const int4*>(tile_map + kMapHdr + t0 * kMapEnt);
+    if constexpr(CHUNKED)
+        total = tile_map[0] * n_ntiles;
+    const int4 a  = e[0]; // expert, row0, nrows, first tile of the expert
+    const int4 b  = e[1]; // tiles of the expert, its first row, its rows, rows per tile
+    if constexpr(CHUNKED)
+        t.ok = work < total;
     const int rel     = work - a.w * n_ntiles;
     t.nt              = rel / max(b.x, 1);
     const int j       = rel - t.nt * b.x;
