@@ -163,6 +163,50 @@ def test_gelu_and_gate_only(dtype, activation, gate_only):
     check(mi.MoeConfig("a", 96, 256, 256, 10, 3, dtype, "softmax_renorm"), seed=4, unfused=True, **kw)
 
 
+def _check_routing(cfg, ids, w, seed=0):
+    """check() with a hand-made routing instead of the generator's."""
+    from tests.gpu_util import rel_l2, run_fused_moe
+    inp = mi.make_inputs_np(cfg, seed)
+    inp["topk_ids"], inp["topk_weight"] = ids.astype(np.int32), w.astype(np.float32)
+    print(f"fused_moe {cfg} hand-made routing", flush=True)
+    got, buf = run_fused_moe(cfg, inp)
+    ref, s = oracle_out(cfg, inp)
+    assert int(buf.total[0]) == s[3]
+    assert np.array_equal(buf.sorted_ids[:s[3]].cpu().numpy(), s[0][:s[3]])
+    err = rel_l2(oracle.bf16_to_f32(got), ref)
+    print(f"  rel-L2 = {err:.3e}", flush=True)
+    assert err <= TOL[cfg.dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
+def test_extreme_routings(dtype):
+    rng = np.random.default_rng(5)
+    # every token picks the same experts: one bucket per slot holds all tokens, every other expert is empty
+    cfg = mi.MoeConfig("x", 700, 256, 256, 16, 3, dtype, "softmax")
+    _check_routing(cfg, np.tile(np.array([11, 2, 7]), (cfg.tokens, 1)), rng.random((cfg.tokens, 3)))
+    # top-k = experts: every token visits every expert, in a different order per token
+    cfg = mi.MoeConfig("x", 40, 128, 128, 8, 8, dtype, "softmax")
+    _check_routing(cfg, np.stack([rng.permutation(8) for _ in range(cfg.tokens)]), rng.random((cfg.tokens, 8)))
+    # a single expert, a single slot; zero and negative top-k weights
+    cfg = mi.MoeConfig("x", 33, 128, 128, 1, 1, dtype, "softmax")
+    _check_routing(cfg, np.zeros((cfg.tokens, 1)), rng.standard_normal((cfg.tokens, 1)) * (rng.random((cfg.tokens, 1)) < 0.7))
+    # the most experts the path takes, a wide top-k, a handful of tokens
+    cfg = mi.MoeConfig("x", 5, 128, 128, 1024, 48, dtype, "softmax")
+    _check_routing(cfg, np.stack([rng.permutation(1024)[:48] for _ in range(cfg.tokens)]), rng.random((cfg.tokens, 48)))
+
+
+def test_no_tokens():
+    import torch
+    import therock_amd as ta
+    t = ta.fused_moe_traits()
+    buf = ta.MoeBuffers(t, 0, 4, 2, 128, 128, "cuda")
+    z = lambda *sh, dt=torch.bfloat16: torch.zeros(sh, dtype=dt, device="cuda")
+    args = ta.make_args(t, buf, z(0, 128), z(4, 256, 128), z(4, 128, 128), z(0, 2, dt=torch.int32), z(0, 2, dt=torch.float32))
+    args.stride_token = 128
+    assert ta.fused_moe(t, args) == 0.0
+    torch.cuda.synchronize()
+
+
 def test_traits_without_kernel_return_minus_one():
     import torch
     import therock_amd as ta

@@ -568,6 +568,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     int rc = check_traits(t);
     if(rc != MI355_MOE_OK)
         return rc;
+    if(a.num_tokens == 0)
+        return MI355_MOE_OK; // an empty batch: nothing to compute, and its tensors may have no storage
     if(!a.a_ptr || !a.g_ptr || !a.d_ptr || !a.o_ptr || !a.sorted_token_ids_ptr || !a.sorted_weight_ptr ||
        !a.sorted_expert_ids_ptr || !a.num_sorted_tiles_ptr)
         return fail(MI355_MOE_E_INVALID, "fused_moegemm: null tensor pointer");
