@@ -195,6 +195,46 @@ def test_extreme_routings(dtype):
     _check_routing(cfg, np.stack([rng.permutation(1024)[:48] for _ in range(cfg.tokens)]), rng.random((cfg.tokens, 48)))
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+def test_no_local_expert(dtype):
+    # a rank that owns none of the experts: nothing is sorted, no tile exists, the output is all zeros
+    from tests.gpu_util import run_fused_moe
+    cfg = mi.MoeConfig("m", 50, 128, 128, 6, 2, dtype, "softmax")
+    inp = mi.make_inputs_np(cfg, 1)
+    mask = np.zeros(cfg.experts, dtype=np.int32)
+    for k in ("g", "d", "g_scale", "d_scale"):  # one expert's worth of storage, never read
+        if inp[k] is not None:
+            inp[k] = inp[k][:1]
+    got, buf = run_fused_moe(cfg, inp, mask=mask)
+    assert int(buf.total[0]) == 0
+    assert np.all(oracle.bf16_to_f32(got) == 0.0)
+
+
+def test_invalid_sizes_are_rejected():
+    import torch
+    import therock_amd as ta
+    t = ta.fused_moe_traits()
+    z = lambda *sh, dt=torch.bfloat16: torch.zeros(sh, dtype=dt, device="cuda")
+
+    def call(T, E, K, H, I, traits=t):
+        buf = ta.MoeBuffers(ta.fused_moe_traits(), T, E, K, 128, 128, "cuda")
+        buf.out = z(T, H)
+        args = ta.make_args(traits, buf, z(T, H), z(E, 2 * I, H), z(E, H, I), z(T, K, dt=torch.int32), z(T, K, dt=torch.float32))
+        return ta.fused_moegemm(traits, args)
+
+    assert call(4, 4, 2, 100, 128) == -1.0      # hidden not a multiple of 32
+    assert call(4, 4, 2, 128, 96 + 16) == -1.0  # intermediate not a multiple of 32
+    with pytest.raises(RuntimeError, match="bad sizes"):
+        call(4, 2000, 2, 128, 128)               # more experts than the path takes
+    t8 = ta.fused_moe_traits(prec_i="fp8", prec_w="fp8")
+    buf = ta.MoeBuffers(t8, 4, 4, 2, 128, 96, "cuda")
+    u8 = lambda *sh: torch.zeros(sh, dtype=torch.uint8, device="cuda")
+    f32 = lambda *sh: torch.ones(sh, dtype=torch.float32, device="cuda")
+    args = ta.make_args(t8, buf, u8(4, 128), u8(4, 192, 128), u8(4, 128, 96), z(4, 2, dt=torch.int32), f32(4, 2),
+                        a_scale=f32(4), g_scale=f32(4, 192), d_scale=f32(4, 128))
+    assert ta.fused_moegemm(t8, args) == -1.0    # fp8 keeps one scale per 32 Y columns in groups of four: inter % 128
+
+
 def test_no_tokens():
     import torch
     import therock_amd as ta
