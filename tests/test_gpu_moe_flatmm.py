@@ -107,6 +107,8 @@ def test_unsupported_and_errors():
     assert ta.moe_flatmm(3, z(4, 64), z(2, 128, 64), z(8, 64), ids, eid, tot, 4, 2, 32) == -1.0
     with pytest.raises(RuntimeError):
         ta.moe_flatmm(ta.GEMM2, z(8, 64), z(2, 64, 64), z(4, 64), ids, eid, tot, 4, 2, 32)  # no sorted weights
+    # an empty batch is a no-op, whatever storage its tensors have
+    assert ta.moe_flatmm(ta.GEMM1_GATE_UP, z(0, 64), z(2, 128, 64), z(0, 64), ids, eid, tot, 0, 2, 32) == 0.0
 
 
 @pytest.mark.parametrize("T,E,K,H,I,unit", [(40, 6, 3, 64, 96, 32), (130, 8, 2, 256, 128, 16)])

@@ -763,6 +763,8 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
     const bool go = kind == MI355_MOE_GEMM1_GATE_ONLY;
     const bool w8 = a.prec_b == MI355_MOE_INT8;
     const bool f8 = a.prec_b == MI355_MOE_FP8;
+    if(a.NumTokens == 0)
+        return MI355_MOE_OK; // an empty batch: nothing to compute, and its tensors may have no storage
     if(!a.p_sorted_token_ids || !a.p_sorted_expert_ids || !a.p_max_token_id || !a.a_ptr || !a.b_ptr || !a.c_ptr ||
        (!g1 && !a.p_sorted_expert_weights))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: null pointer");
