@@ -16,17 +16,21 @@
 //     write into.  Loads of one wave return in order, so the two streams are issued by different
 //     waves (0..3 weights, 4..7 tokens): mixed in one wave, the L2-hit token loads would queue
 //     behind the HBM-miss weight loads.
-//   * What bounds the kernel is the rate at which a compute unit's LDS can be filled: with both
-//     streams running it is about 19 bytes per clock (each stream alone is much faster), and a step
-//     of this tile needs 36.9 KB for 1400 clocks of MFMA work.
+//   * What bounds the kernel is the compute unit's vector memory path: L2 hits queued behind HBM misses do
+//     not overtake them, so the token stream costs its stand-alone time on top of the weight stream (about
+//     19 bytes per clock together; a step of this tile needs up to 36.9 KB for 1400 clocks of MFMA work).
 //   * LDS rows are swizzled: 64-byte token rows keep chunk c of row r at c ^ ((r >> 2) & 3), 128-byte
 //     weight rows at c ^ ((r >> 1) & 7); both the linear DMA writes and the ds_read_b128 operand
-//     fetches are then conflict-free on the 64-bank LDS.  Token rows that do not exist (padding ids,
-//     rows past the tile) fetch some real row instead - their MFMA columns are never stored - so
-//     the number of DMA instructions per wave and step, and with it every wait count, is a
-//     compile-time constant.
-//   * The K loop is specialised on the number of token blocks a wave owns, so the MFMA region is
-//     straight-line code.
+//     fetches are then conflict-free on the 64-bank LDS.  Token rows past the tile's last row inside a
+//     fetched 64-row group (and padding ids) fetch some real row instead - their MFMA columns are never
+//     stored; whole groups the tile does not have are not fetched.
+//   * The K loop is specialised on the number of token blocks a wave owns, on the number of 64-row token
+//     groups the tile has and on whether the weight DMA is non-temporal, so that the MFMA region is
+//     straight-line code and every wait count a compile-time constant: scalar branches in the issue path
+//     cost 5 % of the kernel's time when tried.
+//   * The int8 path runs here too: i8 MFMAs for the gate+up GEMM; for the down GEMM bf16 tokens against
+//     int8 weights that are converted after the LDS read, one 128-byte weight line lasting four K steps.
+//   * Work items go to the XCDs in chunks of 32 (see lookup_tile).
 #include "moe_gemm_device.hpp"
 
 #include <algorithm>
