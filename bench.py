@@ -204,16 +204,25 @@ def run_neighbours(cfg, inp, buf, steps):
                               "what": f"{ne} experts of d [{H}, {I}] to ck_tile's pre-shuffled layout"}
     if cfg.dtype in ("bf16", "fp8"):
         y = torch.empty((T * K, I), dtype=torch.bfloat16, device="cuda")
+        # the caller owns the workspace: allocated once, outside the timed calls
+        ws0 = torch.empty((ta.moe_flatmm_get_workspace_size(ta.GEMM1_GATE_UP, inp["a"], inp["g"], y, buf.sorted_ids,
+                                                            buf.sorted_eid, buf.total, T, K, cfg.unit),),
+                          dtype=torch.uint8, device="cuda")
         ms = timed(lambda: ta.moe_flatmm(ta.GEMM1_GATE_UP, inp["a"], inp["g"], y, buf.sorted_ids, buf.sorted_eid, buf.total,
-                                         T, K, cfg.unit, scale_m=inp["a_scale"], scale_n=inp["g_scale"]), max(2, steps // 4))
+                                         T, K, cfg.unit, scale_m=inp["a_scale"], scale_n=inp["g_scale"], workspace=ws0),
+                   max(2, steps // 4))
         out["flatmm_gate_up"] = {"ms": ms, "tflops": 4.0 * T * K * H * I / ms / 1e9, "what": "stand-alone gate+up GEMM, bf16 C"}
         if cfg.dtype == "fp8":
             yq, ys = ta.rowwise_quant(y, "fp8")
         else:
             yq, ys = y, None
         c = torch.zeros((T, H), dtype=torch.bfloat16, device="cuda")
+        del ws0
+        ws1 = torch.empty((ta.moe_flatmm_get_workspace_size(ta.GEMM2, yq, inp["d"], c, buf.sorted_ids, buf.sorted_eid,
+                                                            buf.total, T, K, cfg.unit),), dtype=torch.uint8, device="cuda")
         ms = timed(lambda: ta.moe_flatmm(ta.GEMM2, yq, inp["d"], c, buf.sorted_ids, buf.sorted_eid, buf.total, T, K, cfg.unit,
-                                         sorted_weights=buf.sorted_w, scale_m=ys, scale_n=inp["d_scale"]), max(2, steps // 4))
+                                         sorted_weights=buf.sorted_w, scale_m=ys, scale_n=inp["d_scale"], workspace=ws1),
+                   max(2, steps // 4))
         out["flatmm_down"] = {"ms": ms, "tflops": 2.0 * T * K * H * I / ms / 1e9,
                               "what": "stand-alone down GEMM + combine, added to bf16 C"}
     return out

@@ -19,6 +19,7 @@
 #include <mutex>
 #include <stdexcept>
 #include <string>
+#include <utility>
 
 #include "mi355_moe.h"
 
@@ -107,31 +108,37 @@ inline float run_timed(const stream_config& s, F&& launch)
     return ms / (s.nrepeat_ > 0 ? s.nrepeat_ : 1);
 }
 
-// grow-only per-device scratch for callers that pass no workspace (CK's fused_moe needs none)
-inline void* cached_workspace(size_t bytes)
+// Workspace for callers that pass none (CK's fused_moe needs none, so CK-style call sites have none to pass).
+// One block per (device, stream): calls on different streams never share intermediates.  A block that was
+// handed out is never freed or moved - work already enqueued, or a captured graph, may still refer to it - so
+// growth allocates a new block and keeps the old one until the process ends.  Growth needs hipMalloc, which a
+// capturing stream does not allow: such callers pass their own workspace (or call once before capturing).
+// Calls that overlap on ONE stream's block from several host threads are the caller's to serialise.
+inline mi355_moe_workspace cached_workspace(size_t bytes, hipStream_t stream)
 {
-    struct Slot
+    struct Block
     {
         void* ptr    = nullptr;
         size_t bytes = 0;
     };
     static std::mutex mu;
-    static std::map<int, Slot> slots;
+    static std::map<std::pair<int, hipStream_t>, Block> blocks;
     int dev = 0;
     hip_check(hipGetDevice(&dev), "hipGetDevice");
     std::lock_guard<std::mutex> lock(mu);
-    Slot& s = slots[dev];
-    if(s.bytes < bytes)
+    Block& b = blocks[std::make_pair(dev, stream)];
+    if(b.bytes < bytes)
     {
-        if(s.ptr != nullptr)
-        {
-            hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize");
-            hip_check(hipFree(s.ptr), "hipFree");
-        }
-        hip_check(hipMalloc(&s.ptr, bytes), "hipMalloc(workspace)");
-        s.bytes = bytes;
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if(hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
+            throw std::runtime_error("mi355: the stream is capturing and the cached workspace would have to grow; "
+                                     "pass a workspace of fused_moe_get_workspace_size() bytes instead");
+        void* p = nullptr;
+        hip_check(hipMalloc(&p, bytes), "hipMalloc(workspace)");
+        b.ptr   = p; // the previous block, if any, stays allocated
+        b.bytes = bytes;
     }
-    return s.ptr;
+    return mi355_moe_workspace{b.ptr, b.bytes};
 }
 
 } // namespace detail
@@ -192,20 +199,21 @@ struct moe_flatmm_args : public mi355_moe_flatmm_args
 {
 };
 
-// ws_ptr may be left null: a cached per-device workspace is used.  Returns -1 when no kernel matches.
-inline float moe_flatmm(MoeFlatmmKind kind, moe_flatmm_args a, stream_config s = {})
+// ws: caller-owned workspace of mi355_moe_flatmm_workspace_size() bytes; when its ptr is null a cached block of
+// this (device, stream) is used.  Returns -1 when no kernel matches.
+inline float moe_flatmm(MoeFlatmmKind kind, moe_flatmm_args a, stream_config s = {}, mi355_moe_workspace ws = {})
 {
     const int k = static_cast<int>(kind);
-    if(a.ws_ptr == nullptr)
+    if(ws.ptr == nullptr)
     {
-        a.ws_bytes = mi355_moe_flatmm_workspace_size(k, &a);
-        if(a.ws_bytes == 0)
+        const size_t bytes = mi355_moe_flatmm_workspace_size(k, &a);
+        if(bytes == 0)
             return -1.f;
-        a.ws_ptr = detail::cached_workspace(a.ws_bytes);
+        ws = detail::cached_workspace(bytes, s.stream_id_);
     }
     bool unsupported = false;
     const float ms   = detail::run_timed(s, [&] {
-        const int rc = mi355_moe_flatmm(k, &a, s.stream_id_);
+        const int rc = mi355_moe_flatmm(k, &a, &ws, s.stream_id_);
         if(rc == MI355_MOE_E_UNSUPPORTED)
         {
             unsupported = true;
@@ -267,11 +275,12 @@ struct fused_moe_traits
     }
 };
 
-// fused_moe_args of CK's example.  ws_ptr may be left null: a cached per-device workspace is used.
+// fused_moe_args of CK's example (ws_ptr is the example's sort workspace and may stay null)
 struct fused_moe_args : public mi355_fused_moe_args
 {
 };
 
+// ck_tile::FusedMoeGemmHostArgs (ops/fused_moe/kernel/fused_moegemm_kernel.hpp:97-120), same layout
 struct fused_moegemm_args : public mi355_fused_moegemm_args
 {
 };
@@ -283,37 +292,44 @@ inline size_t fused_moe_get_workspace_size(const fused_moe_traits& t, int tokens
     return mi355_fused_moe_workspace_size(&p, tokens, num_experts, topk, hidden_size, intermediate_size);
 }
 
-inline float fused_moe(fused_moe_traits t, fused_moe_args a, const stream_config& s = {})
+namespace detail {
+inline bool pick_workspace(const mi355_fused_moe_traits& p, int tokens, int experts, int topk, int hidden, int inter,
+                           hipStream_t stream, mi355_moe_workspace& ws)
+{
+    if(ws.ptr != nullptr)
+        return true;
+    const size_t bytes = mi355_fused_moe_workspace_size(&p, tokens, experts, topk, hidden, inter);
+    if(bytes == 0)
+        return false; // sizes the library cannot index: let the entry point describe the error
+    ws = cached_workspace(bytes, stream);
+    return true;
+}
+} // namespace detail
+
+// CK's signature plus an optional caller-owned workspace (fused_moe_get_workspace_size() bytes, 256-byte aligned);
+// without one a cached block of this (device, stream) is used
+inline float fused_moe(fused_moe_traits t, fused_moe_args a, const stream_config& s = {}, mi355_moe_workspace ws = {})
 {
     const mi355_fused_moe_traits p = t.pod();
     if(!mi355_fused_moe_supported(&p))
         return -1.f;
-    if(a.ws_ptr == nullptr)
-    {
-        a.ws_bytes = mi355_fused_moe_workspace_size(&p, a.num_tokens, a.num_experts, a.topk, a.hidden_size,
-                                                    a.intermediate_size);
-        a.ws_ptr   = detail::cached_workspace(a.ws_bytes);
-    }
+    detail::pick_workspace(p, a.num_tokens, a.num_experts, a.topk, a.hidden_size, a.intermediate_size, s.stream_id_, ws);
     return detail::run_timed(s, [&] {
-        const int rc = mi355_fused_moe(&p, &a, s.stream_id_);
+        const int rc = mi355_fused_moe(&p, &a, &ws, s.stream_id_);
         detail::throw_on_error(rc, "fused_moe");
         return rc;
     });
 }
 
-inline float fused_moegemm(fused_moe_traits t, fused_moegemm_args a, const stream_config& s = {})
+inline float fused_moegemm(fused_moe_traits t, fused_moegemm_args a, const stream_config& s = {},
+                           mi355_moe_workspace ws = {})
 {
     const mi355_fused_moe_traits p = t.pod();
     if(!mi355_fused_moe_supported(&p))
         return -1.f;
-    if(a.ws_ptr == nullptr)
-    {
-        a.ws_bytes = mi355_fused_moe_workspace_size(&p, a.num_tokens, a.num_experts, a.topk, a.hidden_size,
-                                                    a.intermediate_size);
-        a.ws_ptr   = detail::cached_workspace(a.ws_bytes);
-    }
+    detail::pick_workspace(p, a.num_tokens, a.num_experts, a.topk, a.hidden_size, a.intermediate_size, s.stream_id_, ws);
     return detail::run_timed(s, [&] {
-        const int rc = mi355_fused_moegemm(&p, &a, s.stream_id_);
+        const int rc = mi355_fused_moegemm(&p, &a, &ws, s.stream_id_);
         detail::throw_on_error(rc, "fused_moegemm");
         return rc;
     });

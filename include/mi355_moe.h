@@ -3,14 +3,19 @@
  *
  * Every entry point takes plain pointers and sizes; all data pointers are DEVICE pointers owned by
  * the caller, launches are asynchronous on the given HIP stream (passed as void*, NULL = default
- * stream) and nothing is allocated behind the caller's back.  The structs mirror, field for
- * field, the host argument blocks of Composable Kernel's ck_tile fused-MoE (ck_tile 1.2.0, paths
- * relative to /opt/rocm/include/ck_tile):
+ * stream) and nothing is allocated behind the caller's back.  The structs mirror the host argument
+ * blocks of Composable Kernel's ck_tile fused-MoE (ck_tile 1.2.0, paths relative to
+ * /opt/rocm/include/ck_tile):
  *
- *   mi355_moe_sorting_args   <- MoeSortingHostArgs    ops/fused_moe/kernel/moe_sorting_kernel.hpp:188-222
- *   mi355_fused_moegemm_args <- FusedMoeGemmHostArgs  ops/fused_moe/kernel/fused_moegemm_kernel.hpp:97-120
+ *   mi355_moe_sorting_args   == MoeSortingHostArgs    ops/fused_moe/kernel/moe_sorting_kernel.hpp:188-222
+ *   mi355_fused_moegemm_args == FusedMoeGemmHostArgs  ops/fused_moe/kernel/fused_moegemm_kernel.hpp:97-120
  *   mi355_fused_moe_args     <- fused_moe_args  of CK's example/ck_tile/15_fused_moe/fused_moe.hpp
  *   mi355_fused_moe_traits   <- fused_moe_traits of the same example, with enums for its strings
+ *
+ * The first two have the same fields at the same offsets as the ck_tile structs (a pointer to one can
+ * be cast to the other; tests/cpp/abi_layout_check.cpp asserts it against the ck_tile headers).  What
+ * this library needs beyond them - device memory for the intermediate activations - travels beside the
+ * argument block as a mi355_moe_workspace.
  *
  * Return value of every int function: 0 on success, negative on failure (MI355_MOE_E_*);
  * mi355_moe_last_error() returns a human-readable description for the calling thread.
@@ -25,7 +30,7 @@
 extern "C" {
 #endif
 
-#define MI355_MOE_VERSION 100
+#define MI355_MOE_VERSION 200
 
 enum mi355_moe_status
 {
@@ -46,6 +51,17 @@ enum mi355_moe_dtype
     MI355_MOE_INT32 = 4,
     MI355_MOE_FP16 = 5
 };
+
+/* Device memory the GEMM entry points use for their intermediates (tile list, the activations between
+ * the two GEMMs, per-slot partial outputs).  ck_tile's fused kernel needs none, so it is not part of
+ * the argument blocks: it is passed beside them.  ptr: 256-byte aligned device memory of at least the
+ * size the matching *_workspace_size() function returns; it need not be cleared, and holds nothing
+ * between calls.  Calls that share a workspace must not overlap. */
+typedef struct mi355_moe_workspace
+{
+    void* ptr;
+    size_t bytes;
+} mi355_moe_workspace;
 
 /* ------------------------------------------------------------------------------ moe_sorting
  * Replaces ck_tile::MoeSortingKernel / MoeSortingMultiPhaseKernel_* behind MoeSortingHostArgs
@@ -130,9 +146,9 @@ typedef struct mi355_fused_moe_traits
     int32_t local_expert_masking; /* 1 = apply local_expert_mask_ptr in the sort */
 } mi355_fused_moe_traits;
 
-/* FusedMoeGemmHostArgs (fused_moegemm_kernel.hpp:97-120) plus the workspace this build needs for
- * the intermediate activations.  Weights are plain row-major, K contiguous (what ck_tile's host
- * reference takes; FusedMoeGemmWeightPermuteEnum::no_permute, fused_moegemm_traits.hpp:10-17). */
+/* FusedMoeGemmHostArgs (fused_moegemm_kernel.hpp:97-120), field for field.  Weights are plain row-major,
+ * K contiguous (what ck_tile's host reference takes; FusedMoeGemmWeightPermuteEnum::no_permute,
+ * fused_moegemm_traits.hpp:10-17); mi355_moe_permute_weights converts pre-shuffled checkpoints. */
 typedef struct mi355_fused_moegemm_args
 {
     const void* a_ptr;              /* [tokens, stride_token] activations */
@@ -147,8 +163,6 @@ typedef struct mi355_fused_moegemm_args
     const void* sorted_weight_ptr;
     const void* sorted_expert_ids_ptr;
     const void* num_sorted_tiles_ptr;  /* [>=1] int32: [0] holds tokens_post_pad (:243-246) */
-    void* ws_ptr;                   /* mi355_fused_moe_workspace_size() bytes */
-    size_t ws_bytes;
     int32_t hidden_size;
     int32_t intermediate_size;
     int32_t num_tokens;
@@ -157,7 +171,8 @@ typedef struct mi355_fused_moegemm_args
     int32_t stride_token;           /* elements between rows of a and of o (>= hidden_size) */
 } mi355_fused_moegemm_args;
 
-/* fused_moe_args of CK's example: the GEMM arguments plus routing inputs and sort outputs */
+/* fused_moe_args of CK's example (example/ck_tile/15_fused_moe/fused_moe.hpp): the GEMM arguments plus
+ * routing inputs, sort outputs and the sort's workspace, in the example's order */
 typedef struct mi355_fused_moe_args
 {
     const void* a_ptr;
@@ -169,8 +184,8 @@ typedef struct mi355_fused_moe_args
     const void* y_smooth_scale_ptr;
     const void* local_expert_mask_ptr; /* [experts] int32, used when traits.local_expert_masking */
     void* o_ptr;
-    void* ws_ptr;                      /* mi355_fused_moe_workspace_size() bytes */
-    size_t ws_bytes;
+    void* ws_ptr;                      /* the example's sort workspace (mi355_moe_sorting_workspace_size() bytes);
+                                          may be NULL: the mi355_moe_workspace then holds it too */
     const void* topk_ids_ptr;          /* [tokens, topk] int32 */
     const void* topk_weight_ptr;       /* [tokens, topk] fp32 */
     void* sorted_token_ids_ptr;        /* outputs of the sort, sized as for mi355_moe_sorting */
@@ -189,7 +204,8 @@ typedef struct mi355_fused_moe_args
 /* 1 if a kernel exists for these traits, else 0 (ck_tile's dispatcher returns -1 from fused_moe) */
 int mi355_fused_moe_supported(const mi355_fused_moe_traits* traits);
 
-/* bytes of ws_ptr for mi355_fused_moe / mi355_fused_moegemm (includes the sort's own workspace) */
+/* bytes of the mi355_moe_workspace for mi355_fused_moe / mi355_fused_moegemm (includes the sort's own
+ * workspace); 0 for unsupported traits or sizes out of range */
 size_t mi355_fused_moe_workspace_size(const mi355_fused_moe_traits* traits, int32_t tokens,
                                       int32_t num_experts, int32_t topk, int32_t hidden_size,
                                       int32_t intermediate_size);
@@ -203,15 +219,17 @@ int32_t mi355_fused_moe_tile_rows(const mi355_fused_moe_traits* traits, int32_t 
 /* replaces fused_moegemm(traits, args, stream): FusedMoeGemmKernel (fused_moegemm_kernel.hpp:238-259).
  * Gate+up GEMM with SiLU*up, down GEMM, top-k weighted combine into o. */
 int mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_moegemm_args* args,
-                        void* stream);
+                        const mi355_moe_workspace* ws, void* stream);
 
 /* replaces fused_moe(traits, args, stream) of CK's example: mi355_moe_sorting then
  * mi355_fused_moegemm on one stream */
-int mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* args, void* stream);
+int mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* args,
+                    const mi355_moe_workspace* ws, void* stream);
 
 /* per-row dynamic quantisation of bf16 activations, the step in front of the quantised path:
  * scale[m] = amax(row)/qmax, q = convert(saturate(x/scale)) (host/reference/reference_rowwise_quantization2d.hpp:12-31);
- * as in ck_tile the int8 conversion truncates toward zero (core/numeric/int8.hpp:101), e4m3 rounds to nearest even.
+ * as in ck_tile the int8 conversion truncates toward zero (core/numeric/int8.hpp:101), e4m3 rounds to nearest even;
+ * a row of zeros gets scale 1 and codes 0.
  * x [rows, stride_x] bf16 -> q [rows, cols] (FP8 or INT8), scale [rows] fp32. */
 int mi355_moe_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype,
                             void* q, void* scale, void* stream);
@@ -220,7 +238,8 @@ int mi355_moe_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t s
  * MoeSmoothquantHostArgs (ops/smoothquant/kernel/moe_smoothquant_kernel.hpp:12-27): for slot k of token t
  * routed to expert e = topk_ids[t, k]: y = x[t, :] * smscale[e, :] (fp32), yscale[k * tokens + t] =
  * amax|y| / qmax, qy[k * tokens + t, :] = convert(saturate(y / yscale))
- * (ops/smoothquant/pipeline/smoothquant_pipeline_one_pass.hpp:73-118). */
+ * (ops/smoothquant/pipeline/smoothquant_pipeline_one_pass.hpp:73-118).  A row of zeros gets yscale 0 and codes 0
+ * (ck_tile converts 0 / 0 there, which is undefined). */
 typedef struct mi355_moe_smoothquant_args
 {
     const void* p_x;        /* [tokens, x_stride] bf16 */
@@ -251,17 +270,29 @@ int mi355_moe_permute_weights(const void* src, void* dst, int32_t experts, int32
  * The two GEMMs as separate launches, for callers that keep sort / gemm1 / gemm2 apart.  Replaces
  * ck_tile::MoeFlatmmKernel behind MoeFlatmmHostArgs (ops/flatmm/kernel/moe_flatmm_kernel.hpp:17-127, kinds
  * :130-135); semantics as in host/reference/reference_moe_gemm.hpp:18-241:
- *   gate+up: C[token * TopK + slot, n] = silu(A[token] . B[e, n]) * (A[token] . B[e, N/2 + n]),  n < N/2
- *   down   : C[token, n] += sum over the token's slots of w * (A[token * TopK + slot] . B[e, n])
- * with the per-row scale scale_m and the per-channel scale scale_n folded in.  Unlike ck_tile's atomic
- * bf16 epilogue the down GEMM sums a token's slots in fp32, in slot order, and rounds once. */
+ *   gate+up: C[token * TopK + slot, n] = act(A[token] . B[e, n] + bias[e, n], A[token] . B[e, N/2 + n] + bias[e, N/2 + n]),  n < N/2
+ *   gate only: C[token * TopK + slot, n] = act(A[token] . B[e, n] + bias[e, n])
+ *   down   : C[token, n] += sum over the token's slots of w * (A[token * TopK + slot] . B[e, n] + bias[e, n])
+ * with the per-row scale scale_m and the per-channel scale scale_n folded into the dot products.  act is the
+ * FusedActivation of the ck_tile kernel (moe_flatmm_kernel.hpp:139-183): MoeSilu, silu(gate) * linear, or
+ * moe::Swiglu{alpha, limit}, gate' * sigmoid(alpha * gate') * (linear' + 1) with gate' = min(gate, limit) and
+ * linear' = clamp(linear, -limit, limit) (gate only: linear = 1 for MoeSilu).  Unlike ck_tile's atomic bf16
+ * epilogue the down GEMM sums a token's slots in fp32, in slot order, and rounds once. */
 enum mi355_moe_flatmm_kind
 {
-    MI355_MOE_GEMM1_GATE_ONLY = 0, /* C = silu(A x B^T), B [experts, N, K] */
+    MI355_MOE_GEMM1_GATE_ONLY = 0, /* C = act(A x B^T), B [experts, N, K] */
     MI355_MOE_GEMM1_GATE_UP   = 1,
     MI355_MOE_GEMM2           = 2
 };
 
+enum mi355_moe_flatmm_activation
+{
+    MI355_MOE_ACT_SILU   = 0, /* ck_tile::moe::MoeSilu, the default FusedActivation */
+    MI355_MOE_ACT_SWIGLU = 1  /* ck_tile::moe::Swiglu{swiglu_alpha, swiglu_limit} */
+};
+
+/* the arguments of MoeFlatmmHostArgs' constructor (moe_flatmm_kernel.hpp:79-127) in its order, then what the
+ * ck_tile kernel takes as template arguments (operand types, activation) */
 typedef struct mi355_moe_flatmm_args
 {
     const void* p_sorted_token_ids;      /* as written by mi355_moe_sorting: token | slot << 24 */
@@ -271,11 +302,6 @@ typedef struct mi355_moe_flatmm_args
     const void* a_ptr;    /* gate+up: [NumTokens, stride_A]; down: [NumTokens * TopK, stride_A] */
     const void* b_ptr;    /* [NumExperts, N, K], K contiguous (stride_B = K) */
     void* c_ptr;          /* bf16; gate+up: [NumTokens * TopK, stride_C] (N/2 columns); down: [NumTokens, stride_C] */
-    const void* scale_m;  /* fp32 per row of A, or NULL (ScaleM) */
-    const void* scale_n;  /* fp32 [NumExperts, N], or NULL (ScaleN) */
-    const void* exp_bias; /* must be NULL */
-    void* ws_ptr;         /* mi355_moe_flatmm_workspace_size() bytes, 256-byte aligned */
-    size_t ws_bytes;
     int32_t NumTokens;
     int32_t NumExperts;
     int32_t TopK;
@@ -286,13 +312,22 @@ typedef struct mi355_moe_flatmm_args
     int32_t stride_A;
     int32_t stride_B;
     int32_t stride_C;
+    int32_t n_padded_zeros; /* the last n_padded_zeros rows of every expert's B are padding: read as zero */
+    int32_t k_padded_zeros; /* the last k_padded_zeros columns of A and B are padding: read as zero */
+    const void* scale_m;  /* fp32 per row of A, or NULL (ScaleM) */
+    const void* scale_n;  /* fp32 [NumExperts, N], or NULL (ScaleN) */
+    const void* exp_bias; /* fp32 [NumExperts, N] added to the scaled dot products, or NULL (ExpertBias) */
     int32_t prec_a;       /* mi355_moe_dtype of A: BF16, FP8 (with FP8 weights), or INT8 for the gate+up GEMM with int8 weights */
     int32_t prec_b;       /* mi355_moe_dtype of B: BF16 | FP8 | INT8 */
     int32_t block_m;      /* unit_size the sort was run with */
+    int32_t activation;   /* mi355_moe_flatmm_activation (gate GEMMs) */
+    float swiglu_alpha;   /* 1.702 in ck_tile's default */
+    float swiglu_limit;   /* 7.0 in ck_tile's default */
 } mi355_moe_flatmm_args;
 
+/* bytes of the mi355_moe_workspace for this call; 0 when the arguments have no kernel */
 size_t mi355_moe_flatmm_workspace_size(int32_t kind, const mi355_moe_flatmm_args* args);
-int mi355_moe_flatmm(int32_t kind, const mi355_moe_flatmm_args* args, void* stream);
+int mi355_moe_flatmm(int32_t kind, const mi355_moe_flatmm_args* args, const mi355_moe_workspace* ws, void* stream);
 
 /* ------------------------------------------------------------------------------ kernel timing
  * Counterpart of ck_tile::stream_config::time_kernel_ (host/stream_config.hpp:29-39,

@@ -209,7 +209,8 @@ ORACLE_API int moe_oracle_rowwise_quant(const float* x, int64_t M, int64_t N, in
 /* MoE smooth-quant (ops/smoothquant/kernel/moe_smoothquant_kernel.hpp:12-27, 152-175 and
  * pipeline/smoothquant_pipeline_one_pass.hpp:73-118): for slot k of token t routed to expert e,
  * y = x[t,:] * smscale[e,:] in fp32, yscale[k*tokens + t] = amax|y| / qmax, qy[k*tokens + t, :] =
- * convert(saturate(y / yscale)).  Outputs are [topk, tokens, hidden] and [topk, tokens]. */
+ * convert(saturate(y / yscale)).  Outputs are [topk, tokens, hidden] and [topk, tokens].
+ * A row of zeros (ck_tile converts 0 / 0 there, which is undefined behaviour) gets scale 0 and codes 0. */
 ORACLE_API int moe_oracle_smoothquant(const float* x, const float* smscale, const int32_t* topk_ids, int32_t tokens,
                                       int32_t hidden, int32_t experts, int32_t topk, int dt, void* qy, float* yscale)
 {
@@ -232,8 +233,9 @@ ORACLE_API int moe_oracle_smoothquant(const float* x, const float* smscale, cons
             }
             const float ys           = amax / qmax;
             yscale[k * tokens + t]   = ys;
+            const float div          = amax > 0.f ? ys : 1.0f;
             for(int64_t h = 0; h < hidden; h++)
-                quant_store(qy, (k * tokens + t) * hidden + h, (xr[h] * sr[h]) / ys, dt, 0);
+                quant_store(qy, (k * tokens + t) * hidden + h, (xr[h] * sr[h]) / div, dt, 0);
         }
     return 0;
 }

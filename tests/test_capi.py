@@ -32,7 +32,8 @@ def test_struct_layouts_match_the_header(tmp_path):
     structs = {"mi355_moe_sorting_args": _lib.SortingArgs, "mi355_fused_moe_traits": _lib.FusedMoeTraits,
                "mi355_fused_moegemm_args": _lib.FusedMoeGemmArgs, "mi355_fused_moe_args": _lib.FusedMoeArgs,
                "mi355_topk_softmax_args": _lib.TopkSoftmaxArgs, "mi355_topk_softmax_traits": _lib.TopkSoftmaxTraits,
-               "mi355_moe_flatmm_args": _lib.FlatmmArgs, "mi355_moe_smoothquant_args": _lib.SmoothquantArgs}
+               "mi355_moe_flatmm_args": _lib.FlatmmArgs, "mi355_moe_smoothquant_args": _lib.SmoothquantArgs,
+               "mi355_moe_workspace": _lib.Workspace}
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void){"]
     for cname, ct in structs.items():
         lines.append(f'printf("{cname} %zu\\n", sizeof({cname}));')
@@ -50,9 +51,54 @@ def test_struct_layouts_match_the_header(tmp_path):
             assert int(out[f"{cname}.{fname}"]) == getattr(ct, fname).offset, f"{cname}.{fname}"
 
 
+def test_argument_blocks_have_the_layout_of_the_ck_tile_structs(tmp_path):
+    """mi355_fused_moegemm_args / mi355_moe_sorting_args against ck_tile's FusedMoeGemmHostArgs / MoeSortingHostArgs:
+    one translation unit includes both headers and static_asserts size and every field offset."""
+    import shutil
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc is not installed")
+    src = os.path.join(ROOT, "tests", "cpp", "abi_layout_check.cpp")
+    cmd = [hipcc, "-std=c++17", "--cuda-host-only", "-I/opt/rocm/include", "-Wno-everything"]
+    subprocess.run(cmd + ["-fsyntax-only", src], check=True)
+    pre = subprocess.run(cmd + ["-E", src], check=True, capture_output=True, text=True).stdout
+    if "mi355_abi_layout_checked = 1" not in pre:
+        pytest.skip("the ck_tile headers are not installed: nothing to compare with")
+    # the check is live: a struct with an extra field in front of hidden_size must fail to compile
+    bad = tmp_path / "bad.cpp"
+    bad.write_text(open(src).read().replace('#include "../../include/mi355_moe.h"',
+                                            f'#define hidden_size padding_; int32_t hidden_size\n#include "{HEADER}"\n#undef hidden_size'))
+    r = subprocess.run(cmd + ["-fsyntax-only", str(bad)], capture_output=True, text=True)
+    assert r.returncode != 0 and "static assertion failed" in r.stderr
+
+
+def test_sizes_out_of_range_are_rejected_on_the_host():
+    """No entry point divides by or indexes with a size before checking it (0 experts used to kill the process)."""
+    lib = _lib.load()
+    t = _lib.FusedMoeTraits(0, 0, 0, 3, 3, 3, 3, 32, 1, 0, 0, 0)
+    for shape in ((128, 0, 2, 1024, 1024), (128, 8, 0, 1024, 1024), (-1, 8, 2, 1024, 1024), (128, 8, 2, 0, 1024),
+                  (128, 8, 2, 1024, -4), (128, 2000, 2, 1024, 1024), (128, 8, 300, 1024, 1024)):
+        assert lib.mi355_fused_moe_workspace_size(C.byref(t), *shape) == 0, shape
+        assert lib.mi355_fused_moe_tile_rows(C.byref(t), *shape) == 0, shape
+        T, E, K, H, I = shape
+        f = _lib.FusedMoeArgs(block_m=32, hidden_size=H, intermediate_size=I, num_tokens=T, num_experts=E, topk=K,
+                              stride_token=max(H, 0))
+        ws = _lib.Workspace(None, 0)
+        assert lib.mi355_fused_moe(C.byref(t), C.byref(f), C.byref(ws), None) == _lib.E_INVALID, shape
+        assert b"bad sizes" in lib.mi355_moe_last_error()
+        g = _lib.FusedMoeGemmArgs(hidden_size=H, intermediate_size=I, num_tokens=T, num_experts=E, topk=K,
+                                  stride_token=max(H, 0))
+        assert lib.mi355_fused_moegemm(C.byref(t), C.byref(g), C.byref(ws), None) == _lib.E_INVALID, shape
+        assert lib.mi355_fused_moegemm(C.byref(t), C.byref(g), None, None) == _lib.E_INVALID, shape
+    # a valid shape without a workspace: the workspace error, before anything is launched
+    f = _lib.FusedMoeArgs(block_m=32, hidden_size=1024, intermediate_size=1024, num_tokens=128, num_experts=8, topk=2,
+                          stride_token=1024)
+    assert lib.mi355_fused_moe(C.byref(t), C.byref(f), None, None) == _lib.E_WORKSPACE
+
+
 def test_host_only_entry_points():
     lib = _lib.load()
-    assert lib.mi355_moe_version() == 100
+    assert lib.mi355_moe_version() == 200
     assert lib.mi355_moe_max_num_tokens_padded(128, 8, 2, 32) == 2 * 128 + 8 * 32 - 2
     assert lib.mi355_moe_sorting_workspace_size(64, 128, 8) == 0          # one workgroup, no workspace
     assert lib.mi355_moe_sorting_workspace_size(32768, 64, 6) >= 384 * 64 * 4
@@ -64,7 +110,7 @@ def test_host_only_entry_points():
     assert lib.mi355_fused_moe_supported(C.byref(bad)) == 0
     assert lib.mi355_fused_moe_workspace_size(C.byref(bad), 128, 8, 2, 1024, 1024) == 0
     assert lib.mi355_moe_sorting(None, None) == _lib.E_INVALID and b"null" in lib.mi355_moe_last_error()
-    assert lib.mi355_fused_moe(None, None, None) == _lib.E_INVALID
+    assert lib.mi355_fused_moe(None, None, None, None) == _lib.E_INVALID
     # traits of the reference's example API: both activations and both weight layouts have kernels
     for act, gate_only, ok in ((0, 0, 1), (1, 1, 1), (0, 1, 1), (2, 0, 0), (1, 2, 0)):
         t = _lib.FusedMoeTraits(0, 0, 0, 3, 3, 3, 3, 32, act, gate_only, 0, 0)

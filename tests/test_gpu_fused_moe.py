@@ -260,7 +260,7 @@ def test_traits_without_kernel_return_minus_one():
     ids = torch.zeros((4, 2), dtype=torch.int32, device="cuda")
     w = torch.zeros((4, 2), dtype=torch.float32, device="cuda")
     args = ta.make_args(t, buf, a, g, d, ids, w)
-    args.ws_ptr = None
+    args.workspace = None
     with pytest.raises(RuntimeError, match="workspace"):
         ta.fused_moe(t, args)
 

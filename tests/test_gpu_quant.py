@@ -64,6 +64,31 @@ def test_moe_smoothquant(tokens, hidden, experts, topk, kind):
     assert np.array_equal(_raw(qy), rq)
 
 
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+@pytest.mark.parametrize("hidden", [100, 4096])  # the scalar and the 16-byte kernel
+def test_rows_of_zeros_quantise_to_zero(kind, hidden):
+    """Padded batches hold rows of zeros: their codes are 0 (not the 0 / 0 of the plain formula), the scale is 0
+    from smooth-quant (amax / qmax) and 1 from the row-wise quantiser."""
+    import torch
+    import therock_amd as ta
+
+    rng = np.random.default_rng(hidden)
+    x = _bf16(rng.standard_normal((6, hidden)).astype(np.float32))
+    x[1] = 0
+    x[4] = 0
+    sm = torch.from_numpy((0.25 + rng.random((4, hidden)) * 2).astype(np.float32)).cuda()
+    ids = np.stack([rng.permutation(4)[:2] for _ in range(6)]).astype(np.int32)
+    qy, ys = ta.moe_smoothquant(x, sm, torch.from_numpy(ids).cuda(), kind)
+    q, s = ta.rowwise_quant(x, kind)
+    torch.cuda.synchronize()
+    dt = oracle.DT_I8 if kind == "int8" else oracle.DT_E4M3
+    rq, rs = oracle.smoothquant(x.float().cpu().numpy(), sm.cpu().numpy(), ids, dt)
+    assert np.array_equal(ys.cpu().numpy(), rs) and np.array_equal(_raw(qy), rq)
+    for r in (1, 4):
+        assert not _raw(qy)[:, r].any() and not ys.cpu().numpy()[:, r].any()
+        assert not _raw(q)[r].any() and float(s[r]) == 1.0
+
+
 @pytest.mark.parametrize("shape,dtype,nw,kw,kv", [((4, 256, 512), "bf16", 16, 4, 8), ((3, 64, 256), "int8", 16, 4, 16),
                                                    ((2, 64, 64), "bf16", 32, 2, 8), ((8, 4096, 1024), "fp8", 16, 4, 16)])
 def test_permute_weights(shape, dtype, nw, kw, kv):

@@ -141,6 +141,13 @@ def test_quantisers_match_ck_tile_reference():
             y = xb * sm[ids[:, k]]
             assert np.array_equal(ys[k], np.abs(y).max(axis=1) / np.float32(qmax))
             assert np.array_equal(qy[k], oracle.ck_rowwise_quant(y, ys[k], dt))
+        # a row of zeros: scale 0 and codes 0 (the convention where the reference's 0 / 0 is undefined)
+        xz = xb.copy()
+        xz[3] = 0
+        qz, sz = oracle.smoothquant(xz, sm, ids, dt)
+        assert not qz[:, 3].any() and not sz[:, 3].any()
+        keep = np.arange(T) != 3
+        assert np.array_equal(qz[:, keep], qy[:, keep]) and np.array_equal(sz[:, keep], ys[:, keep])
 
 
 @pytest.mark.skipif(oracle.ck_ref() is None, reason="oracle/_ref not built")

@@ -36,8 +36,8 @@ class FusedMoeGemmArgs(C.Structure):
         ("a_ptr", C.c_void_p), ("a_scale_ptr", C.c_void_p), ("g_ptr", C.c_void_p), ("d_ptr", C.c_void_p),
         ("g_scale_ptr", C.c_void_p), ("d_scale_ptr", C.c_void_p), ("y_smooth_scale_ptr", C.c_void_p),
         ("o_ptr", C.c_void_p), ("sorted_token_ids_ptr", C.c_void_p), ("sorted_weight_ptr", C.c_void_p),
-        ("sorted_expert_ids_ptr", C.c_void_p), ("num_sorted_tiles_ptr", C.c_void_p), ("ws_ptr", C.c_void_p),
-        ("ws_bytes", C.c_size_t), ("hidden_size", C.c_int32), ("intermediate_size", C.c_int32),
+        ("sorted_expert_ids_ptr", C.c_void_p), ("num_sorted_tiles_ptr", C.c_void_p),
+        ("hidden_size", C.c_int32), ("intermediate_size", C.c_int32),
         ("num_tokens", C.c_int32), ("num_experts", C.c_int32), ("topk", C.c_int32), ("stride_token", C.c_int32),
     ]
 
@@ -47,7 +47,7 @@ class FusedMoeArgs(C.Structure):
         ("a_ptr", C.c_void_p), ("a_scale_ptr", C.c_void_p), ("g_ptr", C.c_void_p), ("d_ptr", C.c_void_p),
         ("g_scale_ptr", C.c_void_p), ("d_scale_ptr", C.c_void_p), ("y_smooth_scale_ptr", C.c_void_p),
         ("local_expert_mask_ptr", C.c_void_p), ("o_ptr", C.c_void_p), ("ws_ptr", C.c_void_p),
-        ("ws_bytes", C.c_size_t), ("topk_ids_ptr", C.c_void_p), ("topk_weight_ptr", C.c_void_p),
+        ("topk_ids_ptr", C.c_void_p), ("topk_weight_ptr", C.c_void_p),
         ("sorted_token_ids_ptr", C.c_void_p), ("sorted_weight_ptr", C.c_void_p),
         ("sorted_expert_ids_ptr", C.c_void_p), ("num_sorted_tiles_ptr", C.c_void_p), ("block_m", C.c_int32),
         ("hidden_size", C.c_int32), ("intermediate_size", C.c_int32), ("num_tokens", C.c_int32),
@@ -73,12 +73,17 @@ class FlatmmArgs(C.Structure):
     _fields_ = [
         ("p_sorted_token_ids", C.c_void_p), ("p_sorted_expert_weights", C.c_void_p), ("p_sorted_expert_ids", C.c_void_p),
         ("p_max_token_id", C.c_void_p), ("a_ptr", C.c_void_p), ("b_ptr", C.c_void_p), ("c_ptr", C.c_void_p),
-        ("scale_m", C.c_void_p), ("scale_n", C.c_void_p), ("exp_bias", C.c_void_p), ("ws_ptr", C.c_void_p),
-        ("ws_bytes", C.c_size_t), ("NumTokens", C.c_int32), ("NumExperts", C.c_int32), ("TopK", C.c_int32),
-        ("k_batch", C.c_int32), ("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("stride_A", C.c_int32),
-        ("stride_B", C.c_int32), ("stride_C", C.c_int32), ("prec_a", C.c_int32), ("prec_b", C.c_int32),
-        ("block_m", C.c_int32),
+        ("NumTokens", C.c_int32), ("NumExperts", C.c_int32), ("TopK", C.c_int32), ("k_batch", C.c_int32),
+        ("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("stride_A", C.c_int32), ("stride_B", C.c_int32),
+        ("stride_C", C.c_int32), ("n_padded_zeros", C.c_int32), ("k_padded_zeros", C.c_int32),
+        ("scale_m", C.c_void_p), ("scale_n", C.c_void_p), ("exp_bias", C.c_void_p), ("prec_a", C.c_int32),
+        ("prec_b", C.c_int32), ("block_m", C.c_int32), ("activation", C.c_int32), ("swiglu_alpha", C.c_float),
+        ("swiglu_limit", C.c_float),
     ]
+
+
+class Workspace(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("bytes", C.c_size_t)]
 
 
 class SmoothquantArgs(C.Structure):
@@ -98,10 +103,11 @@ PROTOTYPES = {
     "mi355_fused_moe_supported": (C.c_int, [C.POINTER(FusedMoeTraits)]),
     "mi355_fused_moe_workspace_size": (C.c_size_t, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
     "mi355_fused_moe_tile_rows": (C.c_int32, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
-    "mi355_fused_moegemm": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeGemmArgs), C.c_void_p]),
-    "mi355_fused_moe": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.c_void_p]),
+    "mi355_fused_moegemm": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeGemmArgs), C.POINTER(Workspace),
+                                      C.c_void_p]),
+    "mi355_fused_moe": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.POINTER(Workspace), C.c_void_p]),
     "mi355_moe_flatmm_workspace_size": (C.c_size_t, [C.c_int32, C.POINTER(FlatmmArgs)]),
-    "mi355_moe_flatmm": (C.c_int, [C.c_int32, C.POINTER(FlatmmArgs), C.c_void_p]),
+    "mi355_moe_flatmm": (C.c_int, [C.c_int32, C.POINTER(FlatmmArgs), C.POINTER(Workspace), C.c_void_p]),
     "mi355_moe_permute_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int32] * 8 + [C.c_void_p]),
     "mi355_moe_smoothquant": (C.c_int, [C.POINTER(SmoothquantArgs), C.c_int32, C.c_void_p]),
     "mi355_moe_rowwise_quant": (C.c_int, [C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_int32, C.c_void_p,

@@ -183,7 +183,8 @@ __attribute__((visibility("default"))) size_t
 mi355_fused_moe_workspace_size(const mi355_fused_moe_traits* traits, int32_t tokens, int32_t num_experts,
                                int32_t topk, int32_t hidden_size, int32_t intermediate_size)
 {
-    if(traits == nullptr || check_traits(*traits) != MI355_MOE_OK)
+    if(traits == nullptr || check_traits(*traits) != MI355_MOE_OK ||
+       !sizes_in_range(tokens, num_experts, topk, hidden_size, intermediate_size))
         return 0;
     return workspace_layout(*traits, tokens, num_experts, topk, hidden_size, intermediate_size).total;
 }
@@ -192,59 +193,37 @@ __attribute__((visibility("default"))) int32_t
 mi355_fused_moe_tile_rows(const mi355_fused_moe_traits* traits, int32_t tokens, int32_t num_experts, int32_t topk,
                           int32_t hidden_size, int32_t intermediate_size)
 {
-    if(traits == nullptr || check_traits(*traits) != MI355_MOE_OK || num_experts <= 0)
+    if(traits == nullptr || check_traits(*traits) != MI355_MOE_OK ||
+       !sizes_in_range(tokens, num_experts, topk, hidden_size, intermediate_size))
         return 0;
     return gemm_tile_rows(*traits, tokens, num_experts, topk, hidden_size, intermediate_size);
 }
 
 __attribute__((visibility("default"))) int
-mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_moegemm_args* args, void* stream)
+mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_moegemm_args* args,
+                    const mi355_moe_workspace* ws, void* stream)
 {
     if(traits == nullptr || args == nullptr)
         return fail(MI355_MOE_E_INVALID, "fused_moegemm: traits or args is null");
-    return launch_fused_moegemm(*traits, *args, static_cast<hipStream_t>(stream));
+    return launch_fused_moegemm(*traits, *args, ws ? ws->ptr : nullptr, ws ? ws->bytes : 0,
+                                static_cast<hipStream_t>(stream));
 }
 
-__attribute__((visibility("default"))) int
-mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* a, void* stream)
+} // extern "C"
+
+namespace {
+// sort + grouped GEMMs + combine on one stream, everything the kernels need beyond the caller's tensors in ws_ptr
+int run_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* a, void* ws_ptr, size_t ws_bytes,
+                  void* stream)
 {
-    if(traits == nullptr || a == nullptr)
-        return fail(MI355_MOE_E_INVALID, "fused_moe: traits or args is null");
     int rc = check_traits(*traits);
     if(rc != MI355_MOE_OK)
         return rc;
     if(a->block_m != traits->block_m)
         return fail(MI355_MOE_E_INVALID, "fused_moe: args.block_m=%d differs from traits.block_m=%d",
                     a->block_m, traits->block_m);
-    const WorkspaceLayout ws = workspace_layout(*traits, a->num_tokens, a->num_experts, a->topk,
-                                                a->hidden_size, a->intermediate_size);
-    if(a->ws_ptr == nullptr || a->ws_bytes < ws.total)
-        return fail(MI355_MOE_E_WORKSPACE, "fused_moe: workspace of %zu bytes needed, %zu given", ws.total,
-                    a->ws_ptr ? a->ws_bytes : (size_t)0);
-
-    // the combine writes every element of o, so the sort does not need to zero it
-    mi355_moe_sorting_args s{};
-    s.p_topk_ids              = a->topk_ids_ptr;
-    s.p_weights               = a->topk_weight_ptr;
-    s.p_local_expert_mask     = traits->local_expert_masking ? a->local_expert_mask_ptr : nullptr;
-    s.p_local_tokens          = nullptr;
-    s.p_sorted_token_ids      = a->sorted_token_ids_ptr;
-    s.p_sorted_weights        = a->sorted_weight_ptr;
-    s.p_sorted_expert_ids     = a->sorted_expert_ids_ptr;
-    s.p_total_tokens_post_pad = a->num_sorted_tiles_ptr;
-    s.p_moe_buf               = nullptr;
-    s.p_ws                    = static_cast<char*>(a->ws_ptr) + ws.sort_off;
-    s.tokens                  = a->num_tokens;
-    s.unit_size               = a->block_m;
-    s.num_experts             = a->num_experts;
-    s.topk                    = a->topk;
     if(traits->local_expert_masking && a->local_expert_mask_ptr == nullptr)
         return fail(MI355_MOE_E_INVALID, "fused_moe: local_expert_masking set but mask pointer is null");
-    const GemmPlan plan = make_gemm_plan(*traits, a->ws_ptr, a->num_tokens, a->num_experts, a->topk, a->hidden_size,
-                                         a->intermediate_size);
-    rc = launch_moe_sorting(s, static_cast<hipStream_t>(stream), &plan);
-    if(rc != MI355_MOE_OK)
-        return rc;
 
     mi355_fused_moegemm_args g{};
     g.a_ptr                 = a->a_ptr;
@@ -259,15 +238,56 @@ mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args
     g.sorted_weight_ptr     = a->sorted_weight_ptr;
     g.sorted_expert_ids_ptr = a->sorted_expert_ids_ptr;
     g.num_sorted_tiles_ptr  = a->num_sorted_tiles_ptr;
-    g.ws_ptr                = a->ws_ptr;
-    g.ws_bytes              = a->ws_bytes;
     g.hidden_size           = a->hidden_size;
     g.intermediate_size     = a->intermediate_size;
     g.num_tokens            = a->num_tokens;
     g.num_experts           = a->num_experts;
     g.topk                  = a->topk;
     g.stride_token          = a->stride_token;
-    return launch_fused_moegemm(*traits, g, static_cast<hipStream_t>(stream), /*prep_done=*/true);
+    // every host-side check of both halves comes before the first launch: a rejected call has written nothing
+    rc = validate_fused_moegemm(*traits, g, ws_ptr, ws_bytes);
+    if(rc != MI355_MOE_OK)
+        return rc;
+    if(a->num_tokens > 0 && (a->topk_ids_ptr == nullptr || a->topk_weight_ptr == nullptr))
+        return fail(MI355_MOE_E_INVALID, "fused_moe: topk_ids or topk_weight is null");
+    const WorkspaceLayout wl = workspace_layout(*traits, a->num_tokens, a->num_experts, a->topk,
+                                                a->hidden_size, a->intermediate_size);
+
+    // the combine writes every element of o, so the sort does not need to zero it
+    mi355_moe_sorting_args s{};
+    s.p_topk_ids              = a->topk_ids_ptr;
+    s.p_weights               = a->topk_weight_ptr;
+    s.p_local_expert_mask     = traits->local_expert_masking ? a->local_expert_mask_ptr : nullptr;
+    s.p_local_tokens          = nullptr;
+    s.p_sorted_token_ids      = a->sorted_token_ids_ptr;
+    s.p_sorted_weights        = a->sorted_weight_ptr;
+    s.p_sorted_expert_ids     = a->sorted_expert_ids_ptr;
+    s.p_total_tokens_post_pad = a->num_sorted_tiles_ptr;
+    s.p_moe_buf               = nullptr;
+    // the example's own sort workspace when the caller passes one, else the slice of the library workspace
+    s.p_ws                    = a->ws_ptr != nullptr ? a->ws_ptr : static_cast<char*>(ws_ptr) + wl.sort_off;
+    s.tokens                  = a->num_tokens;
+    s.unit_size               = a->block_m;
+    s.num_experts             = a->num_experts;
+    s.topk                    = a->topk;
+    const GemmPlan plan = make_gemm_plan(*traits, ws_ptr, a->num_tokens, a->num_experts, a->topk, a->hidden_size,
+                                         a->intermediate_size);
+    rc = launch_moe_sorting(s, static_cast<hipStream_t>(stream), &plan);
+    if(rc != MI355_MOE_OK)
+        return rc;
+    return launch_fused_moegemm(*traits, g, ws_ptr, ws_bytes, static_cast<hipStream_t>(stream), /*prep_done=*/true);
+}
+} // namespace
+
+extern "C" {
+
+__attribute__((visibility("default"))) int
+mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* a, const mi355_moe_workspace* ws,
+                void* stream)
+{
+    if(traits == nullptr || a == nullptr)
+        return fail(MI355_MOE_E_INVALID, "fused_moe: traits or args is null");
+    return run_fused_moe(traits, a, ws ? ws->ptr : nullptr, ws ? ws->bytes : 0, stream);
 }
 
 __attribute__((visibility("default"))) size_t
@@ -276,11 +296,12 @@ mi355_moe_flatmm_workspace_size(int32_t kind, const mi355_moe_flatmm_args* args)
     return args != nullptr ? moe_flatmm_workspace_bytes(kind, *args) : 0;
 }
 
-__attribute__((visibility("default"))) int mi355_moe_flatmm(int32_t kind, const mi355_moe_flatmm_args* args, void* stream)
+__attribute__((visibility("default"))) int
+mi355_moe_flatmm(int32_t kind, const mi355_moe_flatmm_args* args, const mi355_moe_workspace* ws, void* stream)
 {
     if(args == nullptr)
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: args is null");
-    return launch_moe_flatmm(kind, *args, static_cast<hipStream_t>(stream));
+    return launch_moe_flatmm(kind, *args, ws ? ws->ptr : nullptr, ws ? ws->bytes : 0, static_cast<hipStream_t>(stream));
 }
 
 __attribute__((visibility("default"))) int

@@ -425,7 +425,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
 // large-tile kernel
 inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
 {
-    const int64_t avg = tokens * topk / experts;
+    const int64_t avg = tokens * topk / std::max(experts, 1);
     const int eb  = t.prec_i == MI355_MOE_BF16 ? 2 : 1;
     const int y_b = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
     // the large-tile kernel addresses each operand as a base plus a 32-bit byte offset
@@ -562,13 +562,31 @@ GemmPlan make_gemm_plan(const mi355_fused_moe_traits& t, void* ws_ptr, int32_t t
     return g;
 }
 
-int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a, hipStream_t stream,
-                         bool prep_done)
+bool sizes_in_range(int32_t tokens, int32_t experts, int32_t topk, int32_t hidden, int32_t inter)
+{
+    return tokens >= 0 && tokens <= 0xffffff && experts > 0 && experts <= 1024 && topk > 0 && topk <= 255 && hidden > 0 &&
+           inter > 0;
+}
+
+// Everything that can be checked on the host before anything is launched: the fused entry point calls it ahead
+// of the sort, so that a rejected call leaves the caller's sort outputs and workspace untouched.
+int validate_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a, const void* ws_ptr,
+                           size_t ws_bytes)
 {
     int rc = check_traits(t);
     if(rc != MI355_MOE_OK)
         return rc;
-    if(a.num_tokens == 0)
+    const int H = a.hidden_size, I = a.intermediate_size, T = a.num_tokens, E = a.num_experts, K = a.topk;
+    if(!sizes_in_range(T, E, K, H, I) || a.stride_token < H)
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: bad sizes (H=%d I=%d T=%d E=%d K=%d stride=%d)", H, I, T, E,
+                    K, a.stride_token);
+    const WorkspaceLayout ws = workspace_layout(t, T, E, K, H, I);
+    if(ws_ptr == nullptr || ws_bytes < ws.total)
+        return fail(MI355_MOE_E_WORKSPACE, "fused_moegemm: workspace of %zu bytes needed, %zu given", ws.total,
+                    ws_ptr ? ws_bytes : (size_t)0);
+    if(reinterpret_cast<uintptr_t>(ws_ptr) % 256 != 0)
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: workspace must be 256-byte aligned");
+    if(T == 0)
         return MI355_MOE_OK; // an empty batch: nothing to compute, and its tensors may have no storage
     if(!a.a_ptr || !a.g_ptr || !a.d_ptr || !a.o_ptr || !a.sorted_token_ids_ptr || !a.sorted_weight_ptr ||
        !a.sorted_expert_ids_ptr || !a.num_sorted_tiles_ptr)
@@ -578,10 +596,6 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     const bool quant = t.prec_i != MI355_MOE_BF16;
     if(quant && (!a.a_scale_ptr || !a.g_scale_ptr || !a.d_scale_ptr))
         return fail(MI355_MOE_E_INVALID, "fused_moegemm: quantised dtypes need a_scale, g_scale and d_scale");
-    const int H = a.hidden_size, I = a.intermediate_size, T = a.num_tokens, E = a.num_experts, K = a.topk;
-    if(H <= 0 || I <= 0 || T < 0 || E <= 0 || E > 1024 || K <= 0 || K > 255 || a.stride_token < H)
-        return fail(MI355_MOE_E_INVALID, "fused_moegemm: bad sizes (H=%d I=%d T=%d E=%d K=%d stride=%d)", H, I, T, E,
-                    K, a.stride_token);
     const int eb = quant ? 1 : 2; // bytes per activation / weight element
     if(H % 32 != 0 || I % 32 != 0 || (t.prec_i == MI355_MOE_FP8 && I % 128 != 0) ||
        ((int64_t)a.stride_token * eb) % 16 != 0 || ((int64_t)a.stride_token * 2) % 16 != 0)
@@ -591,16 +605,26 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     for(const void* ptr : {a.a_ptr, a.g_ptr, a.d_ptr, static_cast<const void*>(a.o_ptr)})
         if(reinterpret_cast<uintptr_t>(ptr) % 16 != 0)
             return fail(MI355_MOE_E_INVALID, "fused_moegemm: a, g, d and o must be 16-byte aligned");
-    if(T == 0)
-        return MI355_MOE_OK;
+    const int mblk = pick_mblk(t, T, K, E, H, I);
+    if(mblk > 4 && (int64_t)T * a.stride_token * eb >= ((int64_t)1 << 32))
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: a token buffer of 4 GiB or more (stride_token=%d) is not "
+                                             "supported at this problem size", a.stride_token);
+    return MI355_MOE_OK;
+}
 
+int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a, void* ws_ptr,
+                         size_t ws_bytes, hipStream_t stream, bool prep_done)
+{
+    int rc = validate_fused_moegemm(t, a, ws_ptr, ws_bytes);
+    if(rc != MI355_MOE_OK)
+        return rc;
+    if(a.num_tokens == 0)
+        return MI355_MOE_OK;
+    const bool quant = t.prec_i != MI355_MOE_BF16;
+    const int H = a.hidden_size, I = a.intermediate_size, T = a.num_tokens, E = a.num_experts, K = a.topk;
+    const int eb = quant ? 1 : 2;
     const WorkspaceLayout ws = workspace_layout(t, T, E, K, H, I);
-    if(a.ws_ptr == nullptr || a.ws_bytes < ws.total)
-        return fail(MI355_MOE_E_WORKSPACE, "fused_moegemm: workspace of %zu bytes needed, %zu given", ws.total,
-                    a.ws_ptr ? a.ws_bytes : (size_t)0);
-    if(reinterpret_cast<uintptr_t>(a.ws_ptr) % 256 != 0)
-        return fail(MI355_MOE_E_INVALID, "fused_moegemm: workspace must be 256-byte aligned");
-    unsigned char* wsb = static_cast<unsigned char*>(a.ws_ptr);
+    unsigned char* wsb = static_cast<unsigned char*>(ws_ptr);
     int* tile_map      = reinterpret_cast<int*>(wsb + ws.map_off);
     int* inv           = reinterpret_cast<int*>(wsb + ws.inv_off);
     const int mblk     = pick_mblk(t, T, K, E, H, I);
@@ -649,9 +673,6 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     // decode-sized problems (one 32-row block per tile) have their own kernel
     const bool decode = mblk == 1 && decode_supported((int64_t)T * a.stride_token * eb, ws.max_pad * (int64_t)I * y_b,
                                                       (int64_t)2 * I * H * eb);
-    if(mblk > 4 && (int64_t)T * p.x_row_bytes >= ((int64_t)1 << 32))
-        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: a token buffer of 4 GiB or more (stride_token=%d) is not "
-                                             "supported at this problem size", a.stride_token);
     // the two large-tile GEMMs hand Y over in the slab-major layout
     p.y_slab = (mblk > 4 && ((int64_t)I * y_b) % 64 == 0) ? (int)((int64_t)I * y_b / 64) : 0;
     rc       = launch_grouped_gemm(t.prec_i, true, mblk, decode, p, ws.max_tiles, stream);
@@ -753,7 +774,7 @@ size_t moe_flatmm_workspace_bytes(int kind, const mi355_moe_flatmm_args& a)
     return flatmm_layout(kind, a, L) == MI355_MOE_OK ? L.total : 0;
 }
 
-int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stream)
+int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, size_t ws_bytes, hipStream_t stream)
 {
     FlatmmLayout L{};
     int rc = flatmm_layout(kind, a, L);
@@ -783,12 +804,12 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stre
             return fail(MI355_MOE_E_INVALID, "moe_flatmm: a, b and c must be 16-byte aligned");
     if(T == 0)
         return MI355_MOE_OK;
-    if(a.ws_ptr == nullptr || a.ws_bytes < L.total)
+    if(ws_ptr == nullptr || ws_bytes < L.total)
         return fail(MI355_MOE_E_WORKSPACE, "moe_flatmm: workspace of %zu bytes needed, %zu given", L.total,
-                    a.ws_ptr ? a.ws_bytes : (size_t)0);
-    if(reinterpret_cast<uintptr_t>(a.ws_ptr) % 256 != 0)
+                    ws_ptr ? ws_bytes : (size_t)0);
+    if(reinterpret_cast<uintptr_t>(ws_ptr) % 256 != 0)
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: workspace must be 256-byte aligned");
-    unsigned char* wsb = static_cast<unsigned char*>(a.ws_ptr);
+    unsigned char* wsb = static_cast<unsigned char*>(ws_ptr);
     int* tile_map      = reinterpret_cast<int*>(wsb + L.map_off);
     int* inv           = reinterpret_cast<int*>(wsb + L.inv_off);
     const int mblk     = L.mblk;

@@ -29,9 +29,16 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
 int gemm_tile_rows(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk, int32_t hidden,
                    int32_t inter);
 
+// true when the sizes are ones the path can index (24-bit token ids, 8-bit slots, at most 1024 experts)
+bool sizes_in_range(int32_t tokens, int32_t experts, int32_t topk, int32_t hidden, int32_t inter);
+
+// host-side checks of launch_fused_moegemm, launching nothing
+int validate_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a, const void* ws_ptr,
+                           size_t ws_bytes);
+
 // prep_done: the tile list and the inverse map were already written by the sort (GemmPlan)
-int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a,
-                         hipStream_t stream, bool prep_done = false);
+int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moegemm_args& a, void* ws_ptr,
+                         size_t ws_bytes, hipStream_t stream, bool prep_done = false);
 
 // the plan the sort has to fill for launch_fused_moegemm(..., prep_done = true)
 GemmPlan make_gemm_plan(const mi355_fused_moe_traits& t, void* ws_ptr, int32_t tokens, int32_t experts,
@@ -51,7 +58,7 @@ bool decode_supported(int64_t x_bytes, int64_t y_bytes, int64_t w_expert_bytes);
 int launch_gemm_decode(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream);
 
 size_t moe_flatmm_workspace_bytes(int kind, const mi355_moe_flatmm_args& a);
-int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, hipStream_t stream);
+int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, size_t ws_bytes, hipStream_t stream);
 
 int launch_permute_weights(const void* src, void* dst, int32_t experts, int32_t n, int32_t k, int32_t elem_bytes,
                            int32_t nw, int32_t kw, int32_t kv, int32_t inverse, hipStream_t stream);

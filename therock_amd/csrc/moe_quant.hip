@@ -90,9 +90,12 @@ __device__ inline float quantise_row(const uint16_t* __restrict__ xr, const floa
                 amax = fmaxf(amax, fabsf(t[i]));
         }
         amax          = block_max_256(amax, s_red);
-        const float s = (amax > 0.f || !unit_scale_when_zero) ? amax / qmx : 1.0f;
+        // a row of zeros: the scale written is 1 (row-wise quant) or 0 (smooth-quant, as amax / qmax gives);
+        // either way the row's codes are 0, never the 0 / 0 the plain formula would convert
+        const float s_out = (amax > 0.f || !unit_scale_when_zero) ? amax / qmx : 1.0f;
+        const float s     = amax > 0.f ? s_out : 1.0f;
         if(threadIdx.x == 0)
-            *scale_out = s;
+            *scale_out = s_out;
         auto store = [&](int c, const float (&o)[8]) {
             uint32_t w[2] = {0u, 0u};
 #pragma unroll
@@ -121,9 +124,12 @@ __device__ inline float quantise_row(const uint16_t* __restrict__ xr, const floa
         for(int c = threadIdx.x; c < cols; c += 256)
             amax = fmaxf(amax, fabsf(bf16_bits_to_float(xr[c]) * (SMOOTH ? sr[c] : 1.0f)));
         amax          = block_max_256(amax, s_red);
-        const float s = (amax > 0.f || !unit_scale_when_zero) ? amax / qmx : 1.0f;
+        // a row of zeros: the scale written is 1 (row-wise quant) or 0 (smooth-quant, as amax / qmax gives);
+        // either way the row's codes are 0, never the 0 / 0 the plain formula would convert
+        const float s_out = (amax > 0.f || !unit_scale_when_zero) ? amax / qmx : 1.0f;
+        const float s     = amax > 0.f ? s_out : 1.0f;
         if(threadIdx.x == 0)
-            *scale_out = s;
+            *scale_out = s_out;
         for(int c = threadIdx.x; c < cols; c += 256)
             qr[c] = quantise_one<FP8>((bf16_bits_to_float(xr[c]) * (SMOOTH ? sr[c] : 1.0f)) / s);
         return amax;
@@ -226,10 +232,11 @@ __global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t
                 amax = fmaxf(amax, fabsf(b[i]));
         }
         amax            = block_max_256(amax, s_red[k & 1]); // two buffers: one barrier per slot suffices
-        const float ys  = amax / qmx;
-        const int64_t r = (int64_t)k * tokens + t;
+        const float ys_out = amax / qmx;
+        const float ys     = amax > 0.f ? ys_out : 1.0f; // a row of zeros: scale 0, codes 0 (not 0 / 0)
+        const int64_t r    = (int64_t)k * tokens + t;
         if(threadIdx.x == 0)
-            yscale[r] = ys;
+            yscale[r] = ys_out;
         unsigned char* qr = qy + r * y_stride;
         auto store = [&](int c, const float (&o)[8]) {
             uint32_t w[2] = {0u, 0u};

@@ -99,7 +99,8 @@ class fused_moe_args:
     y_smooth_scale_ptr: object = None
     local_expert_mask_ptr: object = None
     o_ptr: object = None
-    ws_ptr: object = None
+    ws_ptr: object = None       # CK's example: the sort's workspace; may stay None (the library workspace holds it)
+    workspace: object = None    # device tensor of fused_moe_get_workspace_size() bytes, passed beside the arguments
     topk_ids_ptr: object = None
     topk_weight_ptr: object = None
     sorted_token_ids_ptr: object = None
@@ -148,8 +149,17 @@ def fused_moe_get_workspace_size(traits: fused_moe_traits, tokens, num_experts, 
                                                           intermediate_size))
 
 
-def _ws_bytes(ws) -> int:
-    return 0 if ws is None else ws.numel() * ws.element_size()
+def _workspace(ws) -> "_lib.Workspace":
+    return _lib.Workspace(_ptr(ws), 0 if ws is None else ws.numel() * ws.element_size())
+
+
+def _fused_args(a: fused_moe_args) -> "_lib.FusedMoeArgs":
+    return _lib.FusedMoeArgs(_ptr(a.a_ptr), _ptr(a.a_scale_ptr), _ptr(a.g_ptr), _ptr(a.d_ptr), _ptr(a.g_scale_ptr),
+                             _ptr(a.d_scale_ptr), _ptr(a.y_smooth_scale_ptr), _ptr(a.local_expert_mask_ptr),
+                             _ptr(a.o_ptr), _ptr(a.ws_ptr), _ptr(a.topk_ids_ptr),
+                             _ptr(a.topk_weight_ptr), _ptr(a.sorted_token_ids_ptr), _ptr(a.sorted_weight_ptr),
+                             _ptr(a.sorted_expert_ids_ptr), _ptr(a.num_sorted_tiles_ptr), a.block_m, a.hidden_size,
+                             a.intermediate_size, a.num_tokens, a.num_experts, a.topk, a.stride_token)
 
 
 def fused_moe(traits: fused_moe_traits, a: fused_moe_args, stream=None) -> float:
@@ -159,13 +169,9 @@ def fused_moe(traits: fused_moe_traits, a: fused_moe_args, stream=None) -> float
     t = traits.pod()
     if not lib.mi355_fused_moe_supported(C.byref(t)):
         return -1.0
-    f = _lib.FusedMoeArgs(_ptr(a.a_ptr), _ptr(a.a_scale_ptr), _ptr(a.g_ptr), _ptr(a.d_ptr), _ptr(a.g_scale_ptr),
-                          _ptr(a.d_scale_ptr), _ptr(a.y_smooth_scale_ptr), _ptr(a.local_expert_mask_ptr),
-                          _ptr(a.o_ptr), _ptr(a.ws_ptr), _ws_bytes(a.ws_ptr), _ptr(a.topk_ids_ptr),
-                          _ptr(a.topk_weight_ptr), _ptr(a.sorted_token_ids_ptr), _ptr(a.sorted_weight_ptr),
-                          _ptr(a.sorted_expert_ids_ptr), _ptr(a.num_sorted_tiles_ptr), a.block_m, a.hidden_size,
-                          a.intermediate_size, a.num_tokens, a.num_experts, a.topk, a.stride_token)
-    rc = lib.mi355_fused_moe(C.byref(t), C.byref(f), _stream(stream))
+    f = _fused_args(a)
+    ws = _workspace(a.workspace)
+    rc = lib.mi355_fused_moe(C.byref(t), C.byref(f), C.byref(ws), _stream(stream))
     if rc == _lib.E_UNSUPPORTED:
         return -1.0
     _check(rc, "fused_moe")
@@ -181,9 +187,10 @@ def fused_moegemm(traits: fused_moe_traits, a: fused_moe_args, stream=None) -> f
     g = _lib.FusedMoeGemmArgs(_ptr(a.a_ptr), _ptr(a.a_scale_ptr), _ptr(a.g_ptr), _ptr(a.d_ptr), _ptr(a.g_scale_ptr),
                               _ptr(a.d_scale_ptr), _ptr(a.y_smooth_scale_ptr), _ptr(a.o_ptr),
                               _ptr(a.sorted_token_ids_ptr), _ptr(a.sorted_weight_ptr), _ptr(a.sorted_expert_ids_ptr),
-                              _ptr(a.num_sorted_tiles_ptr), _ptr(a.ws_ptr), _ws_bytes(a.ws_ptr), a.hidden_size,
+                              _ptr(a.num_sorted_tiles_ptr), a.hidden_size,
                               a.intermediate_size, a.num_tokens, a.num_experts, a.topk, a.stride_token)
-    rc = lib.mi355_fused_moegemm(C.byref(t), C.byref(g), _stream(stream))
+    ws = _workspace(a.workspace)
+    rc = lib.mi355_fused_moegemm(C.byref(t), C.byref(g), C.byref(ws), _stream(stream))
     if rc == _lib.E_UNSUPPORTED:
         return -1.0
     _check(rc, "fused_moegemm")
@@ -206,24 +213,52 @@ def rowwise_quant(x, q_dtype: str, stream=None):
 GEMM1_GATE_ONLY, GEMM1_GATE_UP, GEMM2 = 0, 1, 2
 
 
-def moe_flatmm(kind: int, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens: int, topk: int, block_m: int,
-               sorted_weights=None, scale_m=None, scale_n=None, stream=None):
-    """One grouped GEMM of the MoE layer as its own launch (ck_tile's MoeFlatmm conventions): kind
-    GEMM1_GATE_UP writes c[token * topk + slot, :N/2] = silu(gate) * up, GEMM1_GATE_ONLY c[.., :N] = silu(a b^T),
-    kind GEMM2 adds the weighted down projection of a[token * topk + slot] to c[token].  b is [experts, N, K]."""
+ACT_SILU, ACT_SWIGLU = 0, 1
+
+
+def _flatmm_args(kind, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens, topk, block_m, sorted_weights,
+                 scale_m, scale_n, exp_bias, activation, swiglu_alpha, swiglu_limit, n_padded_zeros, k_padded_zeros):
     import torch
 
     experts, n, k = b.shape
     dt = {torch.bfloat16: "bf16", torch.int8: "int8", torch.float8_e4m3fn: "fp8", torch.uint8: "fp8"}
-    args = _lib.FlatmmArgs(_ptr(sorted_ids), _ptr(sorted_weights), _ptr(sorted_eid), _ptr(max_token_id), _ptr(a), _ptr(b),
-                           _ptr(c), _ptr(scale_m), _ptr(scale_n), None, None, 0, num_tokens, experts, topk, 1,
-                           sorted_ids.numel(), n, k, a.stride(0), k, c.stride(0), _lib.DTYPES[dt[a.dtype]],
-                           _lib.DTYPES[dt[b.dtype]], block_m)
+    return _lib.FlatmmArgs(_ptr(sorted_ids), _ptr(sorted_weights), _ptr(sorted_eid), _ptr(max_token_id), _ptr(a), _ptr(b),
+                           _ptr(c), num_tokens, experts, topk, 1, sorted_ids.numel(), n, k, a.stride(0), k, c.stride(0),
+                           n_padded_zeros, k_padded_zeros, _ptr(scale_m), _ptr(scale_n), _ptr(exp_bias),
+                           _lib.DTYPES[dt[a.dtype]], _lib.DTYPES[dt[b.dtype]], block_m, activation, swiglu_alpha,
+                           swiglu_limit)
+
+
+def moe_flatmm_get_workspace_size(kind: int, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens: int, topk: int,
+                                  block_m: int, **kw) -> int:
+    """Bytes of the workspace tensor moe_flatmm needs for these arguments (0: no kernel)."""
+    args = _flatmm_args(kind, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens, topk, block_m, None, None, None,
+                        None, ACT_SILU, 1.702, 7.0, kw.get("n_padded_zeros", 0), kw.get("k_padded_zeros", 0))
+    return int(_lib.load().mi355_moe_flatmm_workspace_size(kind, C.byref(args)))
+
+
+def moe_flatmm(kind: int, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens: int, topk: int, block_m: int,
+               sorted_weights=None, scale_m=None, scale_n=None, exp_bias=None, activation: int = ACT_SILU,
+               swiglu_alpha: float = 1.702, swiglu_limit: float = 7.0, n_padded_zeros: int = 0, k_padded_zeros: int = 0,
+               workspace=None, stream=None):
+    """One grouped GEMM of the MoE layer as its own launch (ck_tile's MoeFlatmm conventions): kind
+    GEMM1_GATE_UP writes c[token * topk + slot, :N/2] = act(gate, up), GEMM1_GATE_ONLY c[.., :N] = act(a b^T),
+    kind GEMM2 adds the weighted down projection of a[token * topk + slot] to c[token].  b is [experts, N, K].
+    workspace: a device tensor of moe_flatmm_get_workspace_size() bytes owned by the caller (it must stay alive
+    until the launches have run); when None one is allocated here on torch's current stream, which is then the
+    only stream the call may use."""
+    import torch
+
+    args = _flatmm_args(kind, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens, topk, block_m, sorted_weights,
+                        scale_m, scale_n, exp_bias, activation, swiglu_alpha, swiglu_limit, n_padded_zeros, k_padded_zeros)
     lib = _lib.load()
-    ws_bytes = int(lib.mi355_moe_flatmm_workspace_size(kind, C.byref(args)))
-    ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=a.device)
-    args.ws_ptr, args.ws_bytes = _ptr(ws), ws_bytes
-    rc = lib.mi355_moe_flatmm(kind, C.byref(args), _stream(stream))
+    if workspace is None:
+        if stream is not None and _stream(stream) != _stream(None):
+            raise ValueError("moe_flatmm: pass a caller-owned workspace when launching on a stream other than the current one")
+        ws_bytes = int(lib.mi355_moe_flatmm_workspace_size(kind, C.byref(args)))
+        workspace = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=a.device)
+    ws = _workspace(workspace)
+    rc = lib.mi355_moe_flatmm(kind, C.byref(args), C.byref(ws), _stream(stream))
     if rc == _lib.E_UNSUPPORTED:
         return -1.0
     _check(rc, "moe_flatmm")
@@ -312,7 +347,7 @@ def make_args(traits: fused_moe_traits, buf: MoeBuffers, a, g, d, topk_ids, topk
         E = num_experts
     return fused_moe_args(
         a_ptr=a, a_scale_ptr=a_scale, g_ptr=g, d_ptr=d, g_scale_ptr=g_scale, d_scale_ptr=d_scale,
-        local_expert_mask_ptr=local_expert_mask, o_ptr=buf.out, ws_ptr=buf.ws, topk_ids_ptr=topk_ids,
+        local_expert_mask_ptr=local_expert_mask, o_ptr=buf.out, workspace=buf.ws, topk_ids_ptr=topk_ids,
         topk_weight_ptr=topk_weight, sorted_token_ids_ptr=buf.sorted_ids, sorted_weight_ptr=buf.sorted_w,
         sorted_expert_ids_ptr=buf.sorted_eid, num_sorted_tiles_ptr=buf.total, block_m=traits.block_m,
         hidden_size=H, intermediate_size=n0 if traits.gate_only else n0 // 2, num_tokens=T, num_experts=E, topk=topk_ids.shape[1],
