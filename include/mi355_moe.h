@@ -226,6 +226,19 @@ int mi355_fused_moegemm(const mi355_fused_moe_traits* traits, const mi355_fused_
 int mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* args,
                     const mi355_moe_workspace* ws, void* stream);
 
+/* The same pass with no workspace argument, for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc) and have no workspace to pass.  It has no counterpart
+ * in ck_tile, whose fused kernel needs no workspace.  The intermediates live in a buffer of
+ * mi355_fused_moe_static_ws_capacity() bytes (96 MiB, enough for the decode regime: 256 tokens of a 128-expert
+ * top-8 layer with hidden 4096 and intermediate 1536) that is part of the library's device image: every GPU the
+ * library runs on holds it from the first use of the library until the process ends.  Nothing is allocated or
+ * freed by the call.  A problem whose mi355_fused_moe_workspace_size() exceeds the capacity is rejected with
+ * MI355_MOE_E_WORKSPACE.  All calls on one GPU share the buffer: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered and safe.  The buffer's device address is looked up on the first
+ * call on each device (not a stream operation; make that first call outside a capture). */
+size_t mi355_fused_moe_static_ws_capacity(void);
+int mi355_fused_moe_static_ws(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* args, void* stream);
+
 /* per-row dynamic quantisation of bf16 activations, the step in front of the quantised path:
  * scale[m] = amax(row)/qmax, q = convert(saturate(x/scale)) (host/reference/reference_rowwise_quantization2d.hpp:12-31);
  * as in ck_tile the int8 conversion truncates toward zero (core/numeric/int8.hpp:101), e4m3 rounds to nearest even;

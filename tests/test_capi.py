@@ -96,6 +96,24 @@ def test_sizes_out_of_range_are_rejected_on_the_host():
     assert lib.mi355_fused_moe(C.byref(t), C.byref(f), None, None) == _lib.E_WORKSPACE
 
 
+def test_static_workspace_entry_point_rejects_oversized_problems_on_the_host():
+    lib = _lib.load()
+    cap = lib.mi355_fused_moe_static_ws_capacity()
+    assert cap == 96 << 20
+    t = _lib.FusedMoeTraits(1, 1, 0, 3, 3, 3, 3, 32, 1, 0, 0, 0)
+    assert lib.mi355_fused_moe_workspace_size(C.byref(t), 8192, 256, 8, 7168, 2048) > cap
+    f = _lib.FusedMoeArgs(block_m=32, hidden_size=7168, intermediate_size=2048, num_tokens=8192, num_experts=256, topk=8,
+                          stride_token=7168)
+    assert lib.mi355_fused_moe_static_ws(C.byref(t), C.byref(f), None) == _lib.E_WORKSPACE
+    assert b"library-owned" in lib.mi355_moe_last_error()
+    f.num_experts = 0
+    assert lib.mi355_fused_moe_static_ws(C.byref(t), C.byref(f), None) == _lib.E_INVALID
+    # the benchmark's decode regime fits
+    t8 = _lib.FusedMoeTraits(2, 2, 0, 3, 3, 3, 3, 32, 1, 0, 0, 0)
+    for tokens in (16, 64, 256):
+        assert 0 < lib.mi355_fused_moe_workspace_size(C.byref(t8), tokens, 128, 8, 4096, 1536) <= cap
+
+
 def test_host_only_entry_points():
     lib = _lib.load()
     assert lib.mi355_moe_version() == 200

@@ -106,6 +106,8 @@ PROTOTYPES = {
     "mi355_fused_moegemm": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeGemmArgs), C.POINTER(Workspace),
                                       C.c_void_p]),
     "mi355_fused_moe": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.POINTER(Workspace), C.c_void_p]),
+    "mi355_fused_moe_static_ws_capacity": (C.c_size_t, []),
+    "mi355_fused_moe_static_ws": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.c_void_p]),
     "mi355_moe_flatmm_workspace_size": (C.c_size_t, [C.c_int32, C.POINTER(FlatmmArgs)]),
     "mi355_moe_flatmm": (C.c_int, [C.c_int32, C.POINTER(FlatmmArgs), C.POINTER(Workspace), C.c_void_p]),
     "mi355_moe_permute_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int32] * 8 + [C.c_void_p]),

@@ -92,6 +92,42 @@ void profile_mark(int kind, hipStream_t stream, bool begin)
 
 using namespace mi355;
 
+// ---- library-owned workspace of mi355_fused_moe_static_ws(): device memory that exists from the moment the code
+// object is loaded, so that the entry point never allocates.  In host code `scratch` is only a handle for
+// hipGetSymbolAddress: the address kernels and copies use is the one that call returns, and every device has its own
+// copy of the array at its own address.
+constexpr size_t kStaticWsBytes = (size_t)96 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticWsBytes];
+
+namespace {
+// device address of `scratch` on the current device, resolved once per device; nullptr (and the error text) on failure
+void* static_workspace()
+{
+    constexpr int kMaxDev = 64;
+    static void* ptr[kMaxDev] = {};
+    static std::mutex mu;
+    int dev = 0;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev)
+    {
+        fail(MI355_MOE_E_HIP, "fused_moe_static_ws: no current device (or a device index above %d)", kMaxDev - 1);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if(ptr[dev] == nullptr)
+    {
+        void* p            = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if(e != hipSuccess || p == nullptr)
+        {
+            fail(MI355_MOE_E_HIP, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        ptr[dev] = p;
+    }
+    return ptr[dev];
+}
+} // namespace
+
 extern "C" {
 
 __attribute__((visibility("default"))) const char* mi355_moe_last_error(void) { return error_buffer(); }
@@ -288,6 +324,31 @@ mi355_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args
     if(traits == nullptr || a == nullptr)
         return fail(MI355_MOE_E_INVALID, "fused_moe: traits or args is null");
     return run_fused_moe(traits, a, ws ? ws->ptr : nullptr, ws ? ws->bytes : 0, stream);
+}
+
+__attribute__((visibility("default"))) size_t mi355_fused_moe_static_ws_capacity(void) { return kStaticWsBytes; }
+
+__attribute__((visibility("default"))) int
+mi355_fused_moe_static_ws(const mi355_fused_moe_traits* traits, const mi355_fused_moe_args* a, void* stream)
+{
+    if(traits == nullptr || a == nullptr)
+        return fail(MI355_MOE_E_INVALID, "fused_moe_static_ws: traits or args is null");
+    int rc = check_traits(*traits);
+    if(rc != MI355_MOE_OK)
+        return rc;
+    if(!sizes_in_range(a->num_tokens, a->num_experts, a->topk, a->hidden_size, a->intermediate_size))
+        return fail(MI355_MOE_E_INVALID, "fused_moe_static_ws: bad sizes (H=%d I=%d T=%d E=%d K=%d)", a->hidden_size,
+                    a->intermediate_size, a->num_tokens, a->num_experts, a->topk);
+    const size_t need = workspace_layout(*traits, a->num_tokens, a->num_experts, a->topk, a->hidden_size,
+                                         a->intermediate_size).total;
+    if(need > kStaticWsBytes)
+        return fail(MI355_MOE_E_WORKSPACE,
+                    "fused_moe_static_ws: this problem needs a workspace of %zu bytes, the library-owned one holds %zu; "
+                    "call mi355_fused_moe with a workspace of your own", need, kStaticWsBytes);
+    void* ws_ptr = static_workspace();
+    if(ws_ptr == nullptr)
+        return MI355_MOE_E_HIP;
+    return run_fused_moe(traits, a, ws_ptr, kStaticWsBytes, stream);
 }
 
 __attribute__((visibility("default"))) size_t

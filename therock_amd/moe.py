@@ -178,6 +178,24 @@ def fused_moe(traits: fused_moe_traits, a: fused_moe_args, stream=None) -> float
     return 0.0
 
 
+def fused_moe_static_ws_capacity() -> int:
+    return int(_lib.load().mi355_fused_moe_static_ws_capacity())
+
+
+def fused_moe_static_ws(traits: fused_moe_traits, a: fused_moe_args, stream=None) -> float:
+    """fused_moe() on the library-owned workspace: allocates nothing, a.workspace is ignored.  Problems that need
+    more than fused_moe_static_ws_capacity() bytes raise; calls that overlap on one GPU race."""
+    lib = _lib.load()
+    t = traits.pod()
+    if not lib.mi355_fused_moe_supported(C.byref(t)):
+        return -1.0
+    rc = lib.mi355_fused_moe_static_ws(C.byref(t), C.byref(_fused_args(a)), _stream(stream))
+    if rc == _lib.E_UNSUPPORTED:
+        return -1.0
+    _check(rc, "fused_moe_static_ws")
+    return 0.0
+
+
 def fused_moegemm(traits: fused_moe_traits, a: fused_moe_args, stream=None) -> float:
     """GEMM half only: consumes sorted_* / num_sorted_tiles already written by moe_sorting."""
     lib = _lib.load()
