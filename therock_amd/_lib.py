@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmi355_moe.so")
+# MI355_MOE_LIB names another build of the same library (A/B timing of two builds in one process each)
+LIB_PATH = os.environ.get("MI355_MOE_LIB") or os.path.join(_HERE, "libmi355_moe.so")
 
 OK, E_UNSUPPORTED, E_INVALID, E_HIP, E_WORKSPACE = 0, -1, -2, -3, -4
 DTYPES = {"bf16": 0, "fp8": 1, "int8": 2, "fp32": 3, "int32": 4, "fp16": 5}

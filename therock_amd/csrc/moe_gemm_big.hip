@@ -319,15 +319,26 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if(w_role)
-            {
-                if constexpr(!kW8)
-                    issue_w(k + 4, par_tag, nt_tag);
-                else if constexpr(PAR == 0)
-                    issue_w((k >> 1) + 4, std::integral_constant<int, -1>{}, nt_tag);
-            }
-            else
-                issue_x(k + 2, XG);
+            auto issue_next = [&]() __attribute__((always_inline)) {
+                if(w_role)
+                {
+                    if constexpr(!kW8)
+                        issue_w(k + 4, par_tag, nt_tag);
+                    else if constexpr(PAR == 0)
+                        issue_w((k >> 1) + 4, std::integral_constant<int, -1>{}, nt_tag);
+                }
+                else
+                    issue_x(k + 2, XG);
+            };
+            // Where in the step the transfers go out: right here, or after the MFMAs of token block kIssueAfter.  The
+            // buffers they write are free from the barrier on either way, but issued here the handful of scalar and
+            // DMA instructions sits between the barrier and the first operand fetch, on every wave's critical path;
+            // issued behind the first MFMAs it runs while the matrix pipe is busy (measured -2 % fp8, -4 % bf16 on the
+            // gate+up GEMM).  After all MFMAs is too late (the transfers then start up to a step later), and the fp8
+            // down GEMM has no register to spare for the scheduling fence this needs.
+            constexpr int kIssueAfter = kMx ? -1 : 1;
+            if constexpr(kIssueAfter < 0 || NB <= kIssueAfter)
+                issue_next();
 
             // first unit of the pair that holds this step's weight bytes
             const int pair0          = kW8 ? (k >> 2) << 1 : (k & ~1);
@@ -386,6 +397,12 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                     {
                         acc[i][0] = mfma<MODE>(wf[0], xf[i], xs[i], acc[i][0]);
                         acc[i][1] = mfma<MODE>(wf[1], xf[i], xs[i], acc[i][1]);
+                    }
+                    if(kIssueAfter >= 0 && NB > kIssueAfter && s == 0 && i == kIssueAfter)
+                    {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_next();
+                        __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }

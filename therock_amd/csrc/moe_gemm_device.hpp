@@ -386,92 +386,161 @@ __device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTr
     }
 }
 
-// Shared tail of both GEMM kernels.  NBLK token blocks per wave: block i covers sorted rows
+// Shared tail of both GEMM kernels, in three parts so that a kernel that walks several tiles can fetch the
+// operands early (load), make sure they have arrived at a point of its choosing (pin) and do the arithmetic and
+// the stores later (apply).  NBLK token blocks per wave: block i covers sorted rows
 // row0 + first_row + i * row_step + r32; wblk is the wave's first 32-row weight block of the tile.
 // SKIP_PAD (gemm1): look the sorted id up and do not store partial rows of padding ids - worth the
 // load where padding dominates (decode: a handful of real rows per 32-row unit).
-template <int MODE, bool GEMM0, int NBLK, bool SKIP_PAD>
-__device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2], int expert,
-                                    int row0, int nrows, int first_row, int row_step, int nblk_live, int n_base,
-                                    int wblk, int r32, int kg)
+template <int NBLK>
+struct EpilogueRows
 {
-    // ---- one batch of loads
-    float sc0[16], sc1[16];
+    float sa[NBLK];  // per-row scale
+    bool real[NBLK]; // the row holds a token (not a padding id)
+    int orow[NBLK];  // output row (the launchers keep tokens * topk below 2^31)
+};
+struct EpilogueColumns
+{
+    int col_a, col_b; // first output column of the wave's two accumulator groups for this lane
+    bool a_ok, b_ok, paired;
+};
+template <int NBLK>
+struct EpilogueOperands
+{
+    float sc0[16], sc1[16]; // per-channel scales of the wave's two accumulator groups
+    EpilogueRows<NBLK> rows;
+    EpilogueColumns cols;
+};
+
+template <bool GEMM0>
+__device__ inline EpilogueColumns epilogue_columns(const GemmParams& p, int n_base, int wblk, int kg)
+{
     // gate+up tiles pair weight block 2w (gate) with 2w+1 (up) on the same 32 columns; every other kind of
     // tile (down, gate-only) maps its blocks 2w and 2w+1 to consecutive groups of 32 columns
-    const bool paired = GEMM0 && !p.gate_only;
-    const int col_a = paired ? n_base + wblk * 32 + 16 * kg : n_base + (wblk * 2) * 32 + 16 * kg;
-    const int col_b = paired ? col_a : col_a + 32;
-    const bool a_ok = (paired ? n_base + wblk * 32 : n_base + wblk * 64) < p.n_out;
-    const bool b_ok = paired ? a_ok : (n_base + wblk * 64 + 32) < p.n_out;
-    const float* sbase = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total : nullptr;
-    load_channel_scales(sbase && a_ok ? sbase + col_a : nullptr, sc0);
-    load_channel_scales(sbase && b_ok ? sbase + (paired ? p.n_out + col_a : col_b) : nullptr, sc1);
-    float sa[NBLK];
-    bool real[NBLK];
-    int orow[NBLK]; // output row (the launchers keep tokens * topk below 2^31)
+    EpilogueColumns c;
+    c.paired = GEMM0 && !p.gate_only;
+    c.col_a  = c.paired ? n_base + wblk * 32 + 16 * kg : n_base + (wblk * 2) * 32 + 16 * kg;
+    c.col_b  = c.paired ? c.col_a : c.col_a + 32;
+    c.a_ok   = (c.paired ? n_base + wblk * 32 : n_base + wblk * 64) < p.n_out;
+    c.b_ok   = c.paired ? c.a_ok : (n_base + wblk * 64 + 32) < p.n_out;
+    return c;
+}
+
+template <bool GEMM0, int NBLK, bool SKIP_PAD>
+__device__ inline void load_epilogue_rows(const GemmParams& p, EpilogueRows<NBLK>& o, int row0, int nrows, int first_row,
+                                          int row_step, int r32)
+{
 #pragma unroll
     for(int i = 0; i < NBLK; i++)
     {
-        sa[i]   = 1.0f;
-        real[i] = true;
-        orow[i] = row0 + first_row + i * row_step + r32;
+        o.sa[i]   = 1.0f;
+        o.real[i] = true;
+        o.orow[i] = row0 + first_row + i * row_step + r32;
         if((GEMM0 && (p.x_scale != nullptr || p.slot_rows > 0)) || (!GEMM0 && SKIP_PAD))
         {
             const int r   = min(first_row + i * row_step + r32, nrows - 1); // clamped: always a valid cell
             const int sid = p.sorted_ids[row0 + r];
             const int tok = sid & 0xffffff;
-            real[i]       = tok < p.tokens;
+            o.real[i]     = tok < p.tokens;
             if constexpr(GEMM0)
             {
                 if(p.x_scale != nullptr)
-                    sa[i] = real[i] ? p.x_scale[tok] : 0.0f;
+                    o.sa[i] = o.real[i] ? p.x_scale[tok] : 0.0f;
                 if(p.slot_rows > 0)
-                    orow[i] = real[i] ? (int)slot_row(sid, p.slot_rows) : 0;
+                    o.orow[i] = o.real[i] ? (int)slot_row(sid, p.slot_rows) : 0;
             }
         }
     }
-    // every load above completes here, on every path: a load left pending on a path that does not use
-    // its result would make the compiler guard later register reuse with a wait for all vector memory
-    // operations - inside the caller's K loop when the caller is a persistent kernel
-#pragma unroll
-    for(int v = 0; v < 16; v++)
-        asm volatile("" : "+v"(sc0[v]), "+v"(sc1[v]));
+}
+
+template <int NBLK>
+__device__ inline void pin_epilogue_rows(EpilogueRows<NBLK>& o)
+{
 #pragma unroll
     for(int i = 0; i < NBLK; i++)
-        asm volatile("" : "+v"(sa[i]), "+v"(orow[i]));
-    // ---- apply
+    {
+        int real = o.real[i];
+        asm volatile("" : "+v"(o.sa[i]), "+v"(o.orow[i]), "+v"(real));
+        o.real[i] = real != 0;
+    }
+}
+
+template <int MODE, bool GEMM0, int NBLK, bool SKIP_PAD>
+__device__ inline void load_epilogue(const GemmParams& p, EpilogueOperands<NBLK>& o, int expert, int row0, int nrows,
+                                     int first_row, int row_step, int n_base, int wblk, int r32, int kg)
+{
+    o.cols             = epilogue_columns<GEMM0>(p, n_base, wblk, kg);
+    const float* sbase = p.w_scale ? p.w_scale + (int64_t)expert * p.n_total : nullptr;
+    load_channel_scales(sbase && o.cols.a_ok ? sbase + o.cols.col_a : nullptr, o.sc0);
+    load_channel_scales(sbase && o.cols.b_ok ? sbase + (o.cols.paired ? p.n_out + o.cols.col_a : o.cols.col_b) : nullptr,
+                        o.sc1);
+    load_epilogue_rows<GEMM0, NBLK, SKIP_PAD>(p, o.rows, row0, nrows, first_row, row_step, r32);
+}
+
+// Every load of load_epilogue completes here, on every path: a load left pending on a path that does not use
+// its result would make the compiler guard later register reuse with a wait for all vector memory
+// operations - inside the caller's K loop when the caller walks several tiles.
+template <int NBLK>
+__device__ inline void pin_epilogue(EpilogueOperands<NBLK>& o)
+{
+#pragma unroll
+    for(int v = 0; v < 16; v++)
+        asm volatile("" : "+v"(o.sc0[v]), "+v"(o.sc1[v]));
+    pin_epilogue_rows(o.rows);
+}
+
+// one token block of a wave: scales, activation, packing, stores
+template <int MODE, bool GEMM0, int NBLK>
+__device__ inline void apply_epilogue_block(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[2],
+                                            const float (&sc0)[16], const float (&sc1)[16], const EpilogueRows<NBLK>& rows,
+                                            const EpilogueColumns& c, int i, int row0, int nrows, int first_row,
+                                            int row_step, int r32, int kg)
+{
+    const int r = first_row + i * row_step + r32;
     if constexpr(GEMM0)
     {
-        // block by block, so that a block's accumulators are dead before the next block's temporaries
-        // are needed (the large-tile kernel has no registers to spare)
-#pragma unroll
-        for(int i = 0; i < NBLK; i++)
-        {
-            if(i >= nblk_live)
-                continue;
-            const bool st = first_row + i * row_step + r32 < nrows && (p.slot_rows == 0 || real[i]);
-            if(a_ok)
-                epilogue_gemm0<MODE>(p, acc[i][0], acc[i][1], sc0, sc1, sa[i], orow[i], st, col_a, kg, !paired);
-            if(!paired && b_ok) // gate-only tile: the second accumulator holds the next 32 gate columns
-                epilogue_gemm0<MODE>(p, acc[i][1], acc[i][1], sc1, sc1, sa[i], orow[i], st, col_b, kg, true);
-        }
+        const bool st = r < nrows && (p.slot_rows == 0 || rows.real[i]);
+        if(c.a_ok)
+            epilogue_gemm0<MODE>(p, acc[0], acc[1], sc0, sc1, rows.sa[i], rows.orow[i], st, c.col_a, kg, !c.paired);
+        if(!c.paired && c.b_ok) // gate-only tile: the second accumulator holds the next 32 gate columns
+            epilogue_gemm0<MODE>(p, acc[1], acc[1], sc1, sc1, rows.sa[i], rows.orow[i], st, c.col_b, kg, true);
     }
     else
     {
-#pragma unroll
-        for(int i = 0; i < NBLK; i++)
-        {
-            if(i >= nblk_live)
-                continue;
-            const int r        = first_row + i * row_step + r32;
-            const bool in_tile = r < nrows;
-            if(a_ok)
-                epilogue_gemm1<MODE>(p, acc[i][0], sc0, row0 + r, in_tile && real[i], col_a);
-            if(b_ok)
-                epilogue_gemm1<MODE>(p, acc[i][1], sc1, row0 + r, in_tile && real[i], col_b);
-        }
+        const bool in_tile = r < nrows;
+        if(c.a_ok)
+            epilogue_gemm1<MODE>(p, acc[0], sc0, row0 + r, in_tile && rows.real[i], c.col_a);
+        if(c.b_ok)
+            epilogue_gemm1<MODE>(p, acc[1], sc1, row0 + r, in_tile && rows.real[i], c.col_b);
     }
+}
+
+template <int MODE, bool GEMM0, int NBLK>
+__device__ inline void apply_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2],
+                                      const EpilogueOperands<NBLK>& o, int row0, int nrows, int first_row, int row_step,
+                                      int nblk_live, int r32, int kg)
+{
+    // block by block, so that a block's accumulators are dead before the next block's temporaries
+    // are needed (the large-tile kernel has no registers to spare)
+#pragma unroll
+    for(int i = 0; i < NBLK; i++)
+    {
+        if(i >= nblk_live)
+            continue;
+        apply_epilogue_block<MODE, GEMM0, NBLK>(p, acc[i], o.sc0, o.sc1, o.rows, o.cols, i, row0, nrows, first_row, row_step,
+                                                r32, kg);
+    }
+}
+
+template <int MODE, bool GEMM0, int NBLK, bool SKIP_PAD>
+__device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2], int expert,
+                                    int row0, int nrows, int first_row, int row_step, int nblk_live, int n_base,
+                                    int wblk, int r32, int kg)
+{
+    EpilogueOperands<NBLK> o;
+    load_epilogue<MODE, GEMM0, NBLK, SKIP_PAD>(p, o, expert, row0, nrows, first_row, row_step, n_base, wblk, r32, kg);
+    pin_epilogue(o);
+    apply_epilogue<MODE, GEMM0, NBLK>(p, acc, o, row0, nrows, first_row, row_step, nblk_live, r32, kg);
 }
 
 } // namespace gemm
