@@ -253,10 +253,21 @@ def ck_moe_sorting(topk_ids, weights, experts, unit, local_expert_mask=None, ski
 
 
 # ------------------------------------------------------------------- unfused grouped GEMMs
+ACT_SILU, ACT_SWIGLU = 0, 1
+
+
+def moe_act(act, gate, linear, alpha=1.702, limit=7.0):
+    """The oracle's scalar activation (ck_tile::moe::MoeSilu / Swiglu, host branch)."""
+    f = lib().moe_oracle_moe_act
+    f.restype = C.c_float
+    return float(f(C.c_int(act), C.c_float(gate), C.c_float(linear), C.c_float(alpha), C.c_float(limit)))
+
+
 def moe_gemm(kind, sorted_ids, sorted_eid, sorted_w, post_pad, block_m, a, b, c, num_tokens, topk,
-             scale_a=None, scale_b=None):
-    """Oracle of ck_tile's unfused MoE GEMMs (kind 1 = gate+up with SiLU*up, 2 = down with weights, added to
-    c).  a, b fp32; c bf16 bits [rows, >= N or N/2], updated in place and returned."""
+             scale_a=None, scale_b=None, exp_bias=None, act=ACT_SILU, alpha=1.702, limit=7.0, n_padded_zeros=0,
+             k_padded_zeros=0):
+    """Oracle of ck_tile's unfused MoE GEMMs (kind 0 = gate only, 1 = gate+up with act(gate, up), 2 = down with
+    weights, added to c).  a, b fp32; c bf16 bits [rows, >= N or N/2], updated in place and returned."""
     a, b = _c(a, np.float32), _c(b, np.float32)
     c = np.ascontiguousarray(c, dtype=np.uint16)
     E, N, K = b.shape
@@ -266,15 +277,18 @@ def moe_gemm(kind, sorted_ids, sorted_eid, sorted_w, post_pad, block_m, a, b, c,
     f.restype = C.c_int
     rc = f(C.c_int(kind), _p(ids), _p(eid), _p(w), C.c_int32(int(post_pad)), C.c_int32(block_m), _p(a), _p(b), _p(c),
            C.c_int32(num_tokens), C.c_int32(topk), C.c_int32(N), C.c_int32(K), C.c_int32(a.shape[1]),
-           C.c_int32(c.shape[1]), _p(_c(scale_a, np.float32)), _p(_c(scale_b, np.float32)))
+           C.c_int32(c.shape[1]), _p(_c(scale_a, np.float32)), _p(_c(scale_b, np.float32)),
+           _p(_c(exp_bias, np.float32)), C.c_int32(act), C.c_float(alpha), C.c_float(limit), C.c_int32(n_padded_zeros),
+           C.c_int32(k_padded_zeros))
     if rc != 0:
         raise ValueError(f"moe_oracle_moe_gemm failed ({rc})")
     return c
 
 
 def ck_moe_gemm_gpu(kind, sorted_ids, sorted_eid, sorted_w, post_pad, block_m, a_bf16, b_bf16, c_bf16, num_tokens, topk,
-                    scale_a=None, scale_b=None):
-    """ck_tile::reference_moe_gemm_gpu (a device kernel: needs a GPU) on bf16 operands given as bf16 bits.
+                    scale_a=None, scale_b=None, exp_bias=None, act=ACT_SILU):
+    """ck_tile::reference_moe_gemm_gpu (a device kernel: needs a GPU) on bf16 operands given as bf16 bits, with
+    ck_tile's own activation functor (MoeSilu, or Swiglu with its default alpha 1.702 and limit 7).
     c is updated in place (the down kind adds to it) and returned."""
     r = ck_ref_gpu()
     if r is None:
@@ -288,7 +302,8 @@ def ck_moe_gemm_gpu(kind, sorted_ids, sorted_eid, sorted_w, post_pad, block_m, a
     r.ck_ref_moe_gemm_gpu.restype = C.c_int
     rc = r.ck_ref_moe_gemm_gpu(C.c_int32(kind), _p(ids), _p(eid), C.c_int32(int(post_pad)), _p(a), _p(b), _p(c), _p(w),
                                C.c_int32(num_tokens), C.c_int32(block_m), C.c_int32(topk), C.c_int32(ids.size),
-                               C.c_int32(E), C.c_int32(N), C.c_int32(K), _p(sa), _p(sb))
+                               C.c_int32(E), C.c_int32(N), C.c_int32(K), _p(sa), _p(sb), _p(_c(exp_bias, np.float32)),
+                               C.c_int32(act))
     if rc != 0:
         raise RuntimeError(f"ck_ref_moe_gemm_gpu failed ({rc})")
     return c

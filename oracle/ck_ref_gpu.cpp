@@ -12,6 +12,8 @@
 #include "ck_tile/ops/elementwise/unary_element_wise_operation.hpp"
 #include "ck_tile/ops/common/tensor_layout.hpp"
 #include "ck_tile/host/reference/reference_moe_gemm.hpp"
+#include "ck_tile/host/kernel_launch.hpp"
+#include "ck_tile/ops/flatmm/kernel/moe_flatmm_kernel.hpp" // ck_tile::moe::MoeSilu, ck_tile::moe::Swiglu
 
 using ck_tile::index_t;
 
@@ -20,30 +22,21 @@ namespace {
 // ck_tile's reference of the unfused MoE GEMMs is a device kernel (reference_moe_gemm.hpp:18-330): this
 // wrapper stages host buffers through device memory and runs it on the current GPU.  A, B, C hold bf16
 // bits; scale_a [rows of A] and scale_b [E, N] are fp32 (pass ones for "no scale": the kernel always reads
-// them); activation of the gate+up kind is silu(gate) * up as ck_tile::moe::MoeSilu
-// (ops/flatmm/kernel/moe_flatmm_kernel.hpp:139-149).  Returns 0, or a negative HIP error code.
-struct RefMoeSilu
-{
-    template <typename T>
-    CK_TILE_HOST_DEVICE T operator()(T gate, T linear = 1) const
-    {
-        ck_tile::element_wise::Silu{}(gate, gate);
-        return gate * linear;
-    }
-};
-
-template <int KIND>
+// them); bias [E, N] fp32 or null.  The activation is ck_tile's own functor, default-constructed by the
+// kernel: ck_tile::moe::MoeSilu or ck_tile::moe::Swiglu (alpha 1.702, limit 7;
+// ops/flatmm/kernel/moe_flatmm_kernel.hpp:139-183).  Returns 0, or a negative HIP error code.
+template <int KIND, typename Act>
 static int run_moe_gemm_gpu(const int32_t* ids, const int32_t* eid, int32_t max_token_id, const uint16_t* A,
                             const uint16_t* B, uint16_t* C, const float* w, int32_t T, int32_t block, int32_t topk,
                             int32_t M, int32_t E, int32_t N, int32_t K, int64_t a_rows, int64_t c_rows, int32_t c_cols,
-                            const float* sa, const float* sb)
+                            const float* sa, const float* sb, const float* bias)
 {
     using bf16 = ck_tile::bf16_t;
     using Row  = ck_tile::tensor_layout::gemm::RowMajor;
     using Col  = ck_tile::tensor_layout::gemm::ColumnMajor;
     int32_t *d_ids = nullptr, *d_eid = nullptr, *d_max = nullptr;
     bf16 *d_a = nullptr, *d_b = nullptr, *d_c = nullptr;
-    float *d_w = nullptr, *d_sa = nullptr, *d_sb = nullptr;
+    float *d_w = nullptr, *d_sa = nullptr, *d_sb = nullptr, *d_bias = nullptr;
     const size_t tiles = (size_t)(M + block - 1) / block;
 #define CKR(x)                      \
     do                              \
@@ -70,37 +63,54 @@ static int run_moe_gemm_gpu(const int32_t* ids, const int32_t* eid, int32_t max_
     CKR(hipMemcpy(d_w, w, sizeof(float) * M, hipMemcpyHostToDevice));
     CKR(hipMemcpy(d_sa, sa, sizeof(float) * a_rows, hipMemcpyHostToDevice));
     CKR(hipMemcpy(d_sb, sb, sizeof(float) * (size_t)E * N, hipMemcpyHostToDevice));
-    ck_tile::reference_moe_gemm_gpu<bf16, bf16, float, bf16, Row, Col, Row, KIND, RefMoeSilu>(
-        d_ids, d_eid, d_max, d_a, d_b, d_c, d_w, T, block, topk, M, N, K, K, K, c_cols, 1, 1, K, d_sa, d_sb, nullptr);
+    if(bias != nullptr)
+    {
+        CKR(hipMalloc(&d_bias, sizeof(float) * (size_t)E * N));
+        CKR(hipMemcpy(d_bias, bias, sizeof(float) * (size_t)E * N, hipMemcpyHostToDevice));
+    }
+    ck_tile::reference_moe_gemm_gpu<bf16, bf16, float, bf16, Row, Col, Row, KIND, Act>(
+        d_ids, d_eid, d_max, d_a, d_b, d_c, d_w, T, block, topk, M, N, K, K, K, c_cols, 1, 1, K, d_sa, d_sb, d_bias);
     CKR(hipGetLastError());
     CKR(hipDeviceSynchronize());
     CKR(hipMemcpy(C, d_c, 2 * (size_t)c_rows * c_cols, hipMemcpyDeviceToHost));
 #undef CKR
     for(void* ptr : {(void*)d_ids, (void*)d_eid, (void*)d_max, (void*)d_a, (void*)d_b, (void*)d_c, (void*)d_w,
-                     (void*)d_sa, (void*)d_sb})
+                     (void*)d_sa, (void*)d_sb, (void*)d_bias})
         (void)hipFree(ptr);
     return 0;
+}
+
+template <typename Act>
+static int dispatch_kind(int32_t kind, const int32_t* ids, const int32_t* eid, int32_t max_token_id, const uint16_t* A,
+                         const uint16_t* B, uint16_t* C, const float* w, int32_t T, int32_t block, int32_t topk, int32_t M,
+                         int32_t E, int32_t N, int32_t K, const float* sa, const float* sb, const float* bias)
+{
+    if(kind == 0)
+        return run_moe_gemm_gpu<0, Act>(ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, T, (int64_t)T * topk,
+                                        N, sa, sb, bias);
+    if(kind == 1)
+        return run_moe_gemm_gpu<1, Act>(ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, T, (int64_t)T * topk,
+                                        N / 2, sa, sb, bias);
+    if(kind == 2)
+        return run_moe_gemm_gpu<2, Act>(ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, (int64_t)T * topk, T,
+                                        N, sa, sb, bias);
+    return -1;
 }
 
 } // namespace
 
 extern "C" {
 
+// act: 0 = ck_tile::moe::MoeSilu, 1 = ck_tile::moe::Swiglu (default alpha and limit); bias may be null
 __attribute__((visibility("default"))) int
 ck_ref_moe_gemm_gpu(int32_t kind, const int32_t* ids, const int32_t* eid, int32_t max_token_id, const uint16_t* A,
                     const uint16_t* B, uint16_t* C, const float* w, int32_t T, int32_t block, int32_t topk, int32_t M,
-                    int32_t E, int32_t N, int32_t K, const float* sa, const float* sb)
+                    int32_t E, int32_t N, int32_t K, const float* sa, const float* sb, const float* bias, int32_t act)
 {
-    if(kind == 0)
-        return run_moe_gemm_gpu<0>(ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, T, (int64_t)T * topk, N,
-                                   sa, sb);
-    if(kind == 1)
-        return run_moe_gemm_gpu<1>(ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, T, (int64_t)T * topk,
-                                   N / 2, sa, sb);
-    if(kind == 2)
-        return run_moe_gemm_gpu<2>(ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, (int64_t)T * topk, T, N,
-                                   sa, sb);
-    return -1;
+    if(act == 1)
+        return dispatch_kind<ck_tile::moe::Swiglu>(kind, ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, sa, sb,
+                                                   bias);
+    return dispatch_kind<ck_tile::moe::MoeSilu>(kind, ids, eid, max_token_id, A, B, C, w, T, block, topk, M, E, N, K, sa, sb,
+                                                bias);
 }
-
 }

@@ -482,22 +482,47 @@ ORACLE_API int moe_oracle_fused_moe(const void* a, int a_dt, const float* a_scal
 
 /* ---------------------------------------------------------------------- unfused grouped GEMMs
  * reference_moe_gemm.hpp:41-241 with row-major A and C, B as [experts, N, K], one scale per row of A
- * (scale_a, may be NULL) and per output channel (scale_b [experts, N], may be NULL), no expert bias.
+ * (scale_a, may be NULL) and per output channel (scale_b [experts, N], may be NULL), an optional expert
+ * bias [experts, N] added to the scaled dot products (:205-211).
  *   kind 1 (gate+up): row r of the sorted list with token t, slot s: A row t, C row t*topk+s,
- *       C[., n] = bf16( silu(acc_gate) * acc_up ), gate = B rows [0, N/2), up = B rows [N/2, N)
- *   kind 0 (gate only): the same rows, C[., n] = bf16( silu(acc) ) over all N rows of B (:216-219 with up = 1)
- *   kind 2 (down)   : A row t*topk+s, C row t; ck_tile adds bf16(acc * w[r]) to C with packed bf16 atomics
- *       (:214-238).  Here a token's slots are summed in fp32 in slot order on top of the bf16 value C holds
- *       and rounded once: the same quantity without the order-dependent bf16 rounding of every partial sum.
+ *       C[., n] = bf16( act(acc_gate + bias, acc_up + bias_up) ), gate = B rows [0, N/2), up = B rows [N/2, N)
+ *   kind 0 (gate only): the same rows, C[., n] = bf16( act(acc + bias, 1) ) over all N rows of B (:216-219)
+ *   kind 2 (down)   : A row t*topk+s, C row t; ck_tile adds bf16((acc + bias) * w[r]) to C with packed bf16
+ *       atomics (:214-238).  Here a token's slots are summed in fp32 in slot order on top of the bf16 value C
+ *       holds and rounded once: the same quantity without the order-dependent bf16 rounding of every partial sum.
+ * act: 0 = ck_tile::moe::MoeSilu, silu(gate) * linear; 1 = ck_tile::moe::Swiglu{alpha, limit}:
+ *       gate' = min(gate, limit), linear' = clamp(linear, -limit, limit), gate' * sigmoid(alpha * gate') * (linear' + 1)
+ *       (ops/flatmm/kernel/moe_flatmm_kernel.hpp:139-183, host branch: a true division, no rcp).
+ * n_padded_zeros / k_padded_zeros (MoeFlatmmHostArgs, moe_flatmm_kernel.hpp:29-30): the last rows of every
+ * expert's B, respectively the last columns of A and B, are padding that the device kernel never fetches (its
+ * tensor views end before them, :600-606): they count as zeros.
  * A and B are fp32 (the caller up-converts), C is bf16 bits. */
+static inline float moe_act_f32(int act, float gate, float linear, float alpha, float limit)
+{
+    if(act == 0)
+        return silu_f32(gate) * linear;
+    gate   = gate < limit ? gate : limit;
+    linear = linear < limit ? (linear > -limit ? linear : -limit) : limit;
+    return gate * (1.0f / (1.0f + expf(alpha * -gate))) * (linear + 1.0f);
+}
+
+ORACLE_API float moe_oracle_moe_act(int act, float gate, float linear, float alpha, float limit)
+{
+    return moe_act_f32(act, gate, linear, alpha, limit);
+}
+
 ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const int32_t* sorted_eid, const float* sorted_w,
                                    int32_t max_token_id, int32_t tokens_per_block, const float* A, const float* B,
                                    uint16_t* C, int32_t num_tokens, int32_t topk, int32_t N, int32_t K, int32_t stride_a,
-                                   int32_t stride_c, const float* scale_a, const float* scale_b)
+                                   int32_t stride_c, const float* scale_a, const float* scale_b, const float* exp_bias,
+                                   int32_t act, float alpha, float limit, int32_t n_padded_zeros, int32_t k_padded_zeros)
 {
-    if(kind < 0 || kind > 2)
+    if(kind < 0 || kind > 2 || act < 0 || act > 1 || n_padded_zeros < 0 || n_padded_zeros > N || k_padded_zeros < 0 ||
+       k_padded_zeros > K)
         return -1;
     const int32_t pn = kind == 1 ? N / 2 : N;
+    const int32_t nv = N - n_padded_zeros; /* rows of B that exist */
+    const int32_t kv = K - k_padded_zeros; /* columns that exist */
     float* acc2      = NULL; /* kind 2: fp32 sums [tokens, N], started from C */
     if(kind == 2)
     {
@@ -526,20 +551,24 @@ ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const in
             {
                 const float* b = B + (e * N + n) * K;
                 float acc      = 0.f;
-                for(int32_t k = 0; k < K; k++)
-                    acc += a[k] * b[k];
+                if(n < nv)
+                    for(int32_t k = 0; k < kv; k++)
+                        acc += a[k] * b[k];
                 acc *= sa * (scale_b ? scale_b[e * N + n] : 1.0f);
+                acc += exp_bias ? exp_bias[e * N + n] : 0.f;
                 if(kind == 1)
                 {
                     const float* bu = B + (e * N + n + pn) * K;
                     float up        = 0.f;
-                    for(int32_t k = 0; k < K; k++)
-                        up += a[k] * bu[k];
+                    if(n + pn < nv)
+                        for(int32_t k = 0; k < kv; k++)
+                            up += a[k] * bu[k];
                     up *= sa * (scale_b ? scale_b[e * N + n + pn] : 1.0f);
-                    C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(silu_f32(acc) * up);
+                    up += exp_bias ? exp_bias[e * N + n + pn] : 0.f;
+                    C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(moe_act_f32(act, acc, up, alpha, limit));
                 }
                 else if(kind == 0)
-                    C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(silu_f32(acc));
+                    C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(moe_act_f32(act, acc, 1.0f, alpha, limit));
                 else
                     acc2[c_row * N + n] += acc * sorted_w[r];
             }

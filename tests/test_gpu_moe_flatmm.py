@@ -97,6 +97,127 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, oracle.DT_BF16)) <= tol
 
 
+@pytest.mark.parametrize("T,E,K,H,I,unit", [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (1024, 4, 2, 512, 384, 32)])
+@pytest.mark.parametrize("kind", ["bf16", "int8", "fp8"])
+@pytest.mark.parametrize("act,with_bias", [("silu", True), ("swiglu", False), ("swiglu", True)])  # (silu, no bias) is the test above
+def test_bias_and_swiglu(T, E, K, H, I, unit, kind, act, with_bias):
+    """Expert bias and ck_tile's clamped SwiGLU (moe::Swiglu{alpha, limit}) on all three GEMM kinds, every kernel
+    family (decode, small tiles, large tiles) and every operand type."""
+    import torch
+    import therock_amd as ta
+    from tests.gpu_util import run_sorting
+
+    rng = np.random.default_rng(T + H + with_bias)
+    tol = 1e-2 if kind == "bf16" else 3e-2
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
+    w = rng.random((T, K), dtype=np.float32)
+    s_ids, s_w, s_eid, total = run_sorting(ids, w, E, unit, fill=True)
+    pp = int(total[0])
+    dev = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    bf = lambda a: torch.from_numpy(a).cuda().to(torch.bfloat16)
+    x32 = (rng.standard_normal((T, H)) * 2).astype(np.float32)
+    g32 = (rng.standard_normal((E, 2 * I, H)) * 0.1).astype(np.float32)   # gate / up values reach past the limit
+    d32 = (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32)
+    bias_g = (rng.standard_normal((E, 2 * I)) * 1.5).astype(np.float32) if with_bias else None
+    bias_d = (rng.standard_normal((E, H)) * 0.5).astype(np.float32) if with_bias else None
+    d_ids, d_w, d_eid, d_tot = dev(s_ids), dev(s_w), dev(s_eid), dev(total.astype(np.int32))
+    if kind == "bf16":
+        x, g, d = bf(x32), bf(g32), bf(d32)
+        xr, gr, dr = x.float().cpu().numpy(), g.float().cpu().numpy(), d.float().cpu().numpy()
+        sa = sg = sd = None
+    else:
+        qdt = oracle.DT_I8 if kind == "int8" else oracle.DT_E4M3
+        kw = dict(nearest=True) if kind == "int8" else {}
+        xq, sa = oracle.rowwise_quant(x32, qdt, **kw)
+        gq, sg = oracle.rowwise_quant(g32.reshape(E * 2 * I, H), qdt, **kw)
+        dq, sd = oracle.rowwise_quant(d32.reshape(E * H, I), qdt, **kw)
+        x, g, d = dev(xq), dev(gq.reshape(E, 2 * I, H)), dev(dq.reshape(E, H, I))
+        xr, gr, dr = (oracle.to_f32(xq, qdt), oracle.to_f32(gq.reshape(E, 2 * I, H), qdt),
+                      oracle.to_f32(dq.reshape(E, H, I), qdt))
+        sg, sd = sg.reshape(E, 2 * I), sd.reshape(E, H)
+    a_code = ta.ACT_SWIGLU if act == "swiglu" else ta.ACT_SILU
+    o_code = oracle.ACT_SWIGLU if act == "swiglu" else oracle.ACT_SILU
+    alpha, limit = 1.702, 7.0
+
+    y = torch.full((T * K, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert ta.moe_flatmm(ta.GEMM1_GATE_UP, x, g, y, d_ids, d_eid, d_tot, T, K, unit, scale_m=dev(sa), scale_n=dev(sg),
+                         exp_bias=dev(bias_g), activation=a_code, swiglu_alpha=alpha, swiglu_limit=limit) == 0.0
+    torch.cuda.synchronize()
+    y_ref = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, xr, gr, np.zeros((T * K, I), np.uint16), T, K, sa, sg,
+                            exp_bias=bias_g, act=o_code, alpha=alpha, limit=limit)
+    yg = y.float().cpu().numpy()
+    assert not np.isnan(yg).any()
+    assert _rel(yg, oracle.to_f32(y_ref, oracle.DT_BF16)) <= tol
+
+    g_only = g[:, :I].contiguous()
+    b_only = None if bias_g is None else np.ascontiguousarray(bias_g[:, :I])
+    s_only = None if sg is None else np.ascontiguousarray(sg[:, :I])
+    yo = torch.full((T * K, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert ta.moe_flatmm(ta.GEMM1_GATE_ONLY, x, g_only, yo, d_ids, d_eid, d_tot, T, K, unit, scale_m=dev(sa), scale_n=dev(s_only),
+                         exp_bias=dev(b_only), activation=a_code, swiglu_alpha=alpha, swiglu_limit=limit) == 0.0
+    torch.cuda.synchronize()
+    yo_ref = oracle.moe_gemm(0, s_ids, s_eid, s_w, pp, unit, xr, np.ascontiguousarray(gr[:, :I]),
+                             np.zeros((T * K, I), np.uint16), T, K, sa, s_only, exp_bias=b_only, act=o_code, alpha=alpha,
+                             limit=limit)
+    assert _rel(yo.float().cpu().numpy(), oracle.to_f32(yo_ref, oracle.DT_BF16)) <= tol
+
+    if not with_bias:
+        return  # the down GEMM has no activation
+    y_f32 = oracle.to_f32(y_ref, oracle.DT_BF16)
+    if kind == "fp8":
+        yq, sy = oracle.rowwise_quant(y_f32, oracle.DT_E4M3)
+        y_in, a_ref, s_m = dev(yq), oracle.to_f32(yq, oracle.DT_E4M3), sy
+    else:
+        y_in, a_ref, s_m = torch.from_numpy(y_ref.view(np.int16)).cuda().view(torch.bfloat16), y_f32, None
+    c = bf((rng.standard_normal((T, H)) * 0.1).astype(np.float32))
+    c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, a_ref, dr, _bits(c).copy(), T, K, s_m, sd, exp_bias=bias_d)
+    assert ta.moe_flatmm(ta.GEMM2, y_in, d, c, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w, scale_m=dev(s_m),
+                         scale_n=dev(sd), exp_bias=dev(bias_d)) == 0.0
+    torch.cuda.synchronize()
+    assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, oracle.DT_BF16)) <= tol
+
+
+@pytest.mark.parametrize("T,E,K,H,I,unit", [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (1024, 4, 2, 512, 384, 32)])
+@pytest.mark.parametrize("kind", ["bf16", "int8"])
+def test_padded_zeros(T, E, K, H, I, unit, kind):
+    """n_padded_zeros / k_padded_zeros of MoeFlatmmHostArgs: the last weight rows, respectively the last K columns,
+    hold garbage that must not reach the result."""
+    import torch
+    import therock_amd as ta
+    from tests.gpu_util import run_sorting
+
+    rng = np.random.default_rng(T + I)
+    tol = 1e-2 if kind == "bf16" else 3e-2
+    npad, kpad = 48, 64
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
+    w = rng.random((T, K), dtype=np.float32)
+    s_ids, s_w, s_eid, total = run_sorting(ids, w, E, unit, fill=True)
+    pp = int(total[0])
+    dev = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    x32 = rng.standard_normal((T, H)).astype(np.float32)
+    g32 = (rng.standard_normal((E, 2 * I, H)) * 0.05).astype(np.float32)
+    x32[:, H - kpad:] = 3.0          # what sits in the padding is large ...
+    g32[:, :, H - kpad:] = 1.0
+    g32[:, 2 * I - npad:, :] = 1.0   # ... and would dominate the result if it were read
+    bias = (rng.standard_normal((E, 2 * I))).astype(np.float32)
+    if kind == "bf16":
+        x, g = dev(x32).to(torch.bfloat16), dev(g32).to(torch.bfloat16)
+        xr, gr, sa, sg = x.float().cpu().numpy(), g.float().cpu().numpy(), None, None
+    else:
+        xq, sa = oracle.rowwise_quant(x32, oracle.DT_I8, nearest=True)
+        gq, sg = oracle.rowwise_quant(g32.reshape(E * 2 * I, H), oracle.DT_I8, nearest=True)
+        x, g = dev(xq), dev(gq.reshape(E, 2 * I, H))
+        xr, gr, sg = oracle.to_f32(xq, oracle.DT_I8), oracle.to_f32(gq.reshape(E, 2 * I, H), oracle.DT_I8), sg.reshape(E, 2 * I)
+    y = torch.full((T * K, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    d_ids, d_eid, d_tot = dev(s_ids), dev(s_eid), dev(total.astype(np.int32))
+    assert ta.moe_flatmm(ta.GEMM1_GATE_UP, x, g, y, d_ids, d_eid, d_tot, T, K, unit, scale_m=dev(sa), scale_n=dev(sg),
+                         exp_bias=dev(bias), n_padded_zeros=npad, k_padded_zeros=kpad) == 0.0
+    torch.cuda.synchronize()
+    y_ref = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, xr, gr, np.zeros((T * K, I), np.uint16), T, K, sa, sg,
+                            exp_bias=bias, n_padded_zeros=npad, k_padded_zeros=kpad)
+    assert _rel(y.float().cpu().numpy(), oracle.to_f32(y_ref, oracle.DT_BF16)) <= tol
+
+
 def test_unsupported_and_errors():
     import torch
     import therock_amd as ta
@@ -145,4 +266,27 @@ def test_oracle_against_ck_tile_device_reference(T, E, K, H, I, unit):
     c0 = bf(rng.standard_normal((T, H)) * 0.1)
     o_ck = oracle.ck_moe_gemm_gpu(2, s_ids, s_eid, s_w, pp, unit, y_or, d, c0.copy(), T, K)
     o_or = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, f32(y_or), f32(d), c0.copy(), T, K)
+    assert _rel(f32(o_ck), f32(o_or)) < 8e-3
+
+    # expert bias and ck_tile's own moe::Swiglu functor (default alpha 1.702, limit 7), inputs scaled so that the
+    # clamps bite; the device functor uses exp and an approximate reciprocal: a few bf16 ulps on a few elements
+    bias = (rng.standard_normal((E, 2 * I)) * 2).astype(np.float32)
+    x4 = bf(f32(x) * 4)
+    for act in (oracle.ACT_SILU, oracle.ACT_SWIGLU):
+        y_ck = oracle.ck_moe_gemm_gpu(1, s_ids, s_eid, s_w, pp, unit, x4, g, np.zeros((T * K, I), np.uint16), T, K, sa, sg,
+                                      exp_bias=bias, act=act)
+        y_or = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, f32(x4), f32(g), np.zeros((T * K, I), np.uint16), T, K, sa, sg,
+                               exp_bias=bias, act=act)
+        assert (np.abs(f32(y_or)) >= 7.0).any() or act == oracle.ACT_SILU
+        diff = np.abs(y_ck.astype(np.int32) - y_or.astype(np.int32))
+        assert diff.max() <= 2 and (diff != 0).mean() < 0.02, (act, diff.max(), (diff != 0).mean())
+        z_ck = oracle.ck_moe_gemm_gpu(0, s_ids, s_eid, s_w, pp, unit, x4, g, np.zeros((T * K, 2 * I), np.uint16), T, K, sa, sg,
+                                      exp_bias=bias, act=act)
+        z_or = oracle.moe_gemm(0, s_ids, s_eid, s_w, pp, unit, f32(x4), f32(g), np.zeros((T * K, 2 * I), np.uint16), T, K, sa,
+                               sg, exp_bias=bias, act=act)
+        diff = np.abs(z_ck.astype(np.int32) - z_or.astype(np.int32))
+        assert diff.max() <= 2 and (diff != 0).mean() < 0.02, (act, diff.max(), (diff != 0).mean())
+    bias_d = (rng.standard_normal((E, H)) * 0.5).astype(np.float32)
+    o_ck = oracle.ck_moe_gemm_gpu(2, s_ids, s_eid, s_w, pp, unit, y_or, d, c0.copy(), T, K, exp_bias=bias_d)
+    o_or = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, f32(y_or), f32(d), c0.copy(), T, K, exp_bias=bias_d)
     assert _rel(f32(o_ck), f32(o_or)) < 8e-3

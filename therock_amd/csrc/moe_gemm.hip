@@ -358,7 +358,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
                                                            const float* __restrict__ sorted_w,
                                                            unsigned char* __restrict__ out, int topk, int hidden,
                                                            int64_t out_row_bytes, int accumulate,
-                                                           const float* __restrict__ slot_scale)
+                                                           const float* __restrict__ slot_scale,
+                                                           const float* __restrict__ bias,
+                                                           const int* __restrict__ sorted_eid, int unit)
 {
     const int t  = blockIdx.x;
     const int h0 = (blockIdx.y * 256 + threadIdx.x) * 8;
@@ -410,6 +412,14 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
             {
                 acc[2 * i] += w[j] * __uint_as_float(v[j][i] << 16);
                 acc[2 * i + 1] += w[j] * __uint_as_float(v[j][i] & 0xffff0000u);
+            }
+            if(bias != nullptr) // stand-alone down GEMM with an expert bias: (dot + bias) * top-k weight
+            {
+                const float wk  = sorted_w[pos[j]];
+                const float* bp = bias + (int64_t)sorted_eid[pos[j] / unit] * hidden + h0;
+#pragma unroll
+                for(int i = 0; i < 8; i++)
+                    acc[i] += wk * bp[i];
             }
         }
     }
@@ -704,7 +714,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     KernelTimer timer(MI355_MOE_K_COMBINE, stream);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, inv,
                        static_cast<const float*>(a.sorted_weight_ptr), static_cast<unsigned char*>(a.o_ptr), K, H,
-                       (int64_t)a.stride_token * 2, 0, static_cast<const float*>(nullptr));
+                       (int64_t)a.stride_token * 2, 0, static_cast<const float*>(nullptr), static_cast<const float*>(nullptr),
+                       static_cast<const int*>(nullptr), 1);
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
@@ -740,6 +751,11 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
        a.block_m < 1 || a.block_m > 1024 || a.k_batch > 1 || (g1 && !go && a.N % 2 != 0))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: bad sizes (tokens=%d experts=%d topk=%d N=%d K=%d block_m=%d k_batch=%d)",
                     a.NumTokens, a.NumExperts, a.TopK, a.N, a.K, a.block_m, a.k_batch);
+    if(a.n_padded_zeros < 0 || a.n_padded_zeros >= a.N || a.k_padded_zeros < 0 || a.k_padded_zeros >= a.K)
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: padded zeros (n=%d of N=%d, k=%d of K=%d)", a.n_padded_zeros, a.N,
+                    a.k_padded_zeros, a.K);
+    if(a.activation != MI355_MOE_ACT_SILU && a.activation != MI355_MOE_ACT_SWIGLU)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: activation %d (0 = MoeSilu, 1 = Swiglu)", a.activation);
     L.hidden = g1 ? a.K : a.N;
     L.inter  = g1 ? (go ? a.N : a.N / 2) : a.K;
     if(L.hidden % 32 != 0 || L.inter % 32 != 0 || (f8 && !g1 && L.inter % 128 != 0))
@@ -750,6 +766,17 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
     L.traits       = mi355_fused_moe_traits{prec, prec, MI355_MOE_BF16, MI355_MOE_FP32, MI355_MOE_FP32, MI355_MOE_FP32,
                                             MI355_MOE_FP32, a.block_m, 1, 0, 0, 0};
     L.mblk         = pick_mblk(L.traits, a.NumTokens, a.TopK, a.NumExperts, L.hidden, L.inter);
+    if(a.k_padded_zeros > 0)
+    {
+        // the K loops of the small-tile and decode kernels stop at any multiple of 16 bytes; the large-tile kernel
+        // wants whole 128-byte lines
+        const int a_b = a.prec_a == MI355_MOE_BF16 ? 2 : 1, b_b = a.prec_b == MI355_MOE_BF16 ? 2 : 1;
+        const int k_eff = a.K - a.k_padded_zeros;
+        if((k_eff * a_b) % 16 != 0 || (k_eff * b_b) % 16 != 0 || (f8 && k_eff % 32 != 0))
+            return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: K - k_padded_zeros = %d must cover whole 16-byte pieces of A "
+                                                 "and B (32 elements for fp8)", k_eff);
+        L.mblk = std::min(L.mblk, 4);
+    }
     L.max_pad      = (int64_t)a.TopK * a.NumTokens + (int64_t)a.NumExperts * a.block_m - a.TopK;
     L.max_tiles    = (int32_t)(a.NumExperts + L.max_pad / (L.mblk * 32) + 1);
     L.total        = 0;
@@ -789,8 +816,8 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     if(!a.p_sorted_token_ids || !a.p_sorted_expert_ids || !a.p_max_token_id || !a.a_ptr || !a.b_ptr || !a.c_ptr ||
        (!g1 && !a.p_sorted_expert_weights))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: null pointer");
-    if(a.exp_bias != nullptr)
-        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: expert bias is not implemented");
+    if(a.exp_bias != nullptr && reinterpret_cast<uintptr_t>(a.exp_bias) % 16 != 0)
+        return fail(MI355_MOE_E_INVALID, "moe_flatmm: exp_bias must be 16-byte aligned");
     if((w8 || f8) && (!a.scale_n || ((g1 || f8) && !a.scale_m)))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: quantised weights need scale_n, quantised activations scale_m");
     const int T = a.NumTokens, E = a.NumExperts, K = a.TopK, H = L.hidden, I = L.inter;
@@ -834,15 +861,19 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     p.tile_map       = tile_map;
     p.tokens         = T;
     p.slot_rows      = K;
-    p.act            = 1; // silu, the activation of ck_tile's MoeFlatmmKernel instances
+    p.act            = a.activation == MI355_MOE_ACT_SWIGLU ? 2 : 1; // MoeSilu (ck_tile's default FusedActivation) or Swiglu
+    p.swiglu_alpha   = a.swiglu_alpha;
+    p.swiglu_limit   = a.swiglu_limit;
+    p.n_padded       = a.n_padded_zeros;
+    p.bias           = g1 ? static_cast<const float*>(a.exp_bias) : nullptr; // (the down GEMM's bias is added by the combine)
     p.x              = static_cast<const unsigned char*>(a.a_ptr);
     p.x_row_bytes    = (int64_t)a.stride_A * a_b;
     p.w              = static_cast<const unsigned char*>(a.b_ptr);
     p.w_row_bytes    = (int64_t)a.K * b_b;
     p.w_expert_bytes = (int64_t)a.N * a.K * b_b;
     p.w_scale        = (w8 || f8) ? static_cast<const float*>(a.scale_n) : nullptr;
-    p.k_bytes_x      = a.K * a_b;
-    p.k_bytes_w      = a.K * b_b;
+    p.k_bytes_x      = (a.K - a.k_padded_zeros) * a_b;
+    p.k_bytes_w      = (a.K - a.k_padded_zeros) * b_b;
     const int64_t a_rows = g1 ? T : (int64_t)T * K;
     if(a_rows * p.x_row_bytes >= ((int64_t)1 << 32) && mblk > 4)
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: A of 4 GiB or more is not supported at this problem size");
@@ -877,7 +908,8 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
         KernelTimer timer(MI355_MOE_K_COMBINE, stream);
         hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + L.p_off, inv,
                            static_cast<const float*>(a.p_sorted_expert_weights), static_cast<unsigned char*>(a.c_ptr), K, H,
-                           (int64_t)a.stride_C * 2, 1, f8 ? static_cast<const float*>(a.scale_m) : nullptr);
+                           (int64_t)a.stride_C * 2, 1, f8 ? static_cast<const float*>(a.scale_m) : nullptr,
+                           static_cast<const float*>(a.exp_bias), static_cast<const int*>(a.p_sorted_expert_ids), a.block_m);
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;

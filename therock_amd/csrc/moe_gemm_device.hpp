@@ -63,6 +63,13 @@ struct GemmParams
     // fp8 gate+up GEMM of the stand-alone entry point: write bf16 instead of e4m3 with block scales
     int y_bf16;
     int max_tiles; // entries the tile list has room for (upper bound of live tiles)
+    // stand-alone GEMMs (ck_tile's MoeFlatmmHostArgs, moe_flatmm_kernel.hpp:17-31): expert bias [experts, n_total] added
+    // to the scaled dot products (null: none); the last n_padded weight rows of every expert are padding and
+    // count as zeros; act 2 = moe::Swiglu{swiglu_alpha, swiglu_limit}
+    const float* bias;
+    int n_padded;
+    float swiglu_alpha;
+    float swiglu_limit;
 };
 
 // byte offset of K byte kb of row `row` in the slab-major Y layout
@@ -286,35 +293,95 @@ __device__ inline void load_channel_scales(const float* scale, float (&out)[16])
     }
 }
 
-// gemm0: y = silu(gate) * up with the per-token scale sa and the per-channel scales folded in;
-// stored as bf16 or (fp8 path) as e4m3 with one power-of-two scale per 32 columns.  Every lane of
+// ck_tile::moe::Swiglu (moe_flatmm_kernel.hpp:149-183, device branch): gate' = min(gate, limit),
+// linear' = clamp(linear, -limit, limit), gate' * rcp(1 + exp(-alpha * gate')) * (linear' + 1)
+__device__ inline float swiglu(float gate, float linear, float alpha, float limit)
+{
+    gate   = fminf(gate, limit);
+    linear = fminf(fmaxf(linear, -limit), limit);
+    return gate * __builtin_amdgcn_rcpf(1.0f + __expf(-alpha * gate)) * (linear + 1.0f);
+}
+
+// Bias and padding of the stand-alone GEMMs for the 16 channels chan0 .. chan0 + 15 of one expert (row index
+// inside the expert's weight): v = dot * scale, then the padded channels lose their dot product and every
+// channel gains its bias.  Rare (a uniform branch at the call sites), so the bias is fetched here rather than
+// carried in registers beside the scales.
+__device__ inline void bias_and_padding(const GemmParams& p, float (&v)[16], int expert, int chan0)
+{
+    if(p.n_padded > 0)
+    {
+#pragma unroll
+        for(int i = 0; i < 16; i++)
+            v[i] = chan0 + i < p.n_total - p.n_padded ? v[i] : 0.0f;
+    }
+    if(p.bias != nullptr)
+    {
+        const float4* b4 = reinterpret_cast<const float4*>(p.bias + (int64_t)expert * p.n_total + chan0);
+#pragma unroll
+        for(int q = 0; q < 4; q++)
+        {
+            const float4 t = b4[q];
+            v[4 * q] += t.x; v[4 * q + 1] += t.y; v[4 * q + 2] += t.z; v[4 * q + 3] += t.w;
+        }
+    }
+}
+
+// gemm0: y = act(gate) * up (silu, gelu) or swiglu(gate, up), with the per-token scale sa and the per-channel
+// scales folded in; stored as bf16 or (fp8 path) as e4m3 with one power-of-two scale per 32 columns.  Every lane of
 // the wave must call it (the fp8 path exchanges the block maximum with lane ^ 32); `store` masks
-// the writes.  single: gate-only weights, y = act(gate) and the up operands are ignored.
+// the writes.  single: gate-only weights, y = act(gate) (swiglu: act(gate, 1)) and the up operands are ignored.
+// col0: first of the lane's 16 output columns = first gate channel; the up channels are n_out + col0 ...
 template <int MODE>
 __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc_gate,
                                       const typename ModeTraits<MODE>::Acc& acc_up, const float (&gs)[16],
                                       const float (&us)[16], float sa, int64_t grow, bool store, int col0, int kg,
-                                      bool single = false)
+                                      bool single = false, int expert = 0)
 {
     float y[16];
-    // p.act is uniform: one scalar branch
-    if(p.act == 0)
+    const bool extras = p.bias != nullptr || p.n_padded > 0 || p.act == 2; // uniform
+    if(extras)
     {
+        // stand-alone GEMMs with an expert bias, padded weight rows or the clamped SwiGLU
+        float g[16], u[16];
 #pragma unroll
         for(int v = 0; v < 16; v++)
-            y[v] = gelu(static_cast<float>(acc_gate[v]) * (sa * gs[v]));
+        {
+            g[v] = static_cast<float>(acc_gate[v]) * (sa * gs[v]);
+            u[v] = single ? 1.0f : static_cast<float>(acc_up[v]) * (sa * us[v]);
+        }
+        bias_and_padding(p, g, expert, col0);
+        if(!single)
+            bias_and_padding(p, u, expert, p.n_out + col0);
+#pragma unroll
+        for(int v = 0; v < 16; v++)
+        {
+            if(p.act == 2)
+                y[v] = swiglu(g[v], u[v], p.swiglu_alpha, p.swiglu_limit);
+            else
+                y[v] = (p.act == 0 ? gelu(g[v]) : silu(g[v])) * u[v];
+        }
     }
     else
     {
+        // p.act is uniform: one scalar branch
+        if(p.act == 0)
+        {
 #pragma unroll
-        for(int v = 0; v < 16; v++)
-            y[v] = silu(static_cast<float>(acc_gate[v]) * (sa * gs[v]));
-    }
-    if(!single)
-    {
+            for(int v = 0; v < 16; v++)
+                y[v] = gelu(static_cast<float>(acc_gate[v]) * (sa * gs[v]));
+        }
+        else
+        {
 #pragma unroll
-        for(int v = 0; v < 16; v++)
-            y[v] *= static_cast<float>(acc_up[v]) * (sa * us[v]);
+            for(int v = 0; v < 16; v++)
+                y[v] = silu(static_cast<float>(acc_gate[v]) * (sa * gs[v]));
+        }
+        if(!single)
+        {
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                y[v] *= static_cast<float>(acc_up[v]) * (sa * us[v]);
+        }
     }
     const bool as_fp8  = MODE == kFp8 && !p.y_bf16;
     const int y_b      = as_fp8 ? 1 : 2;
@@ -364,15 +431,17 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
     }
 }
 
-// gemm1: * per-channel scale, bf16 partial row in sorted-row order (the combine applies the top-k weight)
+// gemm1: * per-channel scale (+ expert bias), bf16 partial row in sorted-row order (the combine applies the top-k weight)
 template <int MODE>
 __device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc,
-                                      const float (&ds)[16], int64_t prow, bool store, int col0)
+                                      const float (&ds)[16], int64_t prow, bool store, int col0, int expert = 0)
 {
     float y[16];
 #pragma unroll
     for(int v = 0; v < 16; v++)
         y[v] = static_cast<float>(acc[v]) * ds[v];
+    if(p.bias != nullptr || p.n_padded > 0) // uniform: stand-alone down GEMM with a bias or padded rows
+        bias_and_padding(p, y, expert, col0);
     uint4 o0, o1;
     o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
     o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
@@ -494,31 +563,31 @@ template <int MODE, bool GEMM0, int NBLK>
 __device__ inline void apply_epilogue_block(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[2],
                                             const float (&sc0)[16], const float (&sc1)[16], const EpilogueRows<NBLK>& rows,
                                             const EpilogueColumns& c, int i, int row0, int nrows, int first_row,
-                                            int row_step, int r32, int kg)
+                                            int row_step, int r32, int kg, int expert)
 {
     const int r = first_row + i * row_step + r32;
     if constexpr(GEMM0)
     {
         const bool st = r < nrows && (p.slot_rows == 0 || rows.real[i]);
         if(c.a_ok)
-            epilogue_gemm0<MODE>(p, acc[0], acc[1], sc0, sc1, rows.sa[i], rows.orow[i], st, c.col_a, kg, !c.paired);
+            epilogue_gemm0<MODE>(p, acc[0], acc[1], sc0, sc1, rows.sa[i], rows.orow[i], st, c.col_a, kg, !c.paired, expert);
         if(!c.paired && c.b_ok) // gate-only tile: the second accumulator holds the next 32 gate columns
-            epilogue_gemm0<MODE>(p, acc[1], acc[1], sc1, sc1, rows.sa[i], rows.orow[i], st, c.col_b, kg, true);
+            epilogue_gemm0<MODE>(p, acc[1], acc[1], sc1, sc1, rows.sa[i], rows.orow[i], st, c.col_b, kg, true, expert);
     }
     else
     {
         const bool in_tile = r < nrows;
         if(c.a_ok)
-            epilogue_gemm1<MODE>(p, acc[0], sc0, row0 + r, in_tile && rows.real[i], c.col_a);
+            epilogue_gemm1<MODE>(p, acc[0], sc0, row0 + r, in_tile && rows.real[i], c.col_a, expert);
         if(c.b_ok)
-            epilogue_gemm1<MODE>(p, acc[1], sc1, row0 + r, in_tile && rows.real[i], c.col_b);
+            epilogue_gemm1<MODE>(p, acc[1], sc1, row0 + r, in_tile && rows.real[i], c.col_b, expert);
     }
 }
 
 template <int MODE, bool GEMM0, int NBLK>
 __device__ inline void apply_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2],
                                       const EpilogueOperands<NBLK>& o, int row0, int nrows, int first_row, int row_step,
-                                      int nblk_live, int r32, int kg)
+                                      int nblk_live, int r32, int kg, int expert)
 {
     // block by block, so that a block's accumulators are dead before the next block's temporaries
     // are needed (the large-tile kernel has no registers to spare)
@@ -528,7 +597,7 @@ __device__ inline void apply_epilogue(const GemmParams& p, typename ModeTraits<M
         if(i >= nblk_live)
             continue;
         apply_epilogue_block<MODE, GEMM0, NBLK>(p, acc[i], o.sc0, o.sc1, o.rows, o.cols, i, row0, nrows, first_row, row_step,
-                                                r32, kg);
+                                                r32, kg, expert);
     }
 }
 
@@ -540,7 +609,7 @@ __device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MOD
     EpilogueOperands<NBLK> o;
     load_epilogue<MODE, GEMM0, NBLK, SKIP_PAD>(p, o, expert, row0, nrows, first_row, row_step, n_base, wblk, r32, kg);
     pin_epilogue(o);
-    apply_epilogue<MODE, GEMM0, NBLK>(p, acc, o, row0, nrows, first_row, row_step, nblk_live, r32, kg);
+    apply_epilogue<MODE, GEMM0, NBLK>(p, acc, o, row0, nrows, first_row, row_step, nblk_live, r32, kg, expert);
 }
 
 } // namespace gemm
