@@ -98,45 +98,57 @@ def run_workload(cfg, steps, warmup, seed=0):
     return res, inp, buf
 
 
-TRAFFIC_FILE = os.path.join(ROOT, "profiles", "moe_gemm0_hbm_traffic.txt")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "moe_gemm_hbm_traffic.txt")
 
 
-def measured_traffic(workload):
-    """HBM bytes per launch of the gate+up GEMM as measured with rocprofv3 counters (a committed
-    summary: lines of `workload fetch_bytes write_bytes`); None when there is no entry."""
+def measured_traffic(workload, gemm):
+    """HBM bytes per launch of the gate+up (gemm 0) or down (gemm 1) GEMM as measured with rocprofv3 counters (a
+    committed summary: lines of `workload gemm0_fetch gemm0_write gemm1_fetch gemm1_write`, bytes); None when there
+    is no entry."""
     try:
         for ln in open(TRAFFIC_FILE):
             f = ln.split()
-            if len(f) >= 3 and f[0] == workload:
-                return float(f[1]) + float(f[2])
-    except OSError:
+            if len(f) >= 5 and f[0] == workload:
+                return float(f[1 + 2 * gemm]) + float(f[2 + 2 * gemm])
+    except (OSError, ValueError):
         pass
     return None
 
 
-def roofline_of(cfg, res):
-    """Roofline entry for the dominant kernel of a workload."""
-    k0, k1 = res["kernel_avg_ms"].get("moe_gemm0_gate_up_silu"), res["kernel_avg_ms"].get("moe_gemm1_down")
+def roofline_of(cfg, res, gemm=0):
+    """Roofline entry of a workload's gate+up GEMM (gemm 0, the dominant kernel: 2/3 of the FLOPs) or down GEMM
+    (gemm 1).  Algorithmic work per launch: gemm0 4*T*K*H*I FLOP, bytes = the active experts' gate/up weights and
+    scales + the token matrix + Y written; gemm1 2*T*K*H*I FLOP, bytes = the active experts' down weights and scales
+    + Y read + the per-slot partial rows written."""
+    key = "moe_gemm0_gate_up_silu" if gemm == 0 else "moe_gemm1_down"
+    kms = res["kernel_avg_ms"].get(key)
+    if not kms:
+        return None
     T, K, H, I = cfg.tokens, cfg.topk, cfg.hidden, cfg.inter
-    traffic = measured_traffic(cfg.name)
-    kname = ("moe_gemm_big_kernel" if res["tile_rows"] > 128 else
-             "moe_gemm_decode_kernel" if res["tile_rows"] == 32 else "moe_gemm_kernel") + " (gemm0: gate+up, SiLU*up)"
+    traffic = measured_traffic(cfg.name, gemm)
+    family = ("moe_gemm_big_kernel" if res["tile_rows"] > 128 else
+              "moe_gemm_decode_kernel" if res["tile_rows"] == 32 and gemm == 0 else "moe_gemm_kernel")
+    kname = family + (" (gemm0: gate+up, SiLU*up)" if gemm == 0 else " (gemm1: down)")
     b = {"bf16": 2, "fp8": 1, "int8": 1}[cfg.dtype]
     y_b = 1 if cfg.dtype == "fp8" else 2
-    byt0 = (res["active_experts"] * 2 * I * H * b + res["active_experts"] * 2 * I * 4 + T * H * b
-            + res["post_pad"] * I * y_b)
-    gbps = byt0 / k0 / 1e6
-    tflops = 4.0 * T * K * H * I / k0 / 1e9  # gate+up GEMM: 2/3 of the FLOPs
+    ae = res["active_experts"]
+    if gemm == 0:
+        flop = 4.0 * T * K * H * I
+        byt = ae * 2 * I * H * b + ae * 2 * I * 4 + T * H * b + res["post_pad"] * I * y_b
+    else:
+        flop = 2.0 * T * K * H * I
+        byt = ae * H * I * b + ae * H * 4 + res["post_pad"] * I * y_b + res["post_pad"] * H * 2
+    gbps = byt / kms / 1e6
+    tflops = flop / kms / 1e9
     # prefill-sized workloads (tens of rows or more per expert) are graded against the MFMA peak, the
     # decode regime against HBM; the other fraction is reported beside it
     if T * K / cfg.experts >= 64:
         return {"kernel": kname, "bound": "mfma", "achieved": tflops, "peak": PEAK_MFMA[cfg.dtype], "unit": "TFLOP/s",
-                "frac": tflops / PEAK_MFMA[cfg.dtype], "avg_launch_ms": k0, "traffic": traffic,
-                "algorithmic_flop": 4.0 * T * K * H * I, "algorithmic_bytes": byt0, "hbm_GBps": gbps,
-                "hbm_frac": gbps / PEAK_HBM}
+                "frac": tflops / PEAK_MFMA[cfg.dtype], "avg_launch_ms": kms, "traffic": traffic,
+                "algorithmic_flop": flop, "algorithmic_bytes": byt, "hbm_GBps": gbps, "hbm_frac": gbps / PEAK_HBM}
     return {"kernel": kname, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM, "unit": "GB/s",
-            "frac": gbps / PEAK_HBM, "avg_launch_ms": k0, "traffic": traffic, "algorithmic_bytes": byt0,
-            "algorithmic_flop": 4.0 * T * K * H * I, "mfma_TFLOPs": tflops, "mfma_frac": tflops / PEAK_MFMA[cfg.dtype]}
+            "frac": gbps / PEAK_HBM, "avg_launch_ms": kms, "traffic": traffic, "algorithmic_bytes": byt,
+            "algorithmic_flop": flop, "mfma_TFLOPs": tflops, "mfma_frac": tflops / PEAK_MFMA[cfg.dtype]}
 
 
 def run_router(cfg, steps, warmup):
@@ -338,6 +350,7 @@ def main():
                 steps = max(5, a.steps // 2)
                 r, i2, b2 = run_workload(c, steps, a.warmup)
                 r["roofline"] = roofline_of(c, r)
+                r["roofline_gemm1"] = roofline_of(c, r, 1)
                 others[name] = r
                 log(f"[bench] {name}: {r['ms_per_step']:.3f} ms/step, {r['tflops']:.1f} TFLOP/s, "
                     f"{r['hbm_GBps']:.0f} GB/s, kernels {r['kernel_avg_ms']}")
@@ -357,7 +370,8 @@ def main():
                    "path": "moe_sorting + gemm0(gate,up,SiLU*up) + gemm1(down) + combine, one stream"},
         "frac_of_mfma_peak": res["frac_mfma_peak"], "tokens_per_s": res["tokens_per_s"],
         "hbm_GBps": res["hbm_GBps"], "kernel_avg_ms": res["kernel_avg_ms"], "gemm0_tflops": res["gemm0_tflops"],
-        "gemm1_tflops": res["gemm1_tflops"], "roofline": roof, "cpu_baseline": cpu, "router": router, "neighbours": neighbours, "workloads": others,
+        "gemm1_tflops": res["gemm1_tflops"], "roofline": roof, "roofline_gemm1": roofline_of(cfg, res, 1),
+        "cpu_baseline": cpu, "router": router, "neighbours": neighbours, "workloads": others,
     }
     print(json.dumps(line), flush=True)
 
