@@ -59,34 +59,47 @@ static_assert(kLdsBytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 
 typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
 
+
 __device__ inline uint32_t lds_offset(const void* p)
 {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const lds_byte_t*)p));
 }
 
-// lane i of the wave copies 16 (4) bytes from base + off (a wave-uniform base, a per-lane 32-bit offset)
-// to LDS byte m0 + 16*i (4*i)
-__device__ inline void dma16(const unsigned char* base_uniform, uint32_t off, uint32_t m0_uniform)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0_uniform), "v"(off), "s"(base_uniform)
-                 : "memory");
-}
-__device__ inline void dma16nt(const unsigned char* base_uniform, uint32_t off, uint32_t m0_uniform)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m0_uniform), "v"(off), "s"(base_uniform)
-                 : "memory");
-}
-__device__ inline void dma4(const unsigned char* base_uniform, uint32_t off, uint32_t m0_uniform)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0_uniform), "v"(off), "s"(base_uniform)
-                 : "memory");
-}
 __device__ inline const unsigned char* uniform_ptr(const unsigned char* p)
 {
     const uint64_t v  = reinterpret_cast<uint64_t>(p);
     const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
     const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
     return reinterpret_cast<const unsigned char*>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// lane i of the wave copies 16 (4) bytes from base + off (a wave-uniform base, a per-lane 32-bit offset)
+// to LDS byte m0 + 16*i (4*i)
+__device__ inline void dma16(const unsigned char* base_uniform, uint32_t off, uint32_t m0_uniform)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0_uniform), "v"(off), "s"(uniform_ptr(base_uniform))
+                 : "memory");
+}
+__device__ inline void dma16nt(const unsigned char* base_uniform, uint32_t off, uint32_t m0_uniform)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m0_uniform), "v"(off), "s"(uniform_ptr(base_uniform))
+                 : "memory");
+}
+__device__ inline void dma4(const unsigned char* base_uniform, uint32_t off, uint32_t m0_uniform)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0_uniform), "v"(off), "s"(uniform_ptr(base_uniform))
+                 : "memory");
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): indices that are constants before any loop pass runs
+template <int N, typename F>
+__device__ __attribute__((always_inline)) inline void static_for(F&& f)
+{
+    if constexpr(N > 0)
+    {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
 }
 
 template <int N>
@@ -261,7 +274,12 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             for(int v = 0; v < 16; v++)
                 acc[i][b][v] = 0;
 
-    // prologue: weight units 0..3, token steps 0 and 1
+    // Software-pipelined K loop (kPipe): the operands of step k+1 are fetched from LDS into registers during step
+    // k, each fragment right behind the last MFMA that reads its register, so that after a barrier the MFMAs start
+    // at once instead of waiting for operand fetches that all eight waves issue at the same moment.  The barrier of
+    // step k then has to guarantee the data of step k+1: every transfer runs one step further ahead.
+    constexpr bool kPipe = !kW8 && !kMx;
+    // prologue: weight units 0..3 (0..4 when pipelined), token steps 0 and 1 (and 2)
     using H0 = std::integral_constant<int, 0>;
     using H1 = std::integral_constant<int, 1>;
     if(w_role)
@@ -272,6 +290,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             issue_w(1, H1{}, std::true_type{});
             issue_w(2, H0{}, std::true_type{});
             issue_w(3, H1{}, std::true_type{});
+            if constexpr(kPipe)
+                issue_w(4, H0{}, std::true_type{});
         }
         else
         {
@@ -279,12 +299,16 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             issue_w(1, H1{}, std::false_type{});
             issue_w(2, H0{}, std::false_type{});
             issue_w(3, H1{}, std::false_type{});
+            if constexpr(kPipe)
+                issue_w(4, H0{}, std::false_type{});
         }
     }
     else
     {
         issue_x(0, x_groups);
         issue_x(1, x_groups);
+        if constexpr(kPipe)
+            issue_x(2, x_groups);
     }
 
     // per-lane LDS read offsets (swizzled chunk positions are per-lane constants)
@@ -295,10 +319,121 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     const int x_off = kXOffset + (wt * 32 + r32) * kStepKB;
 
     // NB: token blocks of this wave; XG: slab groups a token-role wave issues per step (0 in a weight-role wave)
-    auto k_loop = [&](auto nb_tag, auto xg_tag, auto nt_tag) {
+    auto k_loop = [&](auto nb_tag, auto xg_tag, auto nt_tag) __attribute__((always_inline)) {
         constexpr int NB = decltype(nb_tag)::value;
         constexpr int XG = decltype(xg_tag)::value;
         constexpr int NF = NB > 0 ? NB : 1;
+        if constexpr(kPipe)
+        {
+            // operand registers of the step about to run
+            Frag wf[kSteps][2];
+            Frag xf[kSteps][NF];
+            uint32_t xs[kSteps][NF];
+            // weight fragment b of sub-step s of step kk (parity P), token fragment i of sub-step s of step kk
+            auto load_wf = [&](int kk, auto p_tag, int s, int b) __attribute__((always_inline)) {
+                constexpr int P          = decltype(p_tag)::value;
+                constexpr int kh         = P * 4; // first chunk of the step inside the 128-byte weight row
+                const unsigned char* wp  = lds + (((kk & ~1) + w_h) % kWSlots) * kWUnitBytes + w_off + b * 32 * (2 * kStepKB);
+                const int cw_lo          = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_w) * 16 : ((kh + kg) ^ sw_w) * 16;
+                const int cw_hi          = ((kh + 2 + kg) ^ sw_w) * 16;
+                Frag f;
+                f.lo = *reinterpret_cast<const uint4*>(wp + cw_lo);
+                if constexpr(kOpB == 32)
+                    f.hi = *reinterpret_cast<const uint4*>(wp + cw_hi);
+                return f;
+            };
+            auto load_xf = [&](int kk, int s, int i, uint32_t& scale) __attribute__((always_inline)) {
+                const unsigned char* xp = lds + x_off + (kk % kXStages) * kXStageBytes + i * 64 * kStepKB;
+                const int cx_lo         = kOpB == 16 ? ((2 * s + kg) ^ sw_x) * 16 : (kg ^ sw_x) * 16;
+                const int cx_hi         = ((2 + kg) ^ sw_x) * 16;
+                Frag f;
+                f.lo = *reinterpret_cast<const uint4*>(xp + cx_lo);
+                if constexpr(kOpB == 32)
+                    f.hi = *reinterpret_cast<const uint4*>(xp + cx_hi);
+                scale = 127;
+                if constexpr(kMx)
+                    scale = lds[kYsOffset + (kk % kXStages) * kYsStageBytes + kg * kYsRows + wt * 32 + r32 + i * 64];
+                return f;
+            };
+            // own transfers of the data named `need` have landed (the instructions issued after them may be
+            // pending), everyone's are visible after the barrier, and nobody reads the buffers of the step before
+            auto sync = [&](bool counted, auto w_tag, auto x_tag) __attribute__((always_inline)) {
+                if(counted)
+                {
+                    if(w_role)
+                        wait_vmcnt<decltype(w_tag)::value>();
+                    else
+                        wait_vmcnt<decltype(x_tag)::value>();
+                }
+                else
+                    wait_vmcnt<0>();
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // own operand fetches are complete
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            };
+            constexpr int kXI = XG + (kMx ? 1 : 0); // token-role instructions of one step
+            // step 0's data: weight units 0 and 1 (2, 3, 4 may be pending), token step 0 (1 and 2 pending)
+            sync(kt_count >= 6, std::integral_constant<int, 12>{}, std::integral_constant<int, 2 * kXI>{});
+            static_for<kSteps>([&](auto s_tag) __attribute__((always_inline)) {
+                constexpr int s = decltype(s_tag)::value;
+                wf[s][0]        = load_wf(0, H0{}, s, 0);
+                wf[s][1]        = load_wf(0, H0{}, s, 1);
+                static_for<NB>([&](auto i_tag) __attribute__((always_inline)) {
+                    constexpr int i = decltype(i_tag)::value;
+                    xf[s][i]        = load_xf(0, s, i, xs[s][i]);
+                });
+            });
+            auto step = [&](int k, auto par_tag) __attribute__((always_inline)) {
+                constexpr int PAR = decltype(par_tag)::value;
+                using NPAR        = std::integral_constant<int, 1 - PAR>;
+                // The barrier of step k guarantees step k+1: token step k+1 (k+2 may be pending) and the weight pair
+                // of step k+1, that is units up to k+1 for even k (k+2 .. k+4 pending) or up to k+2 for odd k.
+                sync(k + 4 < kt_count, std::integral_constant<int, (PAR ? 8 : 12)>{}, std::integral_constant<int, kXI>{});
+                // the transfers of the step go out behind the MFMAs of the second token block (measured: 1 to 2 %
+                // faster than right after the barrier, where all eight waves queue up at the address unit while the
+                // MFMA pipe has nothing to do; one instruction behind every block is 5 % slower)
+                auto issue_next = [&]() __attribute__((always_inline)) {
+                    if(w_role)
+                        issue_w(k + 5, NPAR{}, nt_tag);
+                    else
+                        issue_x(k + 3, XG);
+                };
+                constexpr int kIssueAfter = 1;
+                if constexpr(NB <= kIssueAfter)
+                    issue_next();
+                static_for<kSteps>([&](auto s_tag) __attribute__((always_inline)) {
+                    constexpr int s = decltype(s_tag)::value;
+                    static_for<NB>([&](auto i_tag) __attribute__((always_inline)) {
+                        constexpr int i = decltype(i_tag)::value;
+                        if constexpr(MODE == kFp8 && GEMM0)
+                        {
+                            acc[i][0] = mfma_fp8_unscaled(wf[s][0], xf[s][i], acc[i][0]);
+                            acc[i][1] = mfma_fp8_unscaled(wf[s][1], xf[s][i], acc[i][1]);
+                        }
+                        else
+                        {
+                            acc[i][0] = mfma<MODE>(wf[s][0], xf[s][i], xs[s][i], acc[i][0]);
+                            acc[i][1] = mfma<MODE>(wf[s][1], xf[s][i], xs[s][i], acc[i][1]);
+                        }
+                        // the fragment's registers are free: fetch its successor (stale data after the last step)
+                        __builtin_amdgcn_sched_barrier(0);
+                        xf[s][i] = load_xf(k + 1, s, i, xs[s][i]);
+                        if constexpr(NB > kIssueAfter && s == 0 && i == kIssueAfter)
+                            issue_next();
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
+                    wf[s][0] = load_wf(k + 1, NPAR{}, s, 0);
+                    wf[s][1] = load_wf(k + 1, NPAR{}, s, 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            };
+            for(int k = 0; k < kt_count; k += 2)
+            {
+                step(k, H0{});
+                step(k + 1, H1{});
+            }
+            return;
+        }
         // one compute step; PAR = k & 1
         auto step = [&](int k, auto par_tag) __attribute__((always_inline)) {
             constexpr int PAR = decltype(par_tag)::value;
