@@ -56,6 +56,14 @@ constexpr int kXOffset      = kWSlots * kWUnitBytes;
 constexpr int kYsOffset     = kXOffset + kXStages * kXStageBytes;
 constexpr int kLdsBytes     = kYsOffset + kXStages * kYsStageBytes;
 static_assert(kLdsBytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
+// Gate+up GEMM (token rows gathered by id): a token stage holds 128 bytes of K per row, two compute steps, so that a
+// token DMA instruction fetches eight whole 128-byte lines instead of sixteen half lines (a compute unit's address
+// path moves 100 GB/s in whole lines and 58 GB/s in halves).  Two such stages and a weight ring of five slots.
+constexpr int kXPairBytes   = kBigXRows * 2 * kStepKB;
+constexpr int kWSlotsPair   = 5;
+constexpr int kXOffsetPair  = kWSlotsPair * kWUnitBytes;
+constexpr int kLdsBytesPair = kXOffsetPair + 2 * kXPairBytes;
+static_assert(kLdsBytesPair <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 
 typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
 
@@ -120,6 +128,14 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     constexpr bool kW8 = MODE == kBf16W8;
     constexpr bool kMx   = MODE == kFp8 && !GEMM0;
     static_assert(MODE == kBf16 || MODE == kFp8 || (MODE == kI8 && GEMM0) || (MODE == kBf16W8 && !GEMM0), "no large-tile kernel for this mode");
+    // Software-pipelined K loop (kPipe): the operands of step k+1 are fetched from LDS into registers during step
+    // k, each fragment right behind the last MFMA that reads its register, so that after a barrier the MFMAs start
+    // at once instead of waiting for operand fetches that all eight waves issue at the same moment.  The barrier of
+    // step k then has to guarantee the data of step k+1: every transfer runs one step further ahead.
+    constexpr bool kPipe  = !kW8 && !kMx;
+    constexpr bool kXPair = kPipe && GEMM0; // 128-byte token stages
+    constexpr int kWS     = kXPair ? kWSlotsPair : kWSlots;
+    constexpr int kXO     = kXPair ? kXOffsetPair : kXOffset;
 
     extern __shared__ __align__(16) unsigned char lds[];
 
@@ -161,7 +177,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     // ids, rows past the tile) read row 0 instead: their MFMA columns are never stored.
     const bool w_role = wave < 4;
     const int q4      = wave & 3;
-    uint32_t doff[8];
+    uint32_t doff[kXPair ? 10 : 8];
     const unsigned char* dbase;
     if(w_role)
     {
@@ -186,30 +202,48 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     }
     else
     {
-        dbase            = uniform_ptr(p.x);
-        const int lrow16 = lane >> 2;
-        const int cchunk = (lane & 3) ^ ((lane >> 4) & 3);
-#pragma unroll
-        for(int j = 0; j < 5; j++)
+        dbase = uniform_ptr(p.x);
+        if constexpr(kXPair)
         {
-            const int lrow = (q4 + 4 * j) * 16 + lrow16;
-            uint32_t src   = lrow < nrows ? row0 + lrow : row0;
-            if(GEMM0 || p.slot_rows > 0)
+            // instruction j of wave 4 + q: rows (q + 4 j) * 8 .. + 7 of the tile, 128 bytes each, chunks swizzled
+            // like the weight rows
+#pragma unroll
+            for(int j = 0; j < 10; j++)
             {
-                int sid = p.tokens;
+                const int lrow = (q4 + 4 * j) * 8 + (lane >> 3);
+                int sid        = p.tokens;
                 if(lrow < nrows)
                     sid = p.sorted_ids[row0 + lrow];
-                const bool ok = (sid & 0xffffff) < p.tokens;
-                src           = !ok ? 0u : GEMM0 ? (uint32_t)(sid & 0xffffff) : (uint32_t)slot_row(sid, p.slot_rows);
+                const uint32_t src = (sid & 0xffffff) < p.tokens ? (uint32_t)(sid & 0xffffff) : 0u;
+                doff[j]            = src * (uint32_t)p.x_row_bytes + ((lane & 7) ^ ((lrow >> 1) & 7)) * 16;
             }
-            doff[j] = src * (uint32_t)p.x_row_bytes + cchunk * 16;
-            if(!GEMM0 && p.y_slab > 0) // slab-major Y: whole slabs; slabs past the tile's rows read its first
-                doff[j] = (uint32_t)(((row0 >> 4) + ((q4 + 4 * j) * 16 < nrows ? q4 + 4 * j : 0)) * p.y_slab) * 1024u +
-                          lrow16 * 64 + cchunk * 16;
         }
-        // scales: K block (q >> 1) of the step, rows (q & 1) * 256 .. + 255 (the rows are padded)
-        doff[5] = (uint32_t)((q4 >> 1) * p.ys_kb_stride + row0 + (q4 & 1) * 256 + lane * 4);
-        doff[6] = doff[7] = 0;
+        else
+        {
+            const int lrow16 = lane >> 2;
+            const int cchunk = (lane & 3) ^ ((lane >> 4) & 3);
+#pragma unroll
+            for(int j = 0; j < 5; j++)
+            {
+                const int lrow = (q4 + 4 * j) * 16 + lrow16;
+                uint32_t src   = lrow < nrows ? row0 + lrow : row0;
+                if(GEMM0 || p.slot_rows > 0)
+                {
+                    int sid = p.tokens;
+                    if(lrow < nrows)
+                        sid = p.sorted_ids[row0 + lrow];
+                    const bool ok = (sid & 0xffffff) < p.tokens;
+                    src           = !ok ? 0u : GEMM0 ? (uint32_t)(sid & 0xffffff) : (uint32_t)slot_row(sid, p.slot_rows);
+                }
+                doff[j] = src * (uint32_t)p.x_row_bytes + cchunk * 16;
+                if(!GEMM0 && p.y_slab > 0) // slab-major Y: whole slabs; slabs past the tile's rows read its first
+                    doff[j] = (uint32_t)(((row0 >> 4) + ((q4 + 4 * j) * 16 < nrows ? q4 + 4 * j : 0)) * p.y_slab) * 1024u +
+                              lrow16 * 64 + cchunk * 16;
+            }
+            // scales: K block (q >> 1) of the step, rows (q & 1) * 256 .. + 255 (the rows are padded)
+            doff[5] = (uint32_t)((q4 >> 1) * p.ys_kb_stride + row0 + (q4 & 1) * 256 + lane * 4);
+            doff[6] = doff[7] = 0;
+        }
     }
     const int64_t ys_step = (kStepKB / 32) * p.ys_kb_stride;
     const int x_step      = (!GEMM0 && p.y_slab > 0) ? 1024 : kStepKB; // bytes between token steps
@@ -229,7 +263,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
         constexpr bool NT = decltype(nt_tag)::value;
         if(u >= n_wunits)
             return;
-        const uint32_t sbase     = lds_base + (u % kWSlots) * kWUnitBytes + q4 * 1024;
+        const uint32_t sbase     = lds_base + (u % kWS) * kWUnitBytes + q4 * 1024;
         const unsigned char* src = dbase + (u >> 1) * (2 * kStepKB);
 #pragma unroll
         for(int j = 0; j < 4; j++)
@@ -261,6 +295,21 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                                                 (q4 >> 1) * kYsRows + (q4 & 1) * 256));
     };
 
+    // 128-byte token stages: pair m = steps 2 m and 2 m + 1 -> stage m & 1; two instructions per 64 rows of the tile
+    auto issue_x_pair = [&](int m, int groups) __attribute__((always_inline)) {
+        if constexpr(kXPair)
+        {
+            if(2 * m >= kt_count)
+                return;
+            const uint32_t sbase     = lds_base + kXO + (m & 1) * kXPairBytes + q4 * 1024;
+            const unsigned char* src = dbase + m * (2 * kStepKB);
+#pragma unroll
+            for(int j = 0; j < 10; j++)
+                if(j < 2 * groups)
+                    dma16(src, doff[j], __builtin_amdgcn_readfirstlane(sbase + j * 4096));
+        }
+    };
+
     // token blocks of this wave (blocks wt, wt + 2, ..) and 64-row slab groups that hold rows of the tile
     const int nb_w     = __builtin_amdgcn_readfirstlane(max(0, min(kMaxNB, (nmb - wt + 1) / 2)));
     const int x_groups = __builtin_amdgcn_readfirstlane(max(1, (nmb + 1) / 2));
@@ -274,12 +323,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             for(int v = 0; v < 16; v++)
                 acc[i][b][v] = 0;
 
-    // Software-pipelined K loop (kPipe): the operands of step k+1 are fetched from LDS into registers during step
-    // k, each fragment right behind the last MFMA that reads its register, so that after a barrier the MFMAs start
-    // at once instead of waiting for operand fetches that all eight waves issue at the same moment.  The barrier of
-    // step k then has to guarantee the data of step k+1: every transfer runs one step further ahead.
-    constexpr bool kPipe = !kW8 && !kMx;
-    // prologue: weight units 0..3 (0..4 when pipelined), token steps 0 and 1 (and 2)
+    // prologue: weight units 0..3 (0..4 when pipelined with six slots), token steps 0 and 1 (and 2; or pairs 0 and 1)
     using H0 = std::integral_constant<int, 0>;
     using H1 = std::integral_constant<int, 1>;
     if(w_role)
@@ -290,7 +334,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             issue_w(1, H1{}, std::true_type{});
             issue_w(2, H0{}, std::true_type{});
             issue_w(3, H1{}, std::true_type{});
-            if constexpr(kPipe)
+            if constexpr(kPipe && !kXPair)
                 issue_w(4, H0{}, std::true_type{});
         }
         else
@@ -299,9 +343,14 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             issue_w(1, H1{}, std::false_type{});
             issue_w(2, H0{}, std::false_type{});
             issue_w(3, H1{}, std::false_type{});
-            if constexpr(kPipe)
+            if constexpr(kPipe && !kXPair)
                 issue_w(4, H0{}, std::false_type{});
         }
+    }
+    else if constexpr(kXPair)
+    {
+        issue_x_pair(0, x_groups);
+        issue_x_pair(1, x_groups);
     }
     else
     {
@@ -333,7 +382,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
             auto load_wf = [&](int kk, auto p_tag, int s, int b) __attribute__((always_inline)) {
                 constexpr int P          = decltype(p_tag)::value;
                 constexpr int kh         = P * 4; // first chunk of the step inside the 128-byte weight row
-                const unsigned char* wp  = lds + (((kk & ~1) + w_h) % kWSlots) * kWUnitBytes + w_off + b * 32 * (2 * kStepKB);
+                const unsigned char* wp  = lds + (((kk & ~1) + w_h) % kWS) * kWUnitBytes + w_off + b * 32 * (2 * kStepKB);
                 const int cw_lo          = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_w) * 16 : ((kh + kg) ^ sw_w) * 16;
                 const int cw_hi          = ((kh + 2 + kg) ^ sw_w) * 16;
                 Frag f;
@@ -343,16 +392,29 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 return f;
             };
             auto load_xf = [&](int kk, int s, int i, uint32_t& scale) __attribute__((always_inline)) {
-                const unsigned char* xp = lds + x_off + (kk % kXStages) * kXStageBytes + i * 64 * kStepKB;
-                const int cx_lo         = kOpB == 16 ? ((2 * s + kg) ^ sw_x) * 16 : (kg ^ sw_x) * 16;
-                const int cx_hi         = ((2 + kg) ^ sw_x) * 16;
                 Frag f;
-                f.lo = *reinterpret_cast<const uint4*>(xp + cx_lo);
-                if constexpr(kOpB == 32)
-                    f.hi = *reinterpret_cast<const uint4*>(xp + cx_hi);
                 scale = 127;
-                if constexpr(kMx)
-                    scale = lds[kYsOffset + (kk % kXStages) * kYsStageBytes + kg * kYsRows + wt * 32 + r32 + i * 64];
+                if constexpr(kXPair)
+                {
+                    const unsigned char* xp = lds + kXO + ((kk >> 1) & 1) * kXPairBytes + (wt * 32 + r32 + i * 64) * (2 * kStepKB);
+                    const int kh            = (kk & 1) * 4;
+                    const int cx_lo         = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_w) * 16 : ((kh + kg) ^ sw_w) * 16;
+                    const int cx_hi         = ((kh + 2 + kg) ^ sw_w) * 16;
+                    f.lo                    = *reinterpret_cast<const uint4*>(xp + cx_lo);
+                    if constexpr(kOpB == 32)
+                        f.hi = *reinterpret_cast<const uint4*>(xp + cx_hi);
+                }
+                else
+                {
+                    const unsigned char* xp = lds + x_off + (kk % kXStages) * kXStageBytes + i * 64 * kStepKB;
+                    const int cx_lo         = kOpB == 16 ? ((2 * s + kg) ^ sw_x) * 16 : (kg ^ sw_x) * 16;
+                    const int cx_hi         = ((2 + kg) ^ sw_x) * 16;
+                    f.lo                    = *reinterpret_cast<const uint4*>(xp + cx_lo);
+                    if constexpr(kOpB == 32)
+                        f.hi = *reinterpret_cast<const uint4*>(xp + cx_hi);
+                    if constexpr(kMx)
+                        scale = lds[kYsOffset + (kk % kXStages) * kYsStageBytes + kg * kYsRows + wt * 32 + r32 + i * 64];
+                }
                 return f;
             };
             // own transfers of the data named `need` have landed (the instructions issued after them may be
@@ -372,8 +434,12 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 asm volatile("" ::: "memory");
             };
             constexpr int kXI = XG + (kMx ? 1 : 0); // token-role instructions of one step
-            // step 0's data: weight units 0 and 1 (2, 3, 4 may be pending), token step 0 (1 and 2 pending)
-            sync(kt_count >= 6, std::integral_constant<int, 12>{}, std::integral_constant<int, 2 * kXI>{});
+            // step 0's data: weight units 0 and 1 (2, 3, 4 may be pending), token step 0 (1 and 2 pending); with
+            // 128-byte token stages weight units 2 and 3 and token pair 1 may be pending
+            if constexpr(kXPair)
+                sync(kt_count >= 6, std::integral_constant<int, 8>{}, std::integral_constant<int, 2 * XG>{});
+            else
+                sync(kt_count >= 6, std::integral_constant<int, 12>{}, std::integral_constant<int, 2 * kXI>{});
             static_for<kSteps>([&](auto s_tag) __attribute__((always_inline)) {
                 constexpr int s = decltype(s_tag)::value;
                 wf[s][0]        = load_wf(0, H0{}, s, 0);
@@ -388,12 +454,35 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 using NPAR        = std::integral_constant<int, 1 - PAR>;
                 // The barrier of step k guarantees step k+1: token step k+1 (k+2 may be pending) and the weight pair
                 // of step k+1, that is units up to k+1 for even k (k+2 .. k+4 pending) or up to k+2 for odd k.
-                sync(k + 4 < kt_count, std::integral_constant<int, (PAR ? 8 : 12)>{}, std::integral_constant<int, kXI>{});
+                // 128-byte token stages: a weight unit less is in flight (unit k+3 may be pending at odd k), and the
+                // token pair of steps k+1 and k+2 is due at odd k, where it is the wave's only transfer.
+                // Steps 2 m and 2 m + 1 read the same weight pair and the same token stage, so only the barrier of
+                // the odd step has anything to guarantee, and what the even step overwrites (the slot of weight unit
+                // k - 1) was last read before the barrier of step k - 1: the even step has no barrier.
+                // Measured: without it the bf16 and int8 GEMMs (two MFMA sub-steps per step) run 2 % faster, the fp8
+                // GEMM (one) 5 % slower, so that one keeps it.
+                if constexpr(kXPair)
+                {
+                    if constexpr(PAR == 1 || kSteps == 1)
+                        sync(k + 4 < kt_count, std::integral_constant<int, (PAR ? 4 : 8)>{},
+                             std::integral_constant<int, (PAR ? 0 : 2 * XG)>{});
+                }
+                else
+                    sync(k + 4 < kt_count, std::integral_constant<int, (PAR ? 8 : 12)>{}, std::integral_constant<int, kXI>{});
                 // the transfers of the step go out behind the MFMAs of the second token block (measured: 1 to 2 %
                 // faster than right after the barrier, where all eight waves queue up at the address unit while the
                 // MFMA pipe has nothing to do; one instruction behind every block is 5 % slower)
                 auto issue_next = [&]() __attribute__((always_inline)) {
-                    if(w_role)
+                    if constexpr(kXPair)
+                    {
+                        // slot (k + 4) % 5 held unit k - 1, stage ((k + 3) / 2) & 1 held the pair of steps k - 1 and
+                        // k - 2: both were last read during step k - 1, into registers, before this step's barrier
+                        if(w_role)
+                            issue_w(k + 4, par_tag, nt_tag);
+                        else if constexpr(PAR == 1)
+                            issue_x_pair((k + 3) >> 1, XG);
+                    }
+                    else if(w_role)
                         issue_w(k + 5, NPAR{}, nt_tag);
                     else
                         issue_x(k + 3, XG);
@@ -580,7 +669,7 @@ template <int MODE, bool GEMM0>
 int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
 {
     constexpr bool kMx  = MODE == kFp8 && !GEMM0;
-    const size_t lds    = kMx ? kLdsBytes : kYsOffset;
+    const size_t lds    = (GEMM0 && MODE != kBf16W8) ? kLdsBytesPair : kMx ? kLdsBytes : kYsOffset;
     // the dynamic LDS limit is an attribute of the function on one device: set once per device
     static bool attr_ok[64] = {};
     int dev = 0;
