@@ -38,8 +38,9 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_workload(cfg, steps, warmup, seed=0):
-    """Times `steps` passes of the path.  The dominant kernel's duration comes from HIP events the
+def run_workload(cfg, steps, warmup, seed=0, fused_quant=0):
+    """Times `steps` passes of the path (fused_quant 2: the int8 path re-quantises the intermediate activations
+    per row and runs the down GEMM on int8 MFMAs).  The dominant kernel's duration comes from HIP events the
     library records on the launch stream inside the timed region, the other kernels' from an untimed
     pass just before it."""
     import torch
@@ -50,7 +51,7 @@ def run_workload(cfg, steps, warmup, seed=0):
 
     dev = torch.device("cuda:0")
     inp = mi.make_inputs_torch(cfg, dev, seed)
-    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit)
+    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit, fused_quant=fused_quant)
     buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, dev)
     args = ta.make_args(traits, buf, inp["a"], inp["g"], inp["d"], inp["topk_ids"], inp["topk_weight"],
                         a_scale=inp["a_scale"], g_scale=inp["g_scale"], d_scale=inp["d_scale"])

@@ -142,7 +142,13 @@ typedef struct mi355_fused_moe_traits
     int32_t block_m; /* rows per sorted tile = unit_size of the sort: 16, 32, 64 or 128 */
     int32_t activation;  /* 0 = gelu (erf form, ck_tile::element_wise::Gelu), 1 = silu */
     int32_t gate_only;   /* 0 = gate and up (g [e, 2*inter, hidden]), 1 = gate only (g [e, inter, hidden], y = act(gate)) */
-    int32_t fused_quant; /* 0 = none; quantised dtypes always take a_scale/g_scale/d_scale */
+    int32_t fused_quant; /* 0 = none (quantised dtypes always take a_scale/g_scale/d_scale; the int8 path keeps the
+                            intermediate activations in bf16).  INT8 only: 2 = dynamic-quant, the intermediate
+                            activations are re-quantised to int8 per row between the GEMMs and the down GEMM runs on
+                            int8 MFMAs; 1 = smooth-dynamic-quant, the same after a multiplication by
+                            y_smooth_scale[expert], and the activations arrive as MoeSmoothquant leaves them: one int8
+                            row per (slot, token), a [topk, tokens, stride_token], a_scale [topk, tokens]
+                            (UseSmoothQuant of fused_moegemm_traits.hpp:19-35; layouts moe_sorting_kernel.hpp:82-83) */
     int32_t local_expert_masking; /* 1 = apply local_expert_mask_ptr in the sort */
 } mi355_fused_moe_traits;
 
@@ -151,13 +157,13 @@ typedef struct mi355_fused_moe_traits
  * fused_moegemm_traits.hpp:10-17); mi355_moe_permute_weights converts pre-shuffled checkpoints. */
 typedef struct mi355_fused_moegemm_args
 {
-    const void* a_ptr;              /* [tokens, stride_token] activations */
-    const void* a_scale_ptr;        /* [tokens] fp32 per-token scale (quantised dtypes) or NULL */
+    const void* a_ptr;              /* [tokens, stride_token] activations ([topk, tokens, stride_token] with fused_quant 1) */
+    const void* a_scale_ptr;        /* [tokens] fp32 per-token scale (quantised dtypes; [topk, tokens] with fused_quant 1) or NULL */
     const void* g_ptr;              /* [experts, 2*inter, hidden] gate rows then up rows; gate_only: [experts, inter, hidden] */
     const void* d_ptr;              /* [experts, hidden, inter] */
     const void* g_scale_ptr;        /* [experts, 2*inter] ([experts, inter] when gate_only) fp32 or NULL */
     const void* d_scale_ptr;        /* [experts, hidden] fp32 or NULL */
-    const void* y_smooth_scale_ptr; /* [experts, inter]; accepted, must be NULL */
+    const void* y_smooth_scale_ptr; /* [experts, inter] fp32, 16-byte aligned: with fused_quant 1 and only then, else NULL */
     void* o_ptr;                    /* [tokens, stride_token] output, written (not accumulated) */
     const void* sorted_token_ids_ptr;  /* as written by mi355_moe_sorting */
     const void* sorted_weight_ptr;

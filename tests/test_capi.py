@@ -133,6 +133,13 @@ def test_host_only_entry_points():
     for act, gate_only, ok in ((0, 0, 1), (1, 1, 1), (0, 1, 1), (2, 0, 0), (1, 2, 0)):
         t = _lib.FusedMoeTraits(0, 0, 0, 3, 3, 3, 3, 32, act, gate_only, 0, 0)
         assert lib.mi355_fused_moe_supported(C.byref(t)) == ok
+    # fused_quant 1 / 2 (re-quantised intermediate activations) exist for int8 only and need a larger workspace
+    for prec, fq, ok in ((2, 1, 1), (2, 2, 1), (2, 3, 0), (0, 2, 0), (1, 1, 0)):
+        t = _lib.FusedMoeTraits(prec, prec, 0, 3, 3, 3, 3, 32, 1, 0, fq, 0)
+        assert lib.mi355_fused_moe_supported(C.byref(t)) == ok
+    w0, w2 = (lib.mi355_fused_moe_workspace_size(C.byref(_lib.FusedMoeTraits(2, 2, 0, 3, 3, 3, 3, 32, 1, 0, fq, 0)),
+                                                 256, 128, 8, 4096, 1536) for fq in (0, 2))
+    assert w2 >= w0 + (256 * 8) * 1536
     # rows per GEMM workgroup: decode tiles, small tiles, 320-row tiles (sort unit a multiple of 16)
     rows = lambda prec, unit, *shape: lib.mi355_fused_moe_tile_rows(
         C.byref(_lib.FusedMoeTraits(prec, prec, 0, 3, 3, 3, 3, unit, 1, 0, 0, 0)), *shape)

@@ -26,7 +26,7 @@ using namespace gemm;
 namespace {
 
 // ---------------------------------------------------------------------------------------------
-// GEMM0 : MODE in {kBf16, kFp8, kI8};  GEMM1 : MODE in {kBf16, kFp8, kBf16W8}
+// GEMM0 : MODE in {kBf16, kFp8, kI8};  GEMM1 : MODE in {kBf16, kFp8, kBf16W8, kI8}
 template <int MODE, bool GEMM0, int MBLK>
 __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
 {
@@ -78,11 +78,11 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
         const int r = xrow + kXRowsPerPass * j;
         if constexpr(GEMM0)
         {
-            int tok = p.tokens;
+            int sid = p.tokens;
             if(r < nrows)
-                tok = p.sorted_ids[row0 + r] & 0xffffff;
-            xvalid[j] = tok < p.tokens;
-            xptr[j]   = p.x + (int64_t)(xvalid[j] ? tok : 0) * p.x_row_bytes + xchunk * 16;
+                sid = p.sorted_ids[row0 + r];
+            xvalid[j] = (sid & 0xffffff) < p.tokens;
+            xptr[j]   = p.x + (int64_t)(xvalid[j] ? token_row(p, sid) : 0u) * p.x_row_bytes + xchunk * 16;
         }
         else
         {
@@ -433,21 +433,31 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
 
 // 32-row blocks per M tile, from the expected rows per expert; big_tile_rows()/32 selects the
 // large-tile kernel
+// bytes per element of the intermediate activations the down GEMM reads: e4m3 on the fp8 path, int8 when the
+// int8 path re-quantises them (fused_quant 1 / 2), bf16 otherwise
+inline int y_bytes(const mi355_fused_moe_traits& t)
+{
+    return (t.prec_i == MI355_MOE_FP8 || (t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0)) ? 1 : 2;
+}
+
+// 32-row blocks per M tile, from the expected rows per expert; big_tile_rows()/32 selects the
+// large-tile kernel
 inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
 {
     const int64_t avg = tokens * topk / std::max(experts, 1);
     const int eb  = t.prec_i == MI355_MOE_BF16 ? 2 : 1;
-    const int y_b = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
+    const int y_b = y_bytes(t);
     // the large-tile kernel addresses each operand as a base plus a 32-bit byte offset
     const int64_t lim     = (int64_t)1 << 32;
     const int64_t max_pad = topk * tokens + (int64_t)experts * t.block_m - topk;
-    const bool fits = (int64_t)2 * inter * hidden * eb < lim && max_pad * inter * y_b < lim && tokens * hidden * eb < lim;
+    const int64_t x_rows  = t.fused_quant == 1 ? tokens * topk : tokens; // smooth-quant: a row per (slot, token)
+    const bool fits = (int64_t)2 * inter * hidden * eb < lim && max_pad * inter * y_b < lim && x_rows * hidden * eb < lim;
     // Measured crossovers (fp8, 256 experts; bf16, 8 experts): the decode kernel wins up to about 24 rows per
     // expert, the large-tile kernel from about 28 on - it streams every weight tile once whatever the row
     // count and fetches only the token slabs a tile has - provided its tiles fill the chip.
     const int64_t big_tiles = (int64_t)experts * std::max<int64_t>(1, ceil_div<int64_t>(avg, big_tile_rows())) * ceil_div(inter, 128);
     // (its tiles start on whole 16-row slabs of Y: the sort unit must be a multiple of 16)
-    const bool big_ok = t.block_m % 16 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b);
+    const bool big_ok = t.block_m % 16 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b, y_b == 1);
     if(big_ok && (avg >= 160 || (avg >= 28 && big_tiles >= device_info().num_cu)))
         return big_tile_rows() / 32;
     if(avg <= 32)
@@ -483,22 +493,26 @@ int launch_gemm(int mblk, const GemmParams& p, int max_tiles, hipStream_t stream
 
 // One grouped GEMM over the tile list: sets the column-tile count for the kernel family that runs this
 // tile size and launches it.  use_decode: the caller found the decode kernel applicable (one 32-row block per
-// tile, 32-bit offsets suffice).  The down GEMM of the int8 path multiplies bf16 Y by int8 weights.
-int launch_grouped_gemm(int prec, bool gemm0, int mblk, bool use_decode, GemmParams& p, int max_tiles, hipStream_t stream)
+// tile, 32-bit offsets suffice).  The down GEMM of the int8 path multiplies bf16 Y by int8 weights, or, with
+// y_i8, int8 Y (scaled per row) by int8 weights on the i8 MFMAs.
+int launch_grouped_gemm(int prec, bool gemm0, int mblk, bool use_decode, GemmParams& p, int max_tiles, hipStream_t stream,
+                        bool y_i8 = false)
 {
     // output columns per tile: the tile's weight rows, halved where gate and up rows share them
     const int pair = gemm0 && !p.gate_only ? 2 : 1;
     p.max_tiles    = max_tiles;
     p.n_ntiles     = ceil_div(p.n_out, (use_decode ? decode_tile_cols(false) : 256) / pair);
     if(use_decode)
-        return launch_gemm_decode(prec, gemm0, p, max_tiles, stream);
+        return launch_gemm_decode(prec, gemm0, p, max_tiles, stream, y_i8);
     if(mblk > 4)
-        return launch_gemm_big(prec, gemm0, p, max_tiles, stream);
+        return launch_gemm_big(prec, gemm0, p, max_tiles, stream, y_i8);
     if(prec == MI355_MOE_BF16)
         return gemm0 ? launch_gemm<kBf16, true>(mblk, p, max_tiles, stream) : launch_gemm<kBf16, false>(mblk, p, max_tiles, stream);
     if(prec == MI355_MOE_FP8)
         return gemm0 ? launch_gemm<kFp8, true>(mblk, p, max_tiles, stream) : launch_gemm<kFp8, false>(mblk, p, max_tiles, stream);
-    return gemm0 ? launch_gemm<kI8, true>(mblk, p, max_tiles, stream) : launch_gemm<kBf16W8, false>(mblk, p, max_tiles, stream);
+    if(gemm0)
+        return launch_gemm<kI8, true>(mblk, p, max_tiles, stream);
+    return y_i8 ? launch_gemm<kI8, false>(mblk, p, max_tiles, stream) : launch_gemm<kBf16W8, false>(mblk, p, max_tiles, stream);
 }
 
 // the narrow decode tiles re-read the input rows once per 64 output columns: for the down GEMM they pay off
@@ -523,8 +537,10 @@ int check_traits(const mi355_fused_moe_traits& t)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: activation=%d (0 = gelu, 1 = silu)", t.activation);
     if(t.gate_only != 0 && t.gate_only != 1)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: gate_only=%d (0 or 1)", t.gate_only);
-    if(t.fused_quant != 0)
-        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: fused_quant=%d is not implemented", t.fused_quant);
+    if(t.fused_quant < 0 || t.fused_quant > 2 || (t.fused_quant != 0 && t.prec_i != MI355_MOE_INT8))
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: fused_quant=%d with precision %d (1 = smooth-dynamic-quant and "
+                                             "2 = dynamic-quant of the intermediate activations exist for int8)",
+                    t.fused_quant, t.prec_i);
     if(t.block_m < 1 || t.block_m > 1024)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: block_m=%d", t.block_m);
     return MI355_MOE_OK;
@@ -548,13 +564,18 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
     const int mblk   = pick_mblk(t, tokens, topk, experts, hidden, inter);
     w.max_pad        = (int64_t)topk * tokens + (int64_t)experts * t.block_m - topk;
     w.max_tiles      = (int32_t)(experts + w.max_pad / (mblk * 32) + 1);
-    const int y_b    = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
+    // gemm0 writes e4m3 on the fp8 path and bf16 otherwise; with fused_quant the int8 path re-quantises that bf16
+    // Y into a second buffer the down GEMM reads
+    const bool requant = t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0;
+    const int y_b      = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
     w.sort_off       = bump(sorting_workspace_bytes(tokens, experts, topk));
     w.map_off        = bump(sizeof(int) * (kMapHdr + (size_t)kMapEnt * w.max_tiles));
     w.inv_off        = bump(sizeof(int) * (size_t)tokens * topk);
     w.y_off          = bump((size_t)round_up<int64_t>(w.max_pad, 16) * inter * y_b); // whole 16-row slabs
     w.ys_kb_stride   = round_up<int64_t>(w.max_pad, 256) + 512;
     w.ys_off         = bump(t.prec_i == MI355_MOE_FP8 ? (size_t)w.ys_kb_stride * (inter / 32) : 0);
+    w.yq_off         = bump(requant ? (size_t)round_up<int64_t>(w.max_pad, 16) * inter : 0);
+    w.yrs_off        = bump(requant ? (size_t)w.max_pad * sizeof(float) : 0);
     w.p_off          = bump((size_t)w.max_pad * hidden * 2);
     return w;
 }
@@ -601,8 +622,11 @@ int validate_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_mo
     if(!a.a_ptr || !a.g_ptr || !a.d_ptr || !a.o_ptr || !a.sorted_token_ids_ptr || !a.sorted_weight_ptr ||
        !a.sorted_expert_ids_ptr || !a.num_sorted_tiles_ptr)
         return fail(MI355_MOE_E_INVALID, "fused_moegemm: null tensor pointer");
-    if(a.y_smooth_scale_ptr != nullptr)
-        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: y_smooth_scale is not implemented");
+    if((t.fused_quant == 1) != (a.y_smooth_scale_ptr != nullptr))
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: y_smooth_scale goes with fused_quant 1 and only with it "
+                                         "(fused_quant=%d)", t.fused_quant);
+    if(t.fused_quant == 1 && (reinterpret_cast<uintptr_t>(a.y_smooth_scale_ptr) % 16 != 0 || I % 8 != 0))
+        return fail(MI355_MOE_E_INVALID, "fused_moegemm: y_smooth_scale must be 16-byte aligned");
     const bool quant = t.prec_i != MI355_MOE_BF16;
     if(quant && (!a.a_scale_ptr || !a.g_scale_ptr || !a.d_scale_ptr))
         return fail(MI355_MOE_E_INVALID, "fused_moegemm: quantised dtypes need a_scale, g_scale and d_scale");
@@ -616,7 +640,8 @@ int validate_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_mo
         if(reinterpret_cast<uintptr_t>(ptr) % 16 != 0)
             return fail(MI355_MOE_E_INVALID, "fused_moegemm: a, g, d and o must be 16-byte aligned");
     const int mblk = pick_mblk(t, T, K, E, H, I);
-    if(mblk > 4 && (int64_t)T * a.stride_token * eb >= ((int64_t)1 << 32))
+    // (smooth-quant activations hold a row per (slot, token))
+    if(mblk > 4 && (int64_t)T * (t.fused_quant == 1 ? K : 1) * a.stride_token * eb >= ((int64_t)1 << 32))
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: a token buffer of 4 GiB or more (stride_token=%d) is not "
                                              "supported at this problem size", a.stride_token);
     return MI355_MOE_OK;
@@ -663,7 +688,9 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.ys_kb_stride = ws.ys_kb_stride;
 
     // ---- gemm0: gate+up, SiLU*up
-    const int y_b     = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
+    const bool requant = t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0;
+    const int y_b      = t.prec_i == MI355_MOE_FP8 ? 1 : 2; // bytes per element of what gemm0 writes
+    p.x_slot_major     = t.fused_quant == 1 ? 1 : 0;
     p.x               = static_cast<const unsigned char*>(a.a_ptr);
     p.x_row_bytes     = (int64_t)a.stride_token * eb;
     p.x_scale         = quant ? static_cast<const float*>(a.a_scale_ptr) : nullptr;
@@ -681,18 +708,32 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.n_out           = I;
     p.n_total         = g_rows;
     // decode-sized problems (one 32-row block per tile) have their own kernel
-    const bool decode = mblk == 1 && decode_supported((int64_t)T * a.stride_token * eb, ws.max_pad * (int64_t)I * y_b,
-                                                      (int64_t)2 * I * H * eb);
-    // the two large-tile GEMMs hand Y over in the slab-major layout
-    p.y_slab = (mblk > 4 && ((int64_t)I * y_b) % 64 == 0) ? (int)((int64_t)I * y_b / 64) : 0;
-    rc       = launch_grouped_gemm(t.prec_i, true, mblk, decode, p, ws.max_tiles, stream);
+    const bool decode = mblk == 1 && decode_supported((int64_t)T * (p.x_slot_major ? K : 1) * a.stride_token * eb,
+                                                      ws.max_pad * (int64_t)I * y_b, (int64_t)2 * I * H * eb);
+    // the two large-tile GEMMs hand Y over in the slab-major layout (the re-quantisation pass writes it when there
+    // is one; gemm0 then stores plain rows)
+    const int yq_b   = requant ? 1 : y_b; // bytes per element of what the down GEMM reads
+    const int y_slab = (mblk > 4 && ((int64_t)I * yq_b) % 64 == 0) ? (int)((int64_t)I * yq_b / 64) : 0;
+    p.y_slab         = requant ? 0 : y_slab;
+    rc               = launch_grouped_gemm(t.prec_i, true, mblk, decode, p, ws.max_tiles, stream);
     if(rc != MI355_MOE_OK)
         return rc;
+    p.x_slot_major = 0;
+    if(requant)
+    {
+        rc = launch_requant_y(wsb + ws.y_off, I, static_cast<const float*>(a.y_smooth_scale_ptr), p.sorted_ids,
+                              static_cast<const int*>(a.sorted_expert_ids_ptr),
+                              static_cast<const int*>(a.num_sorted_tiles_ptr), t.block_m, T, y_slab, ws.max_pad,
+                              wsb + ws.yq_off, reinterpret_cast<float*>(wsb + ws.yrs_off), stream);
+        if(rc != MI355_MOE_OK)
+            return rc;
+    }
 
     // ---- gemm1: down, * top-k weight, bf16 partial per (token, slot)
-    p.x              = wsb + ws.y_off;
-    p.x_row_bytes    = (int64_t)I * y_b;
-    p.x_scale        = nullptr;
+    p.y_slab         = y_slab;
+    p.x              = requant ? wsb + ws.yq_off : wsb + ws.y_off;
+    p.x_row_bytes    = (int64_t)I * yq_b;
+    p.x_scale        = requant ? reinterpret_cast<const float*>(wsb + ws.yrs_off) : nullptr;
     p.gate_only      = 0;
     p.w              = static_cast<const unsigned char*>(a.d_ptr);
     p.w_row_bytes    = (int64_t)I * eb;
@@ -700,12 +741,12 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.w_scale        = quant ? static_cast<const float*>(a.d_scale_ptr) : nullptr;
     p.out            = wsb + ws.p_off;
     p.out_row_bytes  = (int64_t)H * 2;
-    p.k_bytes_x      = I * y_b;
+    p.k_bytes_x      = I * yq_b;
     p.k_bytes_w      = I * eb;
     p.n_out          = H;
     p.n_total        = H;
     rc = launch_grouped_gemm(t.prec_i, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p, ws.max_tiles,
-                             stream);
+                             stream, requant);
     if(rc != MI355_MOE_OK)
         return rc;
 

@@ -14,6 +14,8 @@ struct WorkspaceLayout
     size_t y_off;      // intermediate activations Y [max_pad, inter] (bf16 or e4m3)
     size_t ys_off;     // e8m0 block scales of Y [inter / 32][ys_kb_stride] (fp8 path only)
     int64_t ys_kb_stride;
+    size_t yq_off;     // int8 copy of Y [max_pad, inter] and ...
+    size_t yrs_off;    // ... its fp32 per-row scales [max_pad] (int8 path with fused_quant 1 / 2 only)
     size_t p_off;      // partial outputs per sorted row [max_pad, hidden] bf16
     size_t total;
     int64_t max_pad;
@@ -49,13 +51,15 @@ struct GemmParams;
 }
 // large-tile kernel (moe_gemm_big.hip)
 int big_tile_rows();
-bool big_tile_supported(int prec, int k_bytes0, int k_bytes1);
-int launch_gemm_big(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream);
+// (y_i8: the down GEMM of the int8 path reads int8 Y with per-row scales instead of bf16 Y)
+bool big_tile_supported(int prec, int k_bytes0, int k_bytes1, bool y_i8 = false);
+int launch_gemm_big(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream, bool y_i8 = false);
 
 // decode kernel (moe_gemm_decode.hip): tiles of one 32-row block x decode_tile_cols() output columns
 int decode_tile_cols(bool gemm0);
 bool decode_supported(int64_t x_bytes, int64_t y_bytes, int64_t w_expert_bytes);
-int launch_gemm_decode(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream);
+int launch_gemm_decode(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream,
+                       bool y_i8 = false);
 
 size_t moe_flatmm_workspace_bytes(int kind, const mi355_moe_flatmm_args& a);
 int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, size_t ws_bytes, hipStream_t stream);
@@ -64,6 +68,12 @@ int launch_permute_weights(const void* src, void* dst, int32_t experts, int32_t 
                            int32_t nw, int32_t kw, int32_t kv, int32_t inverse, hipStream_t stream);
 
 int launch_moe_smoothquant(const mi355_moe_smoothquant_args& a, int32_t q_dtype, hipStream_t stream);
+
+// int8 re-quantisation of the sorted rows of Y between the two GEMMs (smooth: [experts, inter] or null;
+// total[0] = rows of the sorted prefix; segs > 0: slab-major output)
+int launch_requant_y(const void* y, int32_t inter, const float* smooth, const int* sorted_ids, const int* sorted_expert_ids,
+                     const int* total, int32_t unit, int32_t tokens, int32_t segs, int64_t max_rows, void* yq, float* yscale,
+                     hipStream_t stream);
 
 int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype,
                          void* q, void* scale, hipStream_t stream);

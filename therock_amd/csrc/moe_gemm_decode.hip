@@ -73,11 +73,11 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
         const int r = xrow + kXRowsPerPass * j;
         if constexpr(GEMM0)
         {
-            int tok = p.tokens;
+            int sid = p.tokens;
             if(r < nrows)
-                tok = p.sorted_ids[row0 + r] & 0xffffff;
-            xvalid[j] = tok < p.tokens;
-            xoff[j]   = (uint32_t)(xvalid[j] ? tok : 0) * (uint32_t)p.x_row_bytes + xchunk * 16;
+                sid = p.sorted_ids[row0 + r];
+            xvalid[j] = (sid & 0xffffff) < p.tokens;
+            xoff[j]   = (xvalid[j] ? token_row(p, sid) : 0u) * (uint32_t)p.x_row_bytes + xchunk * 16;
         }
         else
         {
@@ -278,8 +278,10 @@ bool decode_supported(int64_t x_bytes, int64_t y_bytes, int64_t w_expert_bytes)
     return x_bytes < lim && y_bytes < lim && w_expert_bytes < lim;
 }
 
-int launch_gemm_decode(int prec, bool gemm0, const GemmParams& p, int max_tiles, hipStream_t stream)
+int launch_gemm_decode(int prec, bool gemm0, const GemmParams& p, int max_tiles, hipStream_t stream, bool y_i8)
 {
+    if(prec == MI355_MOE_INT8 && !gemm0 && y_i8)
+        return launch_decode_t<kI8, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_BF16)
         return gemm0 ? launch_decode_t<kBf16, true>(p, max_tiles, stream) : launch_decode_t<kBf16, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_FP8)

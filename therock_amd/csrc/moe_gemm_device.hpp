@@ -18,7 +18,7 @@ enum Mode
 {
     kBf16   = 0, // x bf16, w bf16, bf16 MFMA
     kFp8    = 1, // x e4m3, w e4m3, block-scaled f8f6f4 MFMA
-    kI8     = 2, // x int8, w int8, i8 MFMA (gemm0 only)
+    kI8     = 2, // x int8, w int8, i8 MFMA (gemm1: int8 Y with a per-row scale, the fused_quant variants)
     kBf16W8 = 3  // x bf16, w int8 converted to bf16 after the LDS read (gemm1 of the int8 path)
 };
 
@@ -70,7 +70,18 @@ struct GemmParams
     int n_padded;
     float swiglu_alpha;
     float swiglu_limit;
+    // gemm0 of the smooth-quant path (fused_quant 1): the activations are one quantised row per (slot, token),
+    // x [topk, tokens, .] with scales [topk, tokens] (ck_tile's MoeSmoothquant output, moe_sorting_kernel.hpp:82-83);
+    // x_slot_major = 1 selects that addressing, 0 the usual row per token
+    int x_slot_major;
 };
+
+// row of the gate+up GEMM's activations (and index of its per-row scale) a sorted id refers to
+__device__ inline uint32_t token_row(const GemmParams& p, int sid)
+{
+    const uint32_t tok = static_cast<uint32_t>(sid) & 0xffffffu;
+    return p.x_slot_major ? (static_cast<uint32_t>(sid) >> 24) * static_cast<uint32_t>(p.tokens) + tok : tok;
+}
 
 // byte offset of K byte kb of row `row` in the slab-major Y layout
 __device__ inline int64_t y_slab_offset(int64_t row, int kb, int segs)
@@ -432,14 +443,15 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
 }
 
 // gemm1: * per-channel scale (+ expert bias), bf16 partial row in sorted-row order (the combine applies the top-k weight)
+// (sa: per-row scale of a quantised Y, 1 otherwise)
 template <int MODE>
 __device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc,
-                                      const float (&ds)[16], int64_t prow, bool store, int col0, int expert = 0)
+                                      const float (&ds)[16], float sa, int64_t prow, bool store, int col0, int expert = 0)
 {
     float y[16];
 #pragma unroll
     for(int v = 0; v < 16; v++)
-        y[v] = static_cast<float>(acc[v]) * ds[v];
+        y[v] = static_cast<float>(acc[v]) * (sa * ds[v]);
     if(p.bias != nullptr || p.n_padded > 0) // uniform: stand-alone down GEMM with a bias or padded rows
         bias_and_padding(p, y, expert, col0);
     uint4 o0, o1;
@@ -495,7 +507,7 @@ __device__ inline EpilogueColumns epilogue_columns(const GemmParams& p, int n_ba
     return c;
 }
 
-template <bool GEMM0, int NBLK, bool SKIP_PAD>
+template <int MODE, bool GEMM0, int NBLK, bool SKIP_PAD>
 __device__ inline void load_epilogue_rows(const GemmParams& p, EpilogueRows<NBLK>& o, int row0, int nrows, int first_row,
                                           int row_step, int r32)
 {
@@ -514,10 +526,16 @@ __device__ inline void load_epilogue_rows(const GemmParams& p, EpilogueRows<NBLK
             if constexpr(GEMM0)
             {
                 if(p.x_scale != nullptr)
-                    o.sa[i] = o.real[i] ? p.x_scale[tok] : 0.0f;
+                    o.sa[i] = o.real[i] ? p.x_scale[token_row(p, sid)] : 0.0f;
                 if(p.slot_rows > 0)
                     o.orow[i] = o.real[i] ? (int)slot_row(sid, p.slot_rows) : 0;
             }
+        }
+        if constexpr(!GEMM0 && MODE == kI8)
+        {
+            // per-row scale of the int8 intermediate activations, in sorted-row order like Y itself
+            const int r = min(first_row + i * row_step + r32, nrows - 1);
+            o.sa[i]     = p.x_scale[row0 + r];
         }
     }
 }
@@ -543,7 +561,7 @@ __device__ inline void load_epilogue(const GemmParams& p, EpilogueOperands<NBLK>
     load_channel_scales(sbase && o.cols.a_ok ? sbase + o.cols.col_a : nullptr, o.sc0);
     load_channel_scales(sbase && o.cols.b_ok ? sbase + (o.cols.paired ? p.n_out + o.cols.col_a : o.cols.col_b) : nullptr,
                         o.sc1);
-    load_epilogue_rows<GEMM0, NBLK, SKIP_PAD>(p, o.rows, row0, nrows, first_row, row_step, r32);
+    load_epilogue_rows<MODE, GEMM0, NBLK, SKIP_PAD>(p, o.rows, row0, nrows, first_row, row_step, r32);
 }
 
 // Every load of load_epilogue completes here, on every path: a load left pending on a path that does not use
@@ -578,9 +596,9 @@ __device__ inline void apply_epilogue_block(const GemmParams& p, typename ModeTr
     {
         const bool in_tile = r < nrows;
         if(c.a_ok)
-            epilogue_gemm1<MODE>(p, acc[0], sc0, row0 + r, in_tile && rows.real[i], c.col_a, expert);
+            epilogue_gemm1<MODE>(p, acc[0], sc0, rows.sa[i], row0 + r, in_tile && rows.real[i], c.col_a, expert);
         if(c.b_ok)
-            epilogue_gemm1<MODE>(p, acc[1], sc1, row0 + r, in_tile && rows.real[i], c.col_b, expert);
+            epilogue_gemm1<MODE>(p, acc[1], sc1, rows.sa[i], row0 + r, in_tile && rows.real[i], c.col_b, expert);
     }
 }
 

@@ -259,6 +259,107 @@ __global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t
     }
 }
 
+// Re-quantisation of the intermediate activations between the two GEMMs of the int8 path (fused_quant 1 / 2 of
+// ck_tile's fused_moe_traits; y_smooth_scale of FusedMoeGemmHostArgs, fused_moegemm_kernel.hpp:103): sorted row r
+// of Y (bf16, row-major) times the smooth scale of its expert (SMOOTH), per-row dynamic quantisation to int8:
+// scale = amax / 127, codes rounded to nearest even (|value / scale| <= 127 needs no clamp).  ck_tile has no
+// instance of these variants to match bit for bit, so the rounding is chosen for accuracy: truncation, which the
+// stand-alone smooth-quant kernel above has to use to match ck_tile's, doubles the error of the down GEMM's
+// input.  One wave per row; a row of up to 2048 columns is read once.
+// Output row-major, or slab-major when segs > 0 (y_slab_offset); padding rows become zeros with scale 0, rows past
+// the sorted prefix are left alone.
+template <bool SMOOTH>
+__global__ __launch_bounds__(256) void moe_requant_y_kernel(const uint16_t* __restrict__ y, int inter,
+                                                             const float* __restrict__ smooth,
+                                                             const int* __restrict__ sorted_ids,
+                                                             const int* __restrict__ sorted_expert_ids,
+                                                             const int* __restrict__ total, int unit, int tokens, int segs,
+                                                             unsigned char* __restrict__ yq, float* __restrict__ yscale)
+{
+    const int lane    = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if(row >= total[0])
+        return;
+    const int chunks = inter >> 3;
+    auto dst = [&](int c) {
+        return yq + (segs > 0 ? y_slab_offset(row, c * 8, segs) : row * inter + c * 8);
+    };
+    const bool real = (sorted_ids[row] & 0xffffff) < tokens;
+    if(!real)
+    {
+        for(int c = lane; c < chunks; c += 64)
+            *reinterpret_cast<uint2*>(dst(c)) = make_uint2(0u, 0u);
+        if(lane == 0)
+            yscale[row] = 0.f;
+        return;
+    }
+    const uint16_t* yr = y + row * inter;
+    const float* sr    = SMOOTH ? smooth + (int64_t)sorted_expert_ids[row / unit] * inter : nullptr;
+    auto load = [&](int c, float (&o)[8]) {
+        const uint4 r = *reinterpret_cast<const uint4*>(yr + c * 8);
+        const uint32_t d[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            o[2 * i]     = __uint_as_float(d[i] << 16);
+            o[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+        }
+        if constexpr(SMOOTH)
+        {
+            const float4 s0 = *reinterpret_cast<const float4*>(sr + c * 8);
+            const float4 s1 = *reinterpret_cast<const float4*>(sr + c * 8 + 4);
+            o[0] *= s0.x; o[1] *= s0.y; o[2] *= s0.z; o[3] *= s0.w;
+            o[4] *= s1.x; o[5] *= s1.y; o[6] *= s1.z; o[7] *= s1.w;
+        }
+    };
+    float v[kQuantCache][8];
+    float amax = 0.f;
+#pragma unroll
+    for(int j = 0; j < kQuantCache; j++)
+    {
+        const int c = lane + 64 * j;
+        if(c < chunks)
+        {
+            load(c, v[j]);
+#pragma unroll
+            for(int i = 0; i < 8; i++)
+                amax = fmaxf(amax, fabsf(v[j][i]));
+        }
+    }
+    for(int c = lane + 64 * kQuantCache; c < chunks; c += 64)
+    {
+        float t[8];
+        load(c, t);
+#pragma unroll
+        for(int i = 0; i < 8; i++)
+            amax = fmaxf(amax, fabsf(t[i]));
+    }
+#pragma unroll
+    for(int d = 32; d > 0; d >>= 1)
+        amax = fmaxf(amax, __shfl_xor(amax, d));
+    const float ys_out = amax / 127.0f;
+    const float ys     = amax > 0.f ? ys_out : 1.0f; // a row of zeros: scale 0, codes 0
+    if(lane == 0)
+        yscale[row] = ys_out;
+    auto store = [&](int c, const float (&o)[8]) {
+        uint32_t w[2] = {0u, 0u};
+#pragma unroll
+        for(int i = 0; i < 8; i++)
+            w[i >> 2] |= (static_cast<uint32_t>(static_cast<int>(__builtin_rintf(o[i] / ys))) & 0xffu) << (8 * (i & 3));
+        *reinterpret_cast<uint2*>(dst(c)) = make_uint2(w[0], w[1]);
+    };
+#pragma unroll
+    for(int j = 0; j < kQuantCache; j++)
+        if(lane + 64 * j < chunks)
+            store(lane + 64 * j, v[j]);
+    for(int c = lane + 64 * kQuantCache; c < chunks; c += 64)
+    {
+        float t[8];
+        load(c, t);
+        store(c, t);
+    }
+}
+
 // ck_tile's pre-shuffled weight layout b_nr_kr_kw_nw_kv: the row-major [e, n, k] tensor viewed as
 // [e, nr, nw, kr, kw, kv] and permuted to [e, nr, kr, kw, nw, kv].  One thread moves one kv granule.
 template <typename G>
@@ -370,6 +471,23 @@ int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stri
         vec ? launch(rowwise_quant_kernel<true, true>) : launch(rowwise_quant_kernel<true, false>);
     else
         vec ? launch(rowwise_quant_kernel<false, true>) : launch(rowwise_quant_kernel<false, false>);
+    MI355_HIP_TRY(hipGetLastError());
+    return MI355_MOE_OK;
+}
+
+int launch_requant_y(const void* y, int32_t inter, const float* smooth, const int* sorted_ids, const int* sorted_expert_ids,
+                     const int* total, int32_t unit, int32_t tokens, int32_t segs, int64_t max_rows, void* yq, float* yscale,
+                     hipStream_t stream)
+{
+    if(max_rows <= 0)
+        return MI355_MOE_OK;
+    KernelTimer timer(MI355_MOE_K_QUANT, stream);
+    const dim3 grid((unsigned)ceil_div<int64_t>(max_rows, 4));
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(y), inter, smooth, sorted_ids,
+                           sorted_expert_ids, total, unit, tokens, segs, static_cast<unsigned char*>(yq), yscale);
+    };
+    smooth != nullptr ? launch(moe_requant_y_kernel<true>) : launch(moe_requant_y_kernel<false>);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }
