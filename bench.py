@@ -38,7 +38,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_workload(cfg, steps, warmup, seed=0, fused_quant=0):
+def run_workload(cfg, steps, warmup, seed=0, fused_quant=0, hot_expert=False):
     """Times `steps` passes of the path (fused_quant 2: the int8 path re-quantises the intermediate activations
     per row and runs the down GEMM on int8 MFMAs).  The dominant kernel's duration comes from HIP events the
     library records on the launch stream inside the timed region, the other kernels' from an untimed
@@ -51,6 +51,10 @@ def run_workload(cfg, steps, warmup, seed=0, fused_quant=0):
 
     dev = torch.device("cuda:0")
     inp = mi.make_inputs_torch(cfg, dev, seed)
+    if hot_expert:  # expert 0 in every token's top-k: one expert with `tokens` rows among decode-sized ones
+        ids = inp["topk_ids"].clone()
+        ids[~(ids == 0).any(dim=1), cfg.topk - 1] = 0
+        inp["topk_ids"] = ids.contiguous()
     traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit, fused_quant=fused_quant)
     buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, dev)
     args = ta.make_args(traits, buf, inp["a"], inp["g"], inp["d"], inp["topk_ids"], inp["topk_weight"],
@@ -86,7 +90,7 @@ def run_workload(cfg, steps, warmup, seed=0, fused_quant=0):
     byt = mi.decode_bytes(cfg, active, post_pad)
     gemm_ms = kavg.get("moe_gemm0_gate_up_silu", 0) + kavg.get("moe_gemm1_down", 0) + kavg.get("moe_combine", 0) + kavg.get("moe_prep", 0)
     res = {
-        "workload": cfg.name, "dtype": cfg.dtype, "tokens": T, "hidden": H, "inter": I, "experts": cfg.experts,
+        "workload": cfg.name, "dtype": cfg.dtype, "fused_quant": fused_quant, "tokens": T, "hidden": H, "inter": I, "experts": cfg.experts,
         "topk": K, "block_m": cfg.unit, "tile_rows": ta.fused_moe_tile_rows(traits, T, cfg.experts, K, H, I),
         "ms_per_step": ms, "tflops": cfg.flops / ms / 1e9,
         "tokens_per_s": T / ms * 1e3, "algorithmic_GB": byt / 1e9, "hbm_GBps": byt / ms / 1e6,
@@ -138,7 +142,8 @@ def roofline_of(cfg, res, gemm=0):
         byt = ae * 2 * I * H * b + ae * 2 * I * 4 + T * H * b + res["post_pad"] * I * y_b
     else:
         flop = 2.0 * T * K * H * I
-        byt = ae * H * I * b + ae * H * 4 + res["post_pad"] * I * y_b + res["post_pad"] * H * 2
+        yq_b = 1 if res.get("fused_quant") else y_b  # re-quantised intermediate activations
+        byt = ae * H * I * b + ae * H * 4 + res["post_pad"] * I * yq_b + res["post_pad"] * H * 2
     gbps = byt / kms / 1e6
     tflops = flop / kms / 1e9
     # prefill-sized workloads (tens of rows or more per expert) are graded against the MFMA peak, the
@@ -361,6 +366,32 @@ def main():
                 log(f"[bench] {name} failed: {e!r}")
                 others[name] = {"error": repr(e)}
 
+    # Beyond the benchmark configurations: the int8 model at a prefill-sized token count, with the intermediate
+    # activations kept in bf16 (fused_quant 0) or re-quantised to int8 so that the down GEMM runs on int8 MFMAs
+    # (fused_quant 2), and decode-sized batches whose routing is skewed (Zipf; one expert in every token's top-k).
+    extra = {}
+    if not a.headline_only:
+        i8 = mi.CONFIGS["cfg4_decode_int8_t256"]
+        cases = {
+            "cfg4_model_int8_t8192_fused_quant0": (i8.scaled(name="cfg4_model_int8_t8192", tokens=8192), {}),
+            "cfg4_model_int8_t8192_fused_quant2": (i8.scaled(name="cfg4_model_int8_t8192", tokens=8192), {"fused_quant": 2}),
+            "cfg4_decode_int8_t256_zipf": (i8.scaled(name="cfg4_decode_int8_t256_zipf", router="zipf"), {}),
+            "cfg4_decode_int8_t256_hot_expert": (i8.scaled(name="cfg4_decode_int8_t256_hot_expert"), {"hot_expert": True}),
+        }
+        for name, (c, kw) in cases.items():
+            try:
+                r, i2, b2 = run_workload(c, max(5, a.steps // 2), a.warmup, **kw)
+                r["roofline"] = roofline_of(c, r)
+                r["roofline_gemm1"] = roofline_of(c, r, 1)
+                extra[name] = r
+                log(f"[bench] {name}: {r['ms_per_step']:.3f} ms/step, {r['tflops']:.1f} TFLOP/s, "
+                    f"{r['hbm_GBps']:.0f} GB/s, kernels {r['kernel_avg_ms']}")
+                del i2, b2
+                torch.cuda.empty_cache()
+            except Exception as e:
+                log(f"[bench] {name} failed: {e!r}")
+                extra[name] = {"error": repr(e)}
+
     line = {
         "metric": METRIC, "value": res["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
@@ -373,6 +404,7 @@ def main():
         "hbm_GBps": res["hbm_GBps"], "kernel_avg_ms": res["kernel_avg_ms"], "gemm0_tflops": res["gemm0_tflops"],
         "gemm1_tflops": res["gemm1_tflops"], "roofline": roof, "roofline_gemm1": roofline_of(cfg, res, 1),
         "cpu_baseline": cpu, "router": router, "neighbours": neighbours, "workloads": others,
+        "extra_workloads": extra,
     }
     print(json.dumps(line), flush=True)
 
