@@ -302,6 +302,11 @@ def main():
     ap.add_argument("--headline-only", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true")
+    # variations of the named workload, for profiling runs of what `extra_workloads` reports
+    ap.add_argument("--tokens", type=int, default=0, help="token count instead of the workload's own")
+    ap.add_argument("--fused-quant", type=int, default=0, choices=(0, 2),
+                    help="int8 workloads: 2 = re-quantise the intermediate activations (down GEMM on int8 MFMAs)")
+    ap.add_argument("--router", default="", help="routing instead of the workload's own (e.g. zipf)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures one GPU only; run with --gpus 1 (the path is single-GPU: across "
@@ -313,8 +318,11 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     cfg = mi.CONFIGS[a.workload]
+    if a.tokens or a.router:
+        cfg = cfg.scaled(name=f"{cfg.name}_t{a.tokens or cfg.tokens}{'_' + a.router if a.router else ''}",
+                         tokens=a.tokens or cfg.tokens, router=a.router or cfg.router)
     log(f"[bench] {cfg}")
-    res, inp, buf = run_workload(cfg, a.steps, a.warmup)
+    res, inp, buf = run_workload(cfg, a.steps, a.warmup, fused_quant=a.fused_quant)
     log(f"[bench] {cfg.name}: {res['ms_per_step']:.3f} ms/step, {res['tflops']:.1f} TFLOP/s, kernels {res['kernel_avg_ms']}")
     roof = roofline_of(cfg, res)
     if a.calibrate_copy:

@@ -132,9 +132,10 @@ int mi355_topk_softmax(const mi355_topk_softmax_traits* traits, const mi355_topk
 /* ------------------------------------------------------------------------------- fused MoE */
 typedef struct mi355_fused_moe_traits
 {
-    int32_t prec_i;  /* activation dtype  (mi355_moe_dtype): BF16 | FP8 | INT8 */
+    int32_t prec_i;  /* activation dtype  (mi355_moe_dtype): BF16 | FP16 | FP8 | INT8 */
     int32_t prec_w;  /* weight dtype: same as prec_i */
-    int32_t prec_o;  /* output dtype: BF16 */
+    int32_t prec_o;  /* output dtype: BF16; FP16 with FP16 operands (ck_tile's two instances,
+                        fused_moegemm_pipeline_flatmm_policy.hpp:790-807) */
     int32_t prec_st; /* per-token activation scale dtype: FP32 */
     int32_t prec_sw; /* per-channel weight scale dtype: FP32 */
     int32_t prec_sq; /* smooth-quant scale dtype: FP32 (unused) */

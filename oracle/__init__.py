@@ -364,16 +364,28 @@ def fused_moe(a, a_dt, g, g_dt, d, d_dt, sorted_ids, sorted_w, sorted_eid, post_
     return (o, part) if want_partials else o
 
 
+def fused_moe_f16(a, g, d, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, tokens, experts, hidden, inter, topk,
+                  **kw):
+    """The oracle for fp16 operands (numpy float16 arrays) and fp16 output: every fp16 value is an fp32 value, so the
+    operands go in as float32 and the fp32 result is rounded to fp16 once (numpy's cast: IEEE round to nearest even),
+    which is what reference_fused_moe does when instantiated with half_t (reference_fused_moe.hpp:186-197)."""
+    f = lambda x: np.ascontiguousarray(np.asarray(x, dtype=np.float16).astype(np.float32))
+    o = fused_moe(f(a), DT_F32, f(g), DT_F32, f(d), DT_F32, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, tokens,
+                  experts, hidden, inter, topk, out_dt=DT_F32, **kw)
+    return o.astype(np.float16)
+
+
 def ck_fused_moe(a, g, d, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, tokens, experts,
-                 hidden, inter, topk, gate_only=False, f32_inputs=False, activation=1):
-    """ck_tile::reference_fused_moe on bf16 (uint16 bits) or float32 operands -> bf16 bits."""
+                 hidden, inter, topk, gate_only=False, f32_inputs=False, activation=1, f16=False):
+    """ck_tile::reference_fused_moe on bf16 (uint16 bits), fp16 (f16: float16 bits in and out) or float32 operands
+    -> bf16 bits (fp16 bits with f16)."""
     r = ck_ref()
     if r is None:
         raise RuntimeError("oracle/_ref is not built")
     dt = np.float32 if f32_inputs else np.uint16
     a, g, d = _c(a, dt), _c(g, dt), _c(d, dt)
     o = np.empty((tokens, hidden), dtype=np.uint16)
-    fn = r.ck_ref_fused_moe_f32 if f32_inputs else r.ck_ref_fused_moe_bf16
+    fn = r.ck_ref_fused_moe_f32 if f32_inputs else (r.ck_ref_fused_moe_f16 if f16 else r.ck_ref_fused_moe_bf16)
     ids, w, eid = _c(sorted_ids, np.int32), _c(sorted_w, np.float32), _c(sorted_eid, np.int32)
     fn(_p(a), _p(g), _p(d), _p(o), _p(ids), _p(w), _p(eid), int(post_pad), block_m, tokens, experts,
        hidden, inter, topk, int(bool(gate_only)), int(activation))

@@ -37,7 +37,7 @@ HostTensor<T> make_tensor(std::vector<std::size_t> lens, const void* src)
     return t;
 }
 
-template <typename AT, typename GT, typename DT, typename Act>
+template <typename AT, typename GT, typename DT, typename Act, typename OT = ck_tile::bf16_t>
 int run_fused(const void* a, const void* g, const void* d, void* o_bf16,
               const int32_t* sorted_ids, const float* sorted_w, const int32_t* sorted_eid,
               int32_t post_pad, int32_t block_m, int32_t T, int32_t E, int32_t H, int32_t I,
@@ -52,7 +52,8 @@ int run_fused(const void* a, const void* g, const void* d, void* o_bf16,
     auto d_h = make_tensor<DT>({(std::size_t)E, (std::size_t)H, (std::size_t)I}, d);
     HostTensor<float> sa({(std::size_t)T}), sg({(std::size_t)E, n0}), sd({(std::size_t)E, (std::size_t)H}),
         sy({(std::size_t)E, (std::size_t)I});
-    HostTensor<ck_tile::bf16_t> o_h({(std::size_t)T, (std::size_t)H});
+    HostTensor<OT> o_h({(std::size_t)T, (std::size_t)H});
+    static_assert(sizeof(OT) == 2, "16-bit output types");
     auto ids_h = make_tensor<index_t>({max_pad}, nullptr);
     auto w_h   = make_tensor<float>({max_pad}, nullptr);
     auto eid_h = make_tensor<index_t>({tiles}, nullptr);
@@ -120,6 +121,21 @@ ck_ref_fused_moe_bf16(const void* a, const void* g, const void* d, void* o, cons
             a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, T, E, H, I, K, gate_only);
     return run_fused<ck_tile::bf16_t, ck_tile::bf16_t, ck_tile::bf16_t, ck_tile::element_wise::Silu>(
         a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad, block_m, T, E, H, I, K, gate_only);
+}
+
+// fp16 activations, weights and output (ck_tile's other fused-MoE instance)
+__attribute__((visibility("default"))) int
+ck_ref_fused_moe_f16(const void* a, const void* g, const void* d, void* o, const int32_t* sorted_ids,
+                     const float* sorted_w, const int32_t* sorted_eid, int32_t post_pad,
+                     int32_t block_m, int32_t T, int32_t E, int32_t H, int32_t I, int32_t K,
+                     int32_t gate_only, int32_t activation)
+{
+    using h = ck_tile::half_t;
+    if(activation == 0)
+        return run_fused<h, h, h, ck_tile::element_wise::Gelu, h>(a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad,
+                                                                  block_m, T, E, H, I, K, gate_only);
+    return run_fused<h, h, h, ck_tile::element_wise::Silu, h>(a, g, d, o, sorted_ids, sorted_w, sorted_eid, post_pad,
+                                                              block_m, T, E, H, I, K, gate_only);
 }
 
 // fp32 (de-quantised) activations and weights, bf16 output: the definition used for the

@@ -5,7 +5,7 @@ import torch
 
 import therock_amd as ta
 
-TORCH_DT = {"bf16": torch.bfloat16, "fp8": torch.float8_e4m3fn, "int8": torch.int8}
+TORCH_DT = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp8": torch.float8_e4m3fn, "int8": torch.int8}
 NP_VIEW = {"bf16": torch.uint16, "fp8": torch.uint8, "int8": torch.int8}
 
 
@@ -41,9 +41,10 @@ def run_sorting(topk_ids, weights, experts, unit, mask=None, local_tokens=None, 
 
 def run_fused_moe(cfg, inp, mask=None, unfused=False, stride_pad=0, activation=1, gate_only=0):
     """Runs mi355_fused_moe (or sorting + mi355_fused_moegemm) on numpy inputs of
-    therock_amd.inputs.make_inputs_np.  Returns (out bf16 bits [T,H] numpy, buffers)."""
-    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit,
-                                 local_expert_masking=mask is not None, activation=activation, gate_only=gate_only)
+    therock_amd.inputs.make_inputs_np.  Returns (out bf16 bits (fp16 bits for fp16 operands) [T,H] numpy, buffers)."""
+    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, prec_o="fp16" if cfg.dtype == "fp16" else "bf16",
+                                 block_m=cfg.unit, local_expert_masking=mask is not None, activation=activation,
+                                 gate_only=gate_only)
     buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, "cuda")
     view = TORCH_DT[cfg.dtype]
     a = dev(inp["a"]).view(view)
@@ -51,7 +52,7 @@ def run_fused_moe(cfg, inp, mask=None, unfused=False, stride_pad=0, activation=1
         wide = torch.zeros((cfg.tokens, cfg.hidden + stride_pad), dtype=view, device="cuda")
         wide[:, :cfg.hidden] = a
         a = wide[:, :cfg.hidden]
-        buf.out = torch.zeros((cfg.tokens, cfg.hidden + stride_pad), dtype=torch.bfloat16, device="cuda")[:, :cfg.hidden]
+        buf.out = torch.zeros((cfg.tokens, cfg.hidden + stride_pad), dtype=buf.out.dtype, device="cuda")[:, :cfg.hidden]
     g, d = dev(inp["g"]).view(view), dev(inp["d"]).view(view)
     sc = {k: (None if inp[k] is None else dev(inp[k])) for k in ("a_scale", "g_scale", "d_scale")}
     args = ta.make_args(traits, buf, a, g, d, dev(inp["topk_ids"]), dev(inp["topk_weight"]), a_scale=sc["a_scale"],

@@ -273,3 +273,40 @@ def test_large_tile_kernel(dtype):
     check(mi.MoeConfig("b", 700, 320, 128, 4, 1, dtype, "softmax_renorm", unit=64), seed=2)
     check(mi.MoeConfig("b", 2000, 192, 256, 6, 3, dtype, "zipf"), seed=3)
     check(mi.MoeConfig("b", 600, 64, 128, 2, 1, dtype, "softmax_renorm"), seed=4)
+
+
+# ---- fp16 operands and output: ck_tile's other instance (fused_moegemm_pipeline_flatmm_policy.hpp:790-807)
+def check_fp16(cfg, seed=0, **kw):
+    from tests.gpu_util import rel_l2, run_fused_moe
+    inp = mi.make_inputs_np(cfg, seed)
+    if kw.get("gate_only"):
+        inp["g"] = np.ascontiguousarray(inp["g"][:, :cfg.inter])
+    print(f"fused_moe {cfg} seed={seed} {kw}", flush=True)
+    got, buf = run_fused_moe(cfg, inp, **kw)
+    s = oracle.moe_sorting(inp["topk_ids"], inp["topk_weight"], cfg.experts, cfg.unit)
+    ref = oracle.fused_moe_f16(inp["a"].view(np.float16), inp["g"].view(np.float16), inp["d"].view(np.float16), *s, cfg.unit,
+                               cfg.tokens, cfg.experts, cfg.hidden, cfg.inter, cfg.topk, activation=kw.get("activation", 1),
+                               gate_only=bool(kw.get("gate_only", 0))).astype(np.float32)
+    got = got.view(np.float16).astype(np.float32)
+    assert np.all(np.isfinite(got))
+    err = rel_l2(got, ref)
+    print(f"  rel-L2 = {err:.3e} (tolerance 1e-02)", flush=True)
+    assert err <= 1e-2
+    return err
+
+
+@pytest.mark.parametrize("cfg", [
+    mi.MoeConfig("f16_decode", 8, 128, 128, 4, 2, "fp16"),
+    mi.MoeConfig("f16_mid", 300, 512, 384, 8, 2, "fp16"),
+    mi.MoeConfig("f16_mid_sigmoid", 48, 512, 256, 16, 4, "fp16", "sigmoid_renorm"),
+    mi.MoeConfig("f16_big", 2048, 512, 256, 8, 2, "fp16"),
+], ids=lambda c: c.name)
+def test_fp16(cfg):
+    err = check_fp16(cfg)
+    assert err <= 2e-3  # fp16 Y and partial rows: three more bits than the bf16 path's 3.3e-3
+
+
+def test_fp16_variants():
+    check_fp16(mi.MoeConfig("f16_gelu", 128, 256, 256, 8, 2, "fp16"), activation=0)
+    check_fp16(mi.MoeConfig("f16_gate_only", 128, 256, 256, 8, 2, "fp16"), gate_only=1)
+    check_fp16(mi.MoeConfig("f16_unfused", 128, 256, 256, 8, 2, "fp16"), unfused=True)

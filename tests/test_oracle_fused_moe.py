@@ -176,3 +176,23 @@ def test_bit_exact_with_ck_tile_reference(dtype, activation, gate_only):
                                  *s, cfg.unit, cfg.tokens, cfg.experts, cfg.hidden, cfg.inter, cfg.topk, f32_inputs=True,
                                  **kw)
     assert np.array_equal(mine, ck)
+
+
+@pytest.mark.skipif(oracle.ck_ref() is None, reason="oracle/_ref not built")
+@pytest.mark.parametrize("activation,gate_only", [(1, False), (0, False), (1, True)])
+def test_fp16_bit_exact_with_ck_tile_reference(activation, gate_only):
+    """ck_tile's other instance: fp16 operands and output.  The oracle takes the fp16 values as float32 and rounds its
+    fp32 result to fp16 once; reference_fused_moe instantiated with half_t must give the same bits."""
+    cfg = mi.MoeConfig("t", 19, 128, 96, 6, 2, "fp16", "softmax_renorm", unit=8)
+    inp = mi.make_inputs_np(cfg, 13)
+    if gate_only:
+        inp["g"] = np.ascontiguousarray(inp["g"][:, :cfg.inter])
+    s = oracle.moe_sorting(inp["topk_ids"], inp["topk_weight"], cfg.experts, cfg.unit)
+    kw = dict(activation=activation, gate_only=gate_only)
+    mine = oracle.fused_moe_f16(inp["a"].view(np.float16), inp["g"].view(np.float16), inp["d"].view(np.float16), *s,
+                                cfg.unit, cfg.tokens, cfg.experts, cfg.hidden, cfg.inter, cfg.topk, strict=True, **kw)
+    ck = oracle.ck_fused_moe(inp["a"], inp["g"], inp["d"], *s, cfg.unit, cfg.tokens, cfg.experts, cfg.hidden, cfg.inter,
+                             cfg.topk, f16=True, **kw)
+    assert np.array_equal(mine.view(np.uint16), ck)
+    # and it is not the bf16 result in disguise: fp16 keeps three more bits
+    assert mine.dtype == np.float16 and np.isfinite(mine.astype(np.float32)).all()

@@ -67,6 +67,18 @@ __device__ inline uint32_t float_to_bf16_bits(float f)
 }
 
 // two floats -> packed bf16 pair, round-to-nearest-even: a single v_cvt_pk_bf16_f32 on gfx950
+// two floats -> packed fp16 (round to nearest even, overflow to infinity: the IEEE conversion)
+__device__ inline uint32_t pack_f16x2(float lo, float hi)
+{
+    const _Float16 a = static_cast<_Float16>(lo), b = static_cast<_Float16>(hi);
+    return static_cast<uint32_t>(__builtin_bit_cast(unsigned short, a)) |
+           (static_cast<uint32_t>(__builtin_bit_cast(unsigned short, b)) << 16);
+}
+__device__ inline float f16_bits_to_float(uint32_t h)
+{
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(h)));
+}
+
 __device__ inline uint32_t pack_bf16x2(float lo, float hi)
 {
     typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;

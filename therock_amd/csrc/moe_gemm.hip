@@ -360,8 +360,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
                                                            int64_t out_row_bytes, int accumulate,
                                                            const float* __restrict__ slot_scale,
                                                            const float* __restrict__ bias,
-                                                           const int* __restrict__ sorted_eid, int unit)
+                                                           const int* __restrict__ sorted_eid, int unit, int f16)
 {
+    // f16: the partial rows and the output are fp16 instead of bf16 (a uniform branch)
     const int t  = blockIdx.x;
     const int h0 = (blockIdx.y * 256 + threadIdx.x) * 8;
     if(h0 >= hidden)
@@ -410,8 +411,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
 #pragma unroll
             for(int i = 0; i < 4; i++)
             {
-                acc[2 * i] += w[j] * __uint_as_float(v[j][i] << 16);
-                acc[2 * i + 1] += w[j] * __uint_as_float(v[j][i] & 0xffff0000u);
+                acc[2 * i] += w[j] * (f16 ? f16_bits_to_float(v[j][i] & 0xffffu) : __uint_as_float(v[j][i] << 16));
+                acc[2 * i + 1] += w[j] * (f16 ? f16_bits_to_float(v[j][i] >> 16) : __uint_as_float(v[j][i] & 0xffff0000u));
             }
             if(bias != nullptr) // stand-alone down GEMM with an expert bias: (dot + bias) * top-k weight
             {
@@ -424,10 +425,20 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
         }
     }
     uint4 o;
-    o.x = pack_bf16x2(acc[0], acc[1]);
-    o.y = pack_bf16x2(acc[2], acc[3]);
-    o.z = pack_bf16x2(acc[4], acc[5]);
-    o.w = pack_bf16x2(acc[6], acc[7]);
+    if(f16)
+    {
+        o.x = pack_f16x2(acc[0], acc[1]);
+        o.y = pack_f16x2(acc[2], acc[3]);
+        o.z = pack_f16x2(acc[4], acc[5]);
+        o.w = pack_f16x2(acc[6], acc[7]);
+    }
+    else
+    {
+        o.x = pack_bf16x2(acc[0], acc[1]);
+        o.y = pack_bf16x2(acc[2], acc[3]);
+        o.z = pack_bf16x2(acc[4], acc[5]);
+        o.w = pack_bf16x2(acc[6], acc[7]);
+    }
     *reinterpret_cast<uint4*>(out + (int64_t)t * out_row_bytes + (int64_t)h0 * 2) = o;
 }
 
@@ -445,7 +456,7 @@ inline int y_bytes(const mi355_fused_moe_traits& t)
 inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
 {
     const int64_t avg = tokens * topk / std::max(experts, 1);
-    const int eb  = t.prec_i == MI355_MOE_BF16 ? 2 : 1;
+    const int eb  = (t.prec_i == MI355_MOE_BF16 || t.prec_i == MI355_MOE_FP16) ? 2 : 1;
     const int y_b = y_bytes(t);
     // the large-tile kernel addresses each operand as a base plus a 32-bit byte offset
     const int64_t lim     = (int64_t)1 << 32;
@@ -508,6 +519,8 @@ int launch_grouped_gemm(int prec, bool gemm0, int mblk, bool use_decode, GemmPar
         return launch_gemm_big(prec, gemm0, p, max_tiles, stream, y_i8);
     if(prec == MI355_MOE_BF16)
         return gemm0 ? launch_gemm<kBf16, true>(mblk, p, max_tiles, stream) : launch_gemm<kBf16, false>(mblk, p, max_tiles, stream);
+    if(prec == MI355_MOE_FP16)
+        return gemm0 ? launch_gemm<kF16, true>(mblk, p, max_tiles, stream) : launch_gemm<kF16, false>(mblk, p, max_tiles, stream);
     if(prec == MI355_MOE_FP8)
         return gemm0 ? launch_gemm<kFp8, true>(mblk, p, max_tiles, stream) : launch_gemm<kFp8, false>(mblk, p, max_tiles, stream);
     if(gemm0)
@@ -526,8 +539,10 @@ bool down_gemm_wants_decode(int experts, int64_t entries, int hidden)
 
 int check_traits(const mi355_fused_moe_traits& t)
 {
-    const bool prec_ok = (t.prec_i == MI355_MOE_BF16 || t.prec_i == MI355_MOE_FP8 || t.prec_i == MI355_MOE_INT8) &&
-                         t.prec_w == t.prec_i && t.prec_o == MI355_MOE_BF16;
+    // output: bf16, or fp16 with fp16 operands (ck_tile's two instances, fused_moegemm_pipeline_flatmm_policy.hpp:790-807)
+    const bool prec_ok = (t.prec_i == MI355_MOE_BF16 || t.prec_i == MI355_MOE_FP8 || t.prec_i == MI355_MOE_INT8 ||
+                          t.prec_i == MI355_MOE_FP16) &&
+                         t.prec_w == t.prec_i && t.prec_o == (t.prec_i == MI355_MOE_FP16 ? MI355_MOE_FP16 : MI355_MOE_BF16);
     if(!prec_ok)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: unsupported precision (i=%d w=%d o=%d)", t.prec_i, t.prec_w,
                     t.prec_o);
@@ -627,7 +642,7 @@ int validate_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_mo
                                          "(fused_quant=%d)", t.fused_quant);
     if(t.fused_quant == 1 && (reinterpret_cast<uintptr_t>(a.y_smooth_scale_ptr) % 16 != 0 || I % 8 != 0))
         return fail(MI355_MOE_E_INVALID, "fused_moegemm: y_smooth_scale must be 16-byte aligned");
-    const bool quant = t.prec_i != MI355_MOE_BF16;
+    const bool quant = t.prec_i != MI355_MOE_BF16 && t.prec_i != MI355_MOE_FP16;
     if(quant && (!a.a_scale_ptr || !a.g_scale_ptr || !a.d_scale_ptr))
         return fail(MI355_MOE_E_INVALID, "fused_moegemm: quantised dtypes need a_scale, g_scale and d_scale");
     const int eb = quant ? 1 : 2; // bytes per activation / weight element
@@ -655,7 +670,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
         return rc;
     if(a.num_tokens == 0)
         return MI355_MOE_OK;
-    const bool quant = t.prec_i != MI355_MOE_BF16;
+    const bool quant = t.prec_i != MI355_MOE_BF16 && t.prec_i != MI355_MOE_FP16;
     const int H = a.hidden_size, I = a.intermediate_size, T = a.num_tokens, E = a.num_experts, K = a.topk;
     const int eb = quant ? 1 : 2;
     const WorkspaceLayout ws = workspace_layout(t, T, E, K, H, I);
@@ -756,7 +771,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, inv,
                        static_cast<const float*>(a.sorted_weight_ptr), static_cast<unsigned char*>(a.o_ptr), K, H,
                        (int64_t)a.stride_token * 2, 0, static_cast<const float*>(nullptr), static_cast<const float*>(nullptr),
-                       static_cast<const int*>(nullptr), 1);
+                       static_cast<const int*>(nullptr), 1, t.prec_i == MI355_MOE_FP16 ? 1 : 0);
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
@@ -950,7 +965,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
         hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + L.p_off, inv,
                            static_cast<const float*>(a.p_sorted_expert_weights), static_cast<unsigned char*>(a.c_ptr), K, H,
                            (int64_t)a.stride_C * 2, 1, f8 ? static_cast<const float*>(a.scale_m) : nullptr,
-                           static_cast<const float*>(a.exp_bias), static_cast<const int*>(a.p_sorted_expert_ids), a.block_m);
+                           static_cast<const float*>(a.exp_bias), static_cast<const int*>(a.p_sorted_expert_ids), a.block_m, 0);
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;

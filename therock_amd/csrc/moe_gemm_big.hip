@@ -127,7 +127,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     // weight bytes, so the 128-byte lines of a weight unit last four steps instead of two
     constexpr bool kW8 = MODE == kBf16W8;
     constexpr bool kMx   = MODE == kFp8 && !GEMM0;
-    static_assert(MODE == kBf16 || MODE == kFp8 || MODE == kI8 || (MODE == kBf16W8 && !GEMM0), "no large-tile kernel for this mode");
+    static_assert(MODE == kBf16 || MODE == kF16 || MODE == kFp8 || MODE == kI8 || (MODE == kBf16W8 && !GEMM0),
+                  "no large-tile kernel for this mode");
     // Software-pipelined K loop (kPipe): the operands of step k+1 are fetched from LDS into registers during step
     // k, each fragment right behind the last MFMA that reads its register, so that after a barrier the MFMAs start
     // at once instead of waiting for operand fetches that all eight waves issue at the same moment.  The barrier of
@@ -699,7 +700,8 @@ bool big_tile_supported(int prec, int k_bytes0, int k_bytes1, bool y_i8)
     // K in whole pairs of 64-byte steps; the int8 path's down GEMM with bf16 Y against int8 weights in fours
     if(prec == MI355_MOE_INT8)
         return k_bytes0 % (2 * kStepKB) == 0 && k_bytes1 % ((y_i8 ? 2 : 4) * kStepKB) == 0;
-    return (prec == MI355_MOE_BF16 || prec == MI355_MOE_FP8) && k_bytes0 % (2 * kStepKB) == 0 && k_bytes1 % (2 * kStepKB) == 0;
+    return (prec == MI355_MOE_BF16 || prec == MI355_MOE_FP16 || prec == MI355_MOE_FP8) && k_bytes0 % (2 * kStepKB) == 0 &&
+           k_bytes1 % (2 * kStepKB) == 0;
 }
 
 int launch_gemm_big(int prec, bool gemm0, const GemmParams& p, int max_tiles, hipStream_t stream, bool y_i8)
@@ -708,6 +710,8 @@ int launch_gemm_big(int prec, bool gemm0, const GemmParams& p, int max_tiles, hi
         return launch_big_t<kI8, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_BF16)
         return gemm0 ? launch_big_t<kBf16, true>(p, max_tiles, stream) : launch_big_t<kBf16, false>(p, max_tiles, stream);
+    if(prec == MI355_MOE_FP16)
+        return gemm0 ? launch_big_t<kF16, true>(p, max_tiles, stream) : launch_big_t<kF16, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_FP8)
         return gemm0 ? launch_big_t<kFp8, true>(p, max_tiles, stream) : launch_big_t<kFp8, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_INT8)

@@ -284,6 +284,8 @@ int launch_gemm_decode(int prec, bool gemm0, const GemmParams& p, int max_tiles,
         return launch_decode_t<kI8, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_BF16)
         return gemm0 ? launch_decode_t<kBf16, true>(p, max_tiles, stream) : launch_decode_t<kBf16, false>(p, max_tiles, stream);
+    if(prec == MI355_MOE_FP16)
+        return gemm0 ? launch_decode_t<kF16, true>(p, max_tiles, stream) : launch_decode_t<kF16, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_FP8)
         return gemm0 ? launch_decode_t<kFp8, true>(p, max_tiles, stream) : launch_decode_t<kFp8, false>(p, max_tiles, stream);
     if(prec == MI355_MOE_INT8)

@@ -9,6 +9,7 @@ namespace mi355 {
 namespace gemm {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(16))) int i32x16_t;
 typedef __attribute__((ext_vector_type(4))) int i32x4_t;
@@ -19,7 +20,8 @@ enum Mode
     kBf16   = 0, // x bf16, w bf16, bf16 MFMA
     kFp8    = 1, // x e4m3, w e4m3, block-scaled f8f6f4 MFMA
     kI8     = 2, // x int8, w int8, i8 MFMA (gemm1: int8 Y with a per-row scale, the fused_quant variants)
-    kBf16W8 = 3  // x bf16, w int8 converted to bf16 after the LDS read (gemm1 of the int8 path)
+    kBf16W8 = 3, // x bf16, w int8 converted to bf16 after the LDS read (gemm1 of the int8 path)
+    kF16    = 4  // x fp16, w fp16, f16 MFMA; Y, the partial rows and the output are fp16 (ck_tile's other instance)
 };
 
 constexpr int kBlock   = 256;
@@ -156,6 +158,10 @@ struct ModeTraits<kBf16>
     static constexpr int kXKB  = 128;
 };
 template <>
+struct ModeTraits<kF16> : ModeTraits<kBf16>
+{
+};
+template <>
 struct ModeTraits<kFp8>
 {
     using Acc                  = f32x16_t;
@@ -245,6 +251,10 @@ __device__ inline typename ModeTraits<MODE>::Acc mfma(const Frag& w, const Frag&
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(bit_cast_dev<bf16x8_t>(w.lo), bit_cast_dev<bf16x8_t>(x.lo), c,
                                                        0, 0, 0);
     }
+    else if constexpr(MODE == kF16)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(bit_cast_dev<f16x8_t>(w.lo), bit_cast_dev<f16x8_t>(x.lo), c, 0, 0, 0);
+    }
     else if constexpr(MODE == kI8)
     {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8(bit_cast_dev<i32x4_t>(w.lo), bit_cast_dev<i32x4_t>(x.lo), c, 0,
@@ -274,6 +284,16 @@ __device__ inline f32x16_t mfma_fp8_unscaled(const Frag& w, const Frag& x, f32x1
     b[0] = x.lo.x; b[1] = x.lo.y; b[2] = x.lo.z; b[3] = x.lo.w;
     b[4] = x.hi.x; b[5] = x.hi.y; b[6] = x.hi.z; b[7] = x.hi.w;
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// two results -> the 16-bit type the mode stores (fp16 for kF16, bf16 otherwise), both round to nearest even
+template <int MODE>
+__device__ inline uint32_t pack_out2(float lo, float hi)
+{
+    if constexpr(MODE == kF16)
+        return pack_f16x2(lo, hi);
+    else
+        return pack_bf16x2(lo, hi);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -432,10 +452,10 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
     else if(store)
     {
         uint4 o0, o1;
-        o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
-        o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
-        o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
-        o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
+        o0.x = pack_out2<MODE>(y[0], y[1]);   o0.y = pack_out2<MODE>(y[2], y[3]);
+        o0.z = pack_out2<MODE>(y[4], y[5]);   o0.w = pack_out2<MODE>(y[6], y[7]);
+        o1.x = pack_out2<MODE>(y[8], y[9]);   o1.y = pack_out2<MODE>(y[10], y[11]);
+        o1.z = pack_out2<MODE>(y[12], y[13]); o1.w = pack_out2<MODE>(y[14], y[15]);
         uint4* d4 = reinterpret_cast<uint4*>(dst);
         d4[0]     = o0;
         d4[1]     = o1;
@@ -455,10 +475,10 @@ __device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTr
     if(p.bias != nullptr || p.n_padded > 0) // uniform: stand-alone down GEMM with a bias or padded rows
         bias_and_padding(p, y, expert, col0);
     uint4 o0, o1;
-    o0.x = pack_bf16x2(y[0], y[1]);   o0.y = pack_bf16x2(y[2], y[3]);
-    o0.z = pack_bf16x2(y[4], y[5]);   o0.w = pack_bf16x2(y[6], y[7]);
-    o1.x = pack_bf16x2(y[8], y[9]);   o1.y = pack_bf16x2(y[10], y[11]);
-    o1.z = pack_bf16x2(y[12], y[13]); o1.w = pack_bf16x2(y[14], y[15]);
+    o0.x = pack_out2<MODE>(y[0], y[1]);   o0.y = pack_out2<MODE>(y[2], y[3]);
+    o0.z = pack_out2<MODE>(y[4], y[5]);   o0.w = pack_out2<MODE>(y[6], y[7]);
+    o1.x = pack_out2<MODE>(y[8], y[9]);   o1.y = pack_out2<MODE>(y[10], y[11]);
+    o1.z = pack_out2<MODE>(y[12], y[13]); o1.w = pack_out2<MODE>(y[14], y[15]);
     if(store)
     {
         uint4* d4 = reinterpret_cast<uint4*>(p.out + prow * p.out_row_bytes + (int64_t)col0 * 2);

@@ -26,7 +26,7 @@ class MoeConfig:
     inter: int
     experts: int
     topk: int
-    dtype: str = "bf16"  # "bf16" | "fp8" | "int8": storage type of activations and weights
+    dtype: str = "bf16"  # "bf16" | "fp16" | "fp8" | "int8": storage type of activations and weights
     router: str = "softmax_renorm"  # softmax_renorm | softmax | sigmoid_renorm | zipf
     unit: int = 32  # block_m / unit_size used by moe_sorting
 
@@ -136,6 +136,8 @@ def make_inputs_np(cfg: MoeConfig, seed: int = 0) -> dict:
     out = {"topk_ids": ids, "topk_weight": w, "a_scale": None, "g_scale": None, "d_scale": None}
     if cfg.dtype == "bf16":
         out["a"], out["g"], out["d"] = f32_to_bf16_bits(x), f32_to_bf16_bits(g), f32_to_bf16_bits(d)
+    elif cfg.dtype == "fp16":  # fp16 bits
+        out["a"], out["g"], out["d"] = (v.astype(np.float16).view(np.uint16) for v in (x, g, d))
     else:
         xb = bf16_bits_to_f32(f32_to_bf16_bits(x))  # activations start life as bf16
         out["a_bf16"] = f32_to_bf16_bits(x)

@@ -354,7 +354,8 @@ class MoeBuffers:
         self.total = torch.zeros((2,), dtype=torch.int32, device=device)
         ws = fused_moe_get_workspace_size(traits, tokens, experts, topk, hidden, inter)
         self.ws = torch.empty((max(ws, 256),), dtype=torch.uint8, device=device)
-        self.out = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=device)
+        self.out = torch.empty((tokens, hidden), dtype=torch.float16 if traits.prec_o == "fp16" else torch.bfloat16,
+                               device=device)
 
 
 def make_args(traits: fused_moe_traits, buf: MoeBuffers, a, g, d, topk_ids, topk_weight, a_scale=None,
