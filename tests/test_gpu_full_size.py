@@ -169,3 +169,28 @@ def test_fp8_accuracy_over_seeds_and_heavy_tails(seed, outliers):
     total, worst_token, worst_cell = error_profile(buf.out, fused_moe_fp32(cfg, inp))
     print(f"  fp8 seed {seed}, {outliers} outlier channels: rel-L2 {total:.3e}, worst token {worst_token:.3e}", flush=True)
     assert total <= 2.8e-2 and worst_token <= 3.3e-2
+
+
+@pytest.mark.parametrize("tokens", [256, 8192])
+def test_int8_fused_quant_full_size(tokens):
+    """fused_quant 2 on the int8 benchmark model at a decode-sized and a prefill-sized token count (decode kernel /
+    large-tile kernel with int8 x int8 down GEMM): every output element against the fp32 matmul reference of the
+    de-quantised operands, and bit-level determinism.  The re-quantisation of the intermediate activations (per row,
+    round to nearest) is the whole difference to the plain int8 path: bound 3e-2 as for every quantised path."""
+    cfg = mi.CONFIGS["cfg4_decode_int8_t256"].scaled(tokens=tokens)
+    inp = mi.make_inputs_torch(cfg, "cuda", seed=0)
+    traits = ta.fused_moe_traits(prec_i="int8", prec_w="int8", block_m=cfg.unit, fused_quant=2)
+    buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, "cuda")
+    args = ta.make_args(traits, buf, inp["a"], inp["g"], inp["d"], inp["topk_ids"], inp["topk_weight"],
+                        a_scale=inp["a_scale"], g_scale=inp["g_scale"], d_scale=inp["d_scale"])
+    assert ta.fused_moe(traits, args) == 0.0
+    torch.cuda.synchronize()
+    out1 = buf.out.clone()
+    total, worst_token, worst_cell = error_profile(out1, fused_moe_fp32(cfg, inp))
+    print(f"  int8 fused_quant 2, {tokens} tokens: rel-L2 {total:.3e}, worst token {worst_token:.3e}, worst cell "
+          f"{worst_cell:.3e}", flush=True)
+    assert torch.isfinite(out1.float()).all()
+    assert total <= 3e-2 and worst_token <= 4.5e-2
+    assert ta.fused_moe(traits, args) == 0.0
+    torch.cuda.synchronize()
+    assert torch.equal(out1.view(torch.uint16), buf.out.view(torch.uint16))
