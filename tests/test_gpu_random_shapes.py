@@ -71,3 +71,24 @@ def test_random_shapes(dtype):
         if dtype == "fp8" and cfg.tokens * cfg.topk < 16:
             cfg = cfg.scaled(tokens=max(cfg.tokens, 16 // cfg.topk + 1))
         check(cfg, seed=1000 + case, mask=mask, **kw)
+
+
+def test_random_shapes_fp16():
+    from tests.test_gpu_fused_moe import check_fp16
+    rng = np.random.default_rng(404)
+    for case in range(12):
+        cfg = (draw_many_rows if case % 4 == 3 else draw)(rng, "fp16")
+        kw = {0: {}, 1: {"unfused": True}, 2: {"activation": 0}, 3: {"gate_only": 1}}[int(rng.integers(0, 4))]
+        check_fp16(cfg, seed=3000 + case, **kw)
+
+
+@pytest.mark.parametrize("fq", [1, 2])
+def test_random_shapes_int8_fused_quant(fq):
+    """Re-quantised intermediate activations over random shapes and sort units (all three down-GEMM kernels)."""
+    from tests.test_gpu_fused_quant import run
+    rng = np.random.default_rng(500 + fq)
+    for case in range(12):
+        cfg = (draw_many_rows if case % 3 == 2 else draw)(rng, "int8")
+        # the row-wise int8 rounding of Y needs a few hundred values per row and a few rows for a stable rel-L2
+        cfg = cfg.scaled(inter=max(cfg.inter, 128), tokens=max(cfg.tokens, 16 // cfg.topk + 1))
+        run(cfg, fq, seed=4000 + case)
