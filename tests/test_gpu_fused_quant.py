@@ -22,8 +22,9 @@ pytestmark = pytest.mark.gpu
 TOL = 3e-2
 
 
-def reference(cfg, inp, fq, sm_y, a_q, a_scale):
+def reference(cfg, inp, fq, sm_y, a_q, a_scale, mask=None):
     T, K, H, I, E = cfg.tokens, cfg.topk, cfg.hidden, cfg.inter, cfg.experts
+    assert mask is None or fq == 2
     d = inp["d"].astype(np.float32) * inp["d_scale"][:, :, None]
     if fq == 1:
         d = d * sm_y[:, None, :]
@@ -40,16 +41,20 @@ def reference(cfg, inp, fq, sm_y, a_q, a_scale):
         for k in range(K):  # slot order
             acc += part[k * T:(k + 1) * T, 0]
         return oracle.bf16_to_f32(oracle.f32_to_bf16(acc))
-    s = oracle.moe_sorting(inp["topk_ids"], inp["topk_weight"], E, cfg.unit)
-    o = oracle.fused_moe(a_q, oracle.DT_I8, inp["g"], oracle.DT_I8, d, oracle.DT_F32, *s, cfg.unit, T, E, H, I, K,
-                         a_scale=a_scale, g_scale=inp["g_scale"])
+    s = oracle.moe_sorting(inp["topk_ids"], inp["topk_weight"], E, cfg.unit, local_expert_mask=mask)
+    o = oracle.fused_moe(a_q, oracle.DT_I8, inp["g"], oracle.DT_I8, d, oracle.DT_F32, *s, cfg.unit, T, inp["g"].shape[0], H, I,
+                         K, a_scale=a_scale, g_scale=inp["g_scale"])
     return oracle.bf16_to_f32(o)
 
 
-def run(cfg, fq, seed=0):
+def run(cfg, fq, seed=0, mask=None):
     from tests.gpu_util import dev, rel_l2
-    print(f"fused_quant={fq} {cfg} seed={seed}", flush=True)
+    print(f"fused_quant={fq} {cfg} seed={seed} mask={mask is not None}", flush=True)
     inp = mi.make_inputs_np(cfg, seed)
+    if mask is not None:  # weights of the local experts only, indexed by local id
+        nloc = int(mask.sum())
+        for k in ("g", "d", "g_scale", "d_scale"):
+            inp[k] = inp[k][:nloc]
     rng = np.random.Generator(np.random.Philox(seed + 77))
     T, K, H, I, E = cfg.tokens, cfg.topk, cfg.hidden, cfg.inter, cfg.experts
     sm_y = None
@@ -60,15 +65,17 @@ def run(cfg, fq, seed=0):
         a_q, a_scale = oracle.smoothquant(x, sm_x, inp["topk_ids"], oracle.DT_I8)  # [K, T, H], [K, T]
     else:
         a_q, a_scale = inp["a"], inp["a_scale"]
-    ref = reference(cfg, inp, fq, sm_y, a_q, a_scale)
+    ref = reference(cfg, inp, fq, sm_y, a_q, a_scale, mask)
 
-    traits = ta.fused_moe_traits(prec_i="int8", prec_w="int8", block_m=cfg.unit, fused_quant=fq)
+    traits = ta.fused_moe_traits(prec_i="int8", prec_w="int8", block_m=cfg.unit, fused_quant=fq,
+                                 local_expert_masking=mask is not None)
     buf = ta.MoeBuffers(traits, T, E, K, H, I, "cuda")
     buf.ws.fill_(0x5A)  # a dirty workspace
     a_dev = dev(a_q).view(torch.int8)
     args = ta.make_args(traits, buf, a_dev.reshape(-1, H)[:T], dev(inp["g"]).view(torch.int8), dev(inp["d"]).view(torch.int8),
                         dev(inp["topk_ids"]), dev(inp["topk_weight"]), a_scale=dev(a_scale), g_scale=dev(inp["g_scale"]),
-                        d_scale=dev(inp["d_scale"]))
+                        d_scale=dev(inp["d_scale"]), local_expert_mask=None if mask is None else dev(mask.astype(np.int32)),
+                        num_experts=E)
     args.a_ptr = a_dev.data_ptr()
     keep = None
     if fq == 1:
@@ -99,7 +106,15 @@ def test_fused_quant_matches_dequantised_reference(cfg, fq):
     run(cfg, fq)
 
 
-def test_fused_quant_is_deterministic_and_differs_from_plain_int8():
+def test_fused_quant_with_local_expert_mask():
+    """A rank that owns some of the experts: the sort renumbers them, the re-quantisation pass and the down GEMM see
+    local ids, slots of foreign experts drop out."""
+    mask = np.array([1, 0, 1, 1, 0, 1, 0, 1], dtype=np.int32)
+    run(SHAPES[1], 2, mask=mask)
+    run(SHAPES[2], 2, mask=mask)
+
+
+def test_fused_quant_is_deterministic():
     cfg = SHAPES[2]
     a = run(cfg, 2)
     b = run(cfg, 2)
