@@ -7,10 +7,14 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("name,scale", [("cfg4_decode_int8_t64", dict(hidden=1024, inter=512)),
-                                        ("cfg1_cpu_ref_bf16", {}),
-                                        ("cfg3_dsv3_fp8", dict(tokens=2048, hidden=512, inter=256, experts=8))])
-def test_capture_and_replay(name, scale):
+@pytest.mark.parametrize("name,scale,fused_quant", [
+    ("cfg4_decode_int8_t64", dict(hidden=1024, inter=512), 0),
+    ("cfg1_cpu_ref_bf16", {}, 0),
+    ("cfg3_dsv3_fp8", dict(tokens=2048, hidden=512, inter=256, experts=8), 0),
+    # with the re-quantisation pass between the GEMMs (decode kernel / large-tile kernel)
+    ("cfg4_decode_int8_t64", dict(hidden=1024, inter=512), 2),
+    ("cfg4_decode_int8_t64", dict(tokens=2048, hidden=512, inter=256, experts=8), 2)])
+def test_capture_and_replay(name, scale, fused_quant):
     import torch
 
     import therock_amd as ta
@@ -19,7 +23,7 @@ def test_capture_and_replay(name, scale):
     cfg = mi.CONFIGS[name].scaled(**scale) if scale else mi.CONFIGS[name]
     dev = torch.device("cuda:0")
     inp = mi.make_inputs_torch(cfg, dev, 0)
-    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit)
+    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit, fused_quant=fused_quant)
     buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, dev)
     args = ta.make_args(traits, buf, inp["a"], inp["g"], inp["d"], inp["topk_ids"], inp["topk_weight"],
                         a_scale=inp["a_scale"], g_scale=inp["g_scale"], d_scale=inp["d_scale"])
