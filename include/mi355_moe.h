@@ -321,7 +321,7 @@ typedef struct mi355_moe_flatmm_args
     const void* p_max_token_id;          /* [1] int32: rows after padding (p_total_tokens_post_pad) */
     const void* a_ptr;    /* gate+up: [NumTokens, stride_A]; down: [NumTokens * TopK, stride_A] */
     const void* b_ptr;    /* [NumExperts, N, K], K contiguous (stride_B = K) */
-    void* c_ptr;          /* bf16; gate+up: [NumTokens * TopK, stride_C] (N/2 columns); down: [NumTokens, stride_C] */
+    void* c_ptr;          /* bf16 (fp16 with fp16 operands); gate+up: [NumTokens * TopK, stride_C] (N/2 columns); down: [NumTokens, stride_C] */
     int32_t NumTokens;
     int32_t NumExperts;
     int32_t TopK;
@@ -337,8 +337,8 @@ typedef struct mi355_moe_flatmm_args
     const void* scale_m;  /* fp32 per row of A, or NULL (ScaleM) */
     const void* scale_n;  /* fp32 [NumExperts, N], or NULL (ScaleN) */
     const void* exp_bias; /* fp32 [NumExperts, N] added to the scaled dot products, or NULL (ExpertBias) */
-    int32_t prec_a;       /* mi355_moe_dtype of A: BF16, FP8 (with FP8 weights), or INT8 for the gate+up GEMM with int8 weights */
-    int32_t prec_b;       /* mi355_moe_dtype of B: BF16 | FP8 | INT8 */
+    int32_t prec_a;       /* mi355_moe_dtype of A: BF16, FP16 (with FP16 weights), FP8 (with FP8 weights), or INT8 for the gate+up GEMM with int8 weights */
+    int32_t prec_b;       /* mi355_moe_dtype of B: BF16 | FP16 | FP8 | INT8 */
     int32_t block_m;      /* unit_size the sort was run with */
     int32_t activation;   /* mi355_moe_flatmm_activation (gate GEMMs) */
     float swiglu_alpha;   /* 1.702 in ck_tile's default */

@@ -15,7 +15,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
-DT_F32, DT_BF16, DT_E4M3, DT_I8 = 0, 1, 2, 3
+DT_F32, DT_BF16, DT_E4M3, DT_I8, DT_F16 = 0, 1, 2, 3, 4
 _NP_OF_DT = {DT_F32: np.float32, DT_BF16: np.uint16, DT_E4M3: np.uint8, DT_I8: np.int8}
 
 
@@ -139,6 +139,8 @@ def to_f32(x: np.ndarray, dt: int) -> np.ndarray:
         return bf16_to_f32(x)
     if dt == DT_E4M3:
         return e4m3_to_f32(x)
+    if dt == DT_F16:
+        return np.ascontiguousarray(x, dtype=np.uint16).view(np.float16).astype(np.float32)
     return np.asarray(x, dtype=np.int8).astype(np.float32)
 
 
@@ -265,21 +267,22 @@ def moe_act(act, gate, linear, alpha=1.702, limit=7.0):
 
 def moe_gemm(kind, sorted_ids, sorted_eid, sorted_w, post_pad, block_m, a, b, c, num_tokens, topk,
              scale_a=None, scale_b=None, exp_bias=None, act=ACT_SILU, alpha=1.702, limit=7.0, n_padded_zeros=0,
-             k_padded_zeros=0):
+             k_padded_zeros=0, c_dtype=DT_BF16):
     """Oracle of ck_tile's unfused MoE GEMMs (kind 0 = gate only, 1 = gate+up with act(gate, up), 2 = down with
-    weights, added to c).  a, b fp32; c bf16 bits [rows, >= N or N/2], updated in place and returned."""
+    weights, added to c).  a, b fp32; c bf16 bits (fp16 bits with c_dtype=DT_F16) [rows, >= N or N/2], updated in
+    place and returned."""
     a, b = _c(a, np.float32), _c(b, np.float32)
     c = np.ascontiguousarray(c, dtype=np.uint16)
     E, N, K = b.shape
     ids, eid = _c(sorted_ids, np.int32), _c(sorted_eid, np.int32)
     w = _c(sorted_w, np.float32)
-    f = lib().moe_oracle_moe_gemm
+    f = lib().moe_oracle_moe_gemm_dt
     f.restype = C.c_int
     rc = f(C.c_int(kind), _p(ids), _p(eid), _p(w), C.c_int32(int(post_pad)), C.c_int32(block_m), _p(a), _p(b), _p(c),
            C.c_int32(num_tokens), C.c_int32(topk), C.c_int32(N), C.c_int32(K), C.c_int32(a.shape[1]),
            C.c_int32(c.shape[1]), _p(_c(scale_a, np.float32)), _p(_c(scale_b, np.float32)),
            _p(_c(exp_bias, np.float32)), C.c_int32(act), C.c_float(alpha), C.c_float(limit), C.c_int32(n_padded_zeros),
-           C.c_int32(k_padded_zeros))
+           C.c_int32(k_padded_zeros), C.c_int32(c_dtype))
     if rc != 0:
         raise ValueError(f"moe_oracle_moe_gemm failed ({rc})")
     return c

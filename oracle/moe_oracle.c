@@ -54,7 +54,8 @@ enum
     MOE_DT_F32  = 0,
     MOE_DT_BF16 = 1,
     MOE_DT_E4M3 = 2,
-    MOE_DT_I8   = 3
+    MOE_DT_I8   = 3,
+    MOE_DT_F16  = 4
 };
 
 /* ------------------------------------------------------------------ scalar conversions */
@@ -82,6 +83,40 @@ ORACLE_API uint16_t moe_oracle_f32_to_bf16(float f)
         return (uint16_t)((u >> 16) | 0x40u);
     u += 0x7fffu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
+}
+
+/* IEEE binary16 (ck_tile::half_t = _Float16, core/numeric/half.hpp): every value is an fp32 value */
+ORACLE_API float moe_oracle_f16_to_f32(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h >> 15) << 31, ex = (h >> 10) & 0x1fu, man = h & 0x3ffu;
+    float r;
+    if(ex == 0x1f)
+        return bits_to_f32(sign | 0x7f800000u | (man << 13)); /* infinity, or NaN with its payload */
+    r = ex == 0 ? ldexpf((float)man, -24) : ldexpf(1.0f + (float)man / 1024.0f, (int)ex - 15);
+    return sign ? -r : r;
+}
+
+/* round to nearest even, overflow to infinity, subnormals kept (the _Float16 cast of the compiler) */
+ORACLE_API uint16_t moe_oracle_f32_to_f16(float f)
+{
+    const uint32_t u = f32_to_bits(f), sign = (u >> 16) & 0x8000u, mag = u & 0x7fffffffu;
+    if(mag > 0x7f800000u)
+        return (uint16_t)(sign | 0x7e00u); /* quiet NaN */
+    if(mag >= 0x477ff000u) /* 65520 = halfway between the largest finite value and 2^16: rounds to infinity */
+        return (uint16_t)(sign | 0x7c00u);
+    if(mag < 0x33000001u) /* at most 2^-25: rounds to zero (2^-25 itself is a tie with the even code 0) */
+        return (uint16_t)sign;
+    {
+        const int e      = (int)(mag >> 23) - 127;                 /* unbiased exponent, -25 .. 15 */
+        const uint32_t m = (mag & 0x7fffffu) | 0x800000u;          /* 24-bit significand */
+        const int shift  = e >= -14 ? 13 : 13 + (-14 - e);         /* bits dropped (subnormal results drop more) */
+        uint32_t q       = m >> shift;
+        const uint32_t rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+        if(rem > half || (rem == half && (q & 1u)))
+            q++;
+        /* normal: q has the hidden bit at 2^10, adding the exponent field carries correctly when q = 2^11 */
+        return (uint16_t)(sign | (e >= -14 ? (((uint32_t)(e + 14) << 10) + q) : q));
+    }
 }
 
 /* OCP e4m3 ("e4m3fn"): bias 7, no inf, 0x7f/0xff = NaN, max finite 448 */
@@ -496,7 +531,8 @@ ORACLE_API int moe_oracle_fused_moe(const void* a, int a_dt, const float* a_scal
  * n_padded_zeros / k_padded_zeros (MoeFlatmmHostArgs, moe_flatmm_kernel.hpp:29-30): the last rows of every
  * expert's B, respectively the last columns of A and B, are padding that the device kernel never fetches (its
  * tensor views end before them, :600-606): they count as zeros.
- * A and B are fp32 (the caller up-converts), C is bf16 bits. */
+ * A and B are fp32 (the caller up-converts), C holds bf16 bits, or fp16 bits with c_dt = MOE_DT_F16
+ * (moe_oracle_moe_gemm_dt; ck_tile's MoeFlatmm is instantiated for both, CDataType of its kernel). */
 static inline float moe_act_f32(int act, float gate, float linear, float alpha, float limit)
 {
     if(act == 0)
@@ -511,14 +547,20 @@ ORACLE_API float moe_oracle_moe_act(int act, float gate, float linear, float alp
     return moe_act_f32(act, gate, linear, alpha, limit);
 }
 
-ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const int32_t* sorted_eid, const float* sorted_w,
-                                   int32_t max_token_id, int32_t tokens_per_block, const float* A, const float* B,
-                                   uint16_t* C, int32_t num_tokens, int32_t topk, int32_t N, int32_t K, int32_t stride_a,
-                                   int32_t stride_c, const float* scale_a, const float* scale_b, const float* exp_bias,
-                                   int32_t act, float alpha, float limit, int32_t n_padded_zeros, int32_t k_padded_zeros)
+static inline uint16_t c_from_f32(int32_t c_dt, float f)
+{
+    return c_dt == MOE_DT_F16 ? moe_oracle_f32_to_f16(f) : moe_oracle_f32_to_bf16(f);
+}
+
+ORACLE_API int moe_oracle_moe_gemm_dt(int kind, const int32_t* sorted_ids, const int32_t* sorted_eid, const float* sorted_w,
+                                      int32_t max_token_id, int32_t tokens_per_block, const float* A, const float* B,
+                                      uint16_t* C, int32_t num_tokens, int32_t topk, int32_t N, int32_t K, int32_t stride_a,
+                                      int32_t stride_c, const float* scale_a, const float* scale_b, const float* exp_bias,
+                                      int32_t act, float alpha, float limit, int32_t n_padded_zeros, int32_t k_padded_zeros,
+                                      int32_t c_dt)
 {
     if(kind < 0 || kind > 2 || act < 0 || act > 1 || n_padded_zeros < 0 || n_padded_zeros > N || k_padded_zeros < 0 ||
-       k_padded_zeros > K)
+       k_padded_zeros > K || (c_dt != MOE_DT_BF16 && c_dt != MOE_DT_F16))
         return -1;
     const int32_t pn = kind == 1 ? N / 2 : N;
     const int32_t nv = N - n_padded_zeros; /* rows of B that exist */
@@ -531,7 +573,8 @@ ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const in
             return -2;
         for(int64_t t = 0; t < num_tokens; t++)
             for(int64_t n = 0; n < N; n++)
-                acc2[t * N + n] = moe_oracle_bf16_to_f32(C[t * stride_c + n]);
+                acc2[t * N + n] = c_dt == MOE_DT_F16 ? moe_oracle_f16_to_f32(C[t * stride_c + n])
+                                                     : moe_oracle_bf16_to_f32(C[t * stride_c + n]);
     }
     /* slot order inside a token = the order of the reference's reduction: walk slots, then rows */
     for(int32_t s = 0; s < (kind == 2 ? topk : 1); s++)
@@ -565,10 +608,10 @@ ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const in
                             up += a[k] * bu[k];
                     up *= sa * (scale_b ? scale_b[e * N + n + pn] : 1.0f);
                     up += exp_bias ? exp_bias[e * N + n + pn] : 0.f;
-                    C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(moe_act_f32(act, acc, up, alpha, limit));
+                    C[c_row * stride_c + n] = c_from_f32(c_dt, moe_act_f32(act, acc, up, alpha, limit));
                 }
                 else if(kind == 0)
-                    C[c_row * stride_c + n] = moe_oracle_f32_to_bf16(moe_act_f32(act, acc, 1.0f, alpha, limit));
+                    C[c_row * stride_c + n] = c_from_f32(c_dt, moe_act_f32(act, acc, 1.0f, alpha, limit));
                 else
                     acc2[c_row * N + n] += acc * sorted_w[r];
             }
@@ -577,10 +620,21 @@ ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const in
     {
         for(int64_t t = 0; t < num_tokens; t++)
             for(int64_t n = 0; n < N; n++)
-                C[t * stride_c + n] = moe_oracle_f32_to_bf16(acc2[t * N + n]);
+                C[t * stride_c + n] = c_from_f32(c_dt, acc2[t * N + n]);
         free(acc2);
     }
     return 0;
+}
+
+ORACLE_API int moe_oracle_moe_gemm(int kind, const int32_t* sorted_ids, const int32_t* sorted_eid, const float* sorted_w,
+                                   int32_t max_token_id, int32_t tokens_per_block, const float* A, const float* B,
+                                   uint16_t* C, int32_t num_tokens, int32_t topk, int32_t N, int32_t K, int32_t stride_a,
+                                   int32_t stride_c, const float* scale_a, const float* scale_b, const float* exp_bias,
+                                   int32_t act, float alpha, float limit, int32_t n_padded_zeros, int32_t k_padded_zeros)
+{
+    return moe_oracle_moe_gemm_dt(kind, sorted_ids, sorted_eid, sorted_w, max_token_id, tokens_per_block, A, B, C, num_tokens,
+                                  topk, N, K, stride_a, stride_c, scale_a, scale_b, exp_bias, act, alpha, limit,
+                                  n_padded_zeros, k_padded_zeros, MOE_DT_BF16);
 }
 
 /* ------------------------------------------------------------------------------ router

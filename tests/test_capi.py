@@ -114,6 +114,26 @@ def test_static_workspace_entry_point_rejects_oversized_problems_on_the_host():
         assert 0 < lib.mi355_fused_moe_workspace_size(C.byref(t8), tokens, 128, 8, 4096, 1536) <= cap
 
 
+def test_flatmm_operand_types_on_the_host():
+    """Which operand pairs the stand-alone GEMMs take (decided on the host, before any launch): equal 16-bit or
+    8-bit types, and bf16 activations with int8 weights for the down GEMM only."""
+    lib = _lib.load()
+    D = _lib.DTYPES
+
+    def ws(kind, pa, pb):
+        a = _lib.FlatmmArgs()
+        a.NumTokens, a.NumExperts, a.TopK, a.N, a.K, a.block_m, a.k_batch = 64, 4, 2, 256, 128, 32, 1
+        a.prec_a, a.prec_b = D[pa], D[pb]
+        return lib.mi355_moe_flatmm_workspace_size(kind, C.byref(a))
+
+    for kind in (0, 1, 2):
+        for p in ("bf16", "fp16", "fp8"):
+            assert ws(kind, p, p) > 0, (kind, p)
+        assert ws(kind, "bf16", "fp16") == 0 and ws(kind, "fp16", "bf16") == 0 and ws(kind, "fp16", "int8") == 0
+        assert b"operand types" in lib.mi355_moe_last_error()
+    assert ws(1, "int8", "int8") > 0 and ws(2, "bf16", "int8") > 0 and ws(2, "int8", "int8") == 0
+
+
 def test_host_only_entry_points():
     lib = _lib.load()
     assert lib.mi355_moe_version() == 200

@@ -21,15 +21,23 @@ def _rel(a, b):
 SHAPES = [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (130, 6, 2, 1152, 256, 64), (1024, 4, 2, 512, 384, 32)]
 
 
+def _c_types(kind):
+    """C's torch dtype, the oracle's code for it and the rel-L2 tolerance: fp16 operands give an fp16 C."""
+    import torch
+    if kind == "fp16":
+        return torch.float16, oracle.DT_F16, 2e-3
+    return torch.bfloat16, oracle.DT_BF16, (1e-2 if kind == "bf16" else 3e-2)
+
+
 @pytest.mark.parametrize("T,E,K,H,I,unit", SHAPES)
-@pytest.mark.parametrize("kind", ["bf16", "int8", "fp8"])
+@pytest.mark.parametrize("kind", ["bf16", "fp16", "int8", "fp8"])
 def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     import torch
     import therock_amd as ta
     from tests.gpu_util import run_sorting
 
     rng = np.random.default_rng(T + H)
-    tol = 1e-2 if kind == "bf16" else 3e-2
+    cdt, odt, tol = _c_types(kind)
     ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
     w = rng.random((T, K), dtype=np.float32)
     s_ids, s_w, s_eid, total = run_sorting(ids, w, E, unit, fill=True)
@@ -37,12 +45,12 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     ref_sort = oracle.moe_sorting(ids, w, E, unit)
     assert pp == ref_sort[3]
     dev = lambda a: torch.from_numpy(a).cuda()
-    bf = lambda a: torch.from_numpy(a).cuda().to(torch.bfloat16)
+    bf = lambda a: torch.from_numpy(a).cuda().to(cdt)
     x32 = rng.standard_normal((T, H)).astype(np.float32)
     g32 = (rng.standard_normal((E, 2 * I, H)) * 0.05).astype(np.float32)
     d32 = (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32)
     d_ids, d_w, d_eid, d_tot = dev(s_ids), dev(s_w), dev(s_eid), dev(total.astype(np.int32))
-    if kind == "bf16":
+    if kind in ("bf16", "fp16"):
         x, g, d = bf(x32), bf(g32), bf(d32)
         xr, gr, dr = x.float().cpu().numpy(), g.float().cpu().numpy(), d.float().cpu().numpy()
         sa = sg = sd = None
@@ -60,45 +68,47 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
         d_sa, d_sg, d_sd = dev(sa), dev(sg), dev(sd)
 
     # gate+up: every (token, slot) row written exactly, nothing else touched
-    y = torch.full((T * K + 3, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    y = torch.full((T * K + 3, I), float("nan"), dtype=cdt, device="cuda")
     assert ta.moe_flatmm(ta.GEMM1_GATE_UP, x, g, y, d_ids, d_eid, d_tot, T, K, unit, scale_m=d_sa, scale_n=d_sg) == 0.0
     torch.cuda.synchronize()
-    y_ref = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, xr, gr, np.zeros((T * K, I), np.uint16), T, K, sa, sg)
+    y_ref = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, xr, gr, np.zeros((T * K, I), np.uint16), T, K, sa, sg,
+                            c_dtype=odt)
     yg = y.float().cpu().numpy()
     assert np.isnan(yg[T * K:]).all() and not np.isnan(yg[:T * K]).any()
-    assert _rel(yg[:T * K], oracle.to_f32(y_ref, oracle.DT_BF16)) <= tol
+    assert _rel(yg[:T * K], oracle.to_f32(y_ref, odt)) <= tol
 
     # gate only: the gate half of the same weights on their own, c = silu(a b^T)
     g_only = g[:, :I].contiguous()
-    yo = torch.full((T * K + 3, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    yo = torch.full((T * K + 3, I), float("nan"), dtype=cdt, device="cuda")
     assert ta.moe_flatmm(ta.GEMM1_GATE_ONLY, x, g_only, yo, d_ids, d_eid, d_tot, T, K, unit, scale_m=d_sa,
                          scale_n=None if d_sg is None else d_sg[:, :I].contiguous()) == 0.0
     torch.cuda.synchronize()
     yo_ref = oracle.moe_gemm(0, s_ids, s_eid, s_w, pp, unit, xr, np.ascontiguousarray(gr[:, :I]),
-                             np.zeros((T * K, I), np.uint16), T, K, sa, None if sg is None else np.ascontiguousarray(sg[:, :I]))
+                             np.zeros((T * K, I), np.uint16), T, K, sa, None if sg is None else np.ascontiguousarray(sg[:, :I]),
+                             c_dtype=odt)
     yog = yo.float().cpu().numpy()
     assert np.isnan(yog[T * K:]).all() and not np.isnan(yog[:T * K]).any()
-    assert _rel(yog[:T * K], oracle.to_f32(yo_ref, oracle.DT_BF16)) <= tol
+    assert _rel(yog[:T * K], oracle.to_f32(yo_ref, odt)) <= tol
 
-    # down: added to what c holds; a takes the reference's bf16 Y so that the two GEMMs are checked apart
+    # down: added to what c holds; a takes the reference's 16-bit Y so that the two GEMMs are checked apart
     # (fp8: that Y quantised per row, the row scales going in as scale_m)
-    y_f32 = oracle.to_f32(y_ref, oracle.DT_BF16)
+    y_f32 = oracle.to_f32(y_ref, odt)
     if kind == "fp8":
         yq, sy = oracle.rowwise_quant(y_f32, oracle.DT_E4M3)
         y_in, a_ref, s_m, d_sm = dev(yq), oracle.to_f32(yq, oracle.DT_E4M3), sy, dev(sy)
     else:
-        y_in, a_ref, s_m, d_sm = torch.from_numpy(y_ref.view(np.int16)).cuda().view(torch.bfloat16), y_f32, None, None
+        y_in, a_ref, s_m, d_sm = torch.from_numpy(y_ref.view(np.int16)).cuda().view(cdt), y_f32, None, None
     c0 = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
     c = bf(c0)
-    c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, a_ref, dr, _bits(c).copy(), T, K, s_m, sd)
+    c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, a_ref, dr, _bits(c).copy(), T, K, s_m, sd, c_dtype=odt)
     assert ta.moe_flatmm(ta.GEMM2, y_in, d, c, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w, scale_m=d_sm,
                          scale_n=d_sd) == 0.0
     torch.cuda.synchronize()
-    assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, oracle.DT_BF16)) <= tol
+    assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, odt)) <= tol
 
 
 @pytest.mark.parametrize("T,E,K,H,I,unit", [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (1024, 4, 2, 512, 384, 32)])
-@pytest.mark.parametrize("kind", ["bf16", "int8", "fp8"])
+@pytest.mark.parametrize("kind", ["bf16", "fp16", "int8", "fp8"])
 @pytest.mark.parametrize("act,with_bias", [("silu", True), ("swiglu", False), ("swiglu", True)])  # (silu, no bias) is the test above
 def test_bias_and_swiglu(T, E, K, H, I, unit, kind, act, with_bias):
     """Expert bias and ck_tile's clamped SwiGLU (moe::Swiglu{alpha, limit}) on all three GEMM kinds, every kernel
@@ -108,20 +118,20 @@ def test_bias_and_swiglu(T, E, K, H, I, unit, kind, act, with_bias):
     from tests.gpu_util import run_sorting
 
     rng = np.random.default_rng(T + H + with_bias)
-    tol = 1e-2 if kind == "bf16" else 3e-2
+    cdt, odt, tol = _c_types(kind)
     ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
     w = rng.random((T, K), dtype=np.float32)
     s_ids, s_w, s_eid, total = run_sorting(ids, w, E, unit, fill=True)
     pp = int(total[0])
     dev = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    bf = lambda a: torch.from_numpy(a).cuda().to(torch.bfloat16)
+    bf = lambda a: torch.from_numpy(a).cuda().to(cdt)
     x32 = (rng.standard_normal((T, H)) * 2).astype(np.float32)
     g32 = (rng.standard_normal((E, 2 * I, H)) * 0.1).astype(np.float32)   # gate / up values reach past the limit
     d32 = (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32)
     bias_g = (rng.standard_normal((E, 2 * I)) * 1.5).astype(np.float32) if with_bias else None
     bias_d = (rng.standard_normal((E, H)) * 0.5).astype(np.float32) if with_bias else None
     d_ids, d_w, d_eid, d_tot = dev(s_ids), dev(s_w), dev(s_eid), dev(total.astype(np.int32))
-    if kind == "bf16":
+    if kind in ("bf16", "fp16"):
         x, g, d = bf(x32), bf(g32), bf(d32)
         xr, gr, dr = x.float().cpu().numpy(), g.float().cpu().numpy(), d.float().cpu().numpy()
         sa = sg = sd = None
@@ -139,42 +149,43 @@ def test_bias_and_swiglu(T, E, K, H, I, unit, kind, act, with_bias):
     o_code = oracle.ACT_SWIGLU if act == "swiglu" else oracle.ACT_SILU
     alpha, limit = 1.702, 7.0
 
-    y = torch.full((T * K, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    y = torch.full((T * K, I), float("nan"), dtype=cdt, device="cuda")
     assert ta.moe_flatmm(ta.GEMM1_GATE_UP, x, g, y, d_ids, d_eid, d_tot, T, K, unit, scale_m=dev(sa), scale_n=dev(sg),
                          exp_bias=dev(bias_g), activation=a_code, swiglu_alpha=alpha, swiglu_limit=limit) == 0.0
     torch.cuda.synchronize()
     y_ref = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, xr, gr, np.zeros((T * K, I), np.uint16), T, K, sa, sg,
-                            exp_bias=bias_g, act=o_code, alpha=alpha, limit=limit)
+                            exp_bias=bias_g, act=o_code, alpha=alpha, limit=limit, c_dtype=odt)
     yg = y.float().cpu().numpy()
     assert not np.isnan(yg).any()
-    assert _rel(yg, oracle.to_f32(y_ref, oracle.DT_BF16)) <= tol
+    assert _rel(yg, oracle.to_f32(y_ref, odt)) <= tol
 
     g_only = g[:, :I].contiguous()
     b_only = None if bias_g is None else np.ascontiguousarray(bias_g[:, :I])
     s_only = None if sg is None else np.ascontiguousarray(sg[:, :I])
-    yo = torch.full((T * K, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    yo = torch.full((T * K, I), float("nan"), dtype=cdt, device="cuda")
     assert ta.moe_flatmm(ta.GEMM1_GATE_ONLY, x, g_only, yo, d_ids, d_eid, d_tot, T, K, unit, scale_m=dev(sa), scale_n=dev(s_only),
                          exp_bias=dev(b_only), activation=a_code, swiglu_alpha=alpha, swiglu_limit=limit) == 0.0
     torch.cuda.synchronize()
     yo_ref = oracle.moe_gemm(0, s_ids, s_eid, s_w, pp, unit, xr, np.ascontiguousarray(gr[:, :I]),
                              np.zeros((T * K, I), np.uint16), T, K, sa, s_only, exp_bias=b_only, act=o_code, alpha=alpha,
-                             limit=limit)
-    assert _rel(yo.float().cpu().numpy(), oracle.to_f32(yo_ref, oracle.DT_BF16)) <= tol
+                             limit=limit, c_dtype=odt)
+    assert _rel(yo.float().cpu().numpy(), oracle.to_f32(yo_ref, odt)) <= tol
 
     if not with_bias:
         return  # the down GEMM has no activation
-    y_f32 = oracle.to_f32(y_ref, oracle.DT_BF16)
+    y_f32 = oracle.to_f32(y_ref, odt)
     if kind == "fp8":
         yq, sy = oracle.rowwise_quant(y_f32, oracle.DT_E4M3)
         y_in, a_ref, s_m = dev(yq), oracle.to_f32(yq, oracle.DT_E4M3), sy
     else:
-        y_in, a_ref, s_m = torch.from_numpy(y_ref.view(np.int16)).cuda().view(torch.bfloat16), y_f32, None
+        y_in, a_ref, s_m = torch.from_numpy(y_ref.view(np.int16)).cuda().view(cdt), y_f32, None
     c = bf((rng.standard_normal((T, H)) * 0.1).astype(np.float32))
-    c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, a_ref, dr, _bits(c).copy(), T, K, s_m, sd, exp_bias=bias_d)
+    c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, a_ref, dr, _bits(c).copy(), T, K, s_m, sd, exp_bias=bias_d,
+                            c_dtype=odt)
     assert ta.moe_flatmm(ta.GEMM2, y_in, d, c, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w, scale_m=dev(s_m),
                          scale_n=dev(sd), exp_bias=dev(bias_d)) == 0.0
     torch.cuda.synchronize()
-    assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, oracle.DT_BF16)) <= tol
+    assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, odt)) <= tol
 
 
 @pytest.mark.parametrize("T,E,K,H,I,unit", [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (1024, 4, 2, 512, 384, 32)])

@@ -71,6 +71,39 @@ def test_bf16_rne_all_upper_halves_and_tie_patterns():
     assert oracle.lib().moe_oracle_f32_to_bf16(1.005859375) == 0x3F81  # tie rounds to even -> 1.0078125
 
 
+def test_f16_conversions_match_ieee_binary16():
+    """Every fp16 code decodes to numpy's float16 value; encoding is checked on every fp16 value, its fp32
+    neighbours, every midpoint between adjacent codes (ties to even) and its neighbours, the overflow and
+    underflow thresholds and random bit patterns, against numpy's IEEE cast."""
+    import ctypes as C
+    l = oracle.lib()
+    l.moe_oracle_f16_to_f32.restype, l.moe_oracle_f16_to_f32.argtypes = C.c_float, [C.c_uint16]
+    l.moe_oracle_f32_to_f16.restype, l.moe_oracle_f32_to_f16.argtypes = C.c_uint16, [C.c_float]
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    ref = bits.view(np.float16).astype(np.float32)
+    got = np.array([l.moe_oracle_f16_to_f32(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(ref)
+    assert np.array_equal(got.view(np.uint32)[~nan], ref.view(np.uint32)[~nan]) and np.isnan(got[nan]).all()
+    fin = ref[np.isfinite(ref)]
+    u = fin.view(np.uint32)
+    srt = np.sort(fin)
+    mid = ((srt[:-1].astype(np.float64) + srt[1:].astype(np.float64)) / 2).astype(np.float32)  # exact in fp32
+    rng = np.random.Generator(np.random.Philox(5))
+    x = np.concatenate([fin, (u + 1).view(np.float32), (u - 1).view(np.float32), mid,
+                        np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf)),
+                        np.array([65504, 65519.996, 65520, 65536, 1e30, np.inf, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0000001,
+                                  2.0 ** -26, 1e-40, 0.0], dtype=np.float32),
+                        rng.integers(0, 1 << 32, 100000, dtype=np.uint64).astype(np.uint32).view(np.float32)])
+    x = np.concatenate([x, -x])
+    x = x[~np.isnan(x)]
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    got = np.array([l.moe_oracle_f32_to_f16(float(v)) for v in x], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    assert l.moe_oracle_f32_to_f16(float("nan")) & 0x7fff > 0x7c00
+    assert l.moe_oracle_f32_to_f16(1.00048828125) == 0x3c00 and l.moe_oracle_f32_to_f16(1.00146484375) == 0x3c02  # ties to even
+
+
 def test_silu_closed_form_and_special_cases():
     l = oracle.lib()
     assert l.moe_oracle_silu(0.0) == 0.0

@@ -47,6 +47,35 @@ def test_against_dense_float64(T, E, K, H, I, unit):
         np.testing.assert_allclose(o[t], ref, rtol=1.2e-2, atol=1e-5)
 
 
+def test_fp16_output_is_the_same_sums_rounded_to_fp16():
+    """c_dtype=DT_F16: the fp32 results before the final rounding are those of the bf16 variant (checked through the
+    dense float64 formulation at fp16's tighter precision), and the down kind starts from the fp16 value c holds."""
+    T, E, K, H, I, unit = 40, 6, 3, 64, 96, 32
+    x, g, d, ids, w, s_ids, s_w, s_eid, pp = _problem(11, T, E, K, H, I, unit)
+    f16 = lambda a: a.astype(np.float16).astype(np.float32)
+    x, g, d = f16(x), f16(g), f16(d)
+    y = oracle.to_f32(oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, x, g, np.zeros((T * K, I), np.uint16), T, K,
+                                      c_dtype=oracle.DT_F16), oracle.DT_F16)
+    for t in range(T):
+        for k in range(K):
+            e = ids[t, k]
+            ref = _silu(x[t].astype(np.float64) @ g[e, :I].T.astype(np.float64)) * (x[t].astype(np.float64) @ g[e, I:].T)
+            np.testing.assert_allclose(y[t * K + k], ref, rtol=1.5e-3, atol=1e-6)  # one fp16 rounding (2^-11) + fp32 sums
+    c0 = np.full((T, H), 0.3, np.float32).astype(np.float16)
+    o = oracle.to_f32(oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, y, d, c0.view(np.uint16).copy(), T, K,
+                                      c_dtype=oracle.DT_F16), oracle.DT_F16)
+    for t in range(T):
+        ref = float(c0[0, 0]) + sum(w[t, k] * (y[t * K + k].astype(np.float64) @ d[ids[t, k]].T.astype(np.float64))
+                                    for k in range(K))
+        np.testing.assert_allclose(o[t], ref, rtol=1.5e-3, atol=2e-5)
+    # the bf16 variant of the same call differs only by the coarser rounding
+    ob = oracle.to_f32(oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, y, d, np.zeros((T, H), np.uint16), T, K), oracle.DT_BF16)
+    of = oracle.to_f32(oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, y, d, np.zeros((T, H), np.uint16), T, K,
+                                       c_dtype=oracle.DT_F16), oracle.DT_F16)
+    assert np.array_equal(oracle.f32_to_bf16(of) , oracle.f32_to_bf16(ob)) or \
+        np.abs(of - ob).max() <= np.abs(ob).max() * 2.0 ** -8
+
+
 def test_composition_matches_fused_oracle():
     T, E, K, H, I, unit = 48, 8, 2, 128, 64, 32
     x, g, d, ids, w, s_ids, s_w, s_eid, pp = _problem(3, T, E, K, H, I, unit)

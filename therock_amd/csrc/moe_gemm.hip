@@ -375,8 +375,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
 #pragma unroll
         for(int i = 0; i < 4; i++)
         {
-            acc[2 * i]     = __uint_as_float(d[i] << 16);
-            acc[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+            acc[2 * i]     = f16 ? f16_bits_to_float(d[i] & 0xffffu) : __uint_as_float(d[i] << 16);
+            acc[2 * i + 1] = f16 ? f16_bits_to_float(d[i] >> 16) : __uint_as_float(d[i] & 0xffff0000u);
         }
     }
     // four slots at a time (eight measured the same): their rows are fetched together (read once: non-temporal), then added in slot order
@@ -798,11 +798,13 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
     const bool go     = kind == MI355_MOE_GEMM1_GATE_ONLY;
     const bool w8     = a.prec_b == MI355_MOE_INT8;
     const bool f8     = a.prec_b == MI355_MOE_FP8;
-    const bool ok_typ = (a.prec_b == MI355_MOE_BF16 && a.prec_a == MI355_MOE_BF16) || (f8 && a.prec_a == MI355_MOE_FP8) ||
-                        (w8 && a.prec_a == (g1 ? MI355_MOE_INT8 : MI355_MOE_BF16));
+    const bool f16    = a.prec_b == MI355_MOE_FP16;
+    const bool ok_typ = (a.prec_b == MI355_MOE_BF16 && a.prec_a == MI355_MOE_BF16) || (f16 && a.prec_a == MI355_MOE_FP16) ||
+                        (f8 && a.prec_a == MI355_MOE_FP8) || (w8 && a.prec_a == (g1 ? MI355_MOE_INT8 : MI355_MOE_BF16));
     if(!ok_typ)
-        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: operand types a=%d b=%d (bf16 x bf16, fp8 x fp8, int8 x int8 for "
-                                             "the gate+up GEMM, bf16 x int8 for the down GEMM)", a.prec_a, a.prec_b);
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: operand types a=%d b=%d (bf16 x bf16, fp16 x fp16, fp8 x fp8, "
+                                             "int8 x int8 for the gate+up GEMM, bf16 x int8 for the down GEMM)", a.prec_a,
+                    a.prec_b);
     if(a.NumTokens < 0 || a.NumExperts <= 0 || a.NumExperts > 1024 || a.TopK <= 0 || a.TopK > 255 || a.N <= 0 || a.K <= 0 ||
        a.block_m < 1 || a.block_m > 1024 || a.k_batch > 1 || (g1 && !go && a.N % 2 != 0))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: bad sizes (tokens=%d experts=%d topk=%d N=%d K=%d block_m=%d k_batch=%d)",
@@ -818,15 +820,16 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: N and K must give hidden and intermediate sizes that are "
                                              "multiples of 32, K of the fp8 down GEMM of 128 (hidden=%d inter=%d)", L.hidden,
                     L.inter);
-    const int prec = w8 ? MI355_MOE_INT8 : f8 ? MI355_MOE_FP8 : MI355_MOE_BF16;
-    L.traits       = mi355_fused_moe_traits{prec, prec, MI355_MOE_BF16, MI355_MOE_FP32, MI355_MOE_FP32, MI355_MOE_FP32,
+    const int prec = w8 ? MI355_MOE_INT8 : f8 ? MI355_MOE_FP8 : f16 ? MI355_MOE_FP16 : MI355_MOE_BF16;
+    L.traits       = mi355_fused_moe_traits{prec, prec, f16 ? MI355_MOE_FP16 : MI355_MOE_BF16, MI355_MOE_FP32, MI355_MOE_FP32, MI355_MOE_FP32,
                                             MI355_MOE_FP32, a.block_m, 1, 0, 0, 0};
     L.mblk         = pick_mblk(L.traits, a.NumTokens, a.TopK, a.NumExperts, L.hidden, L.inter);
     if(a.k_padded_zeros > 0)
     {
         // the K loops of the small-tile and decode kernels stop at any multiple of 16 bytes; the large-tile kernel
         // wants whole 128-byte lines
-        const int a_b = a.prec_a == MI355_MOE_BF16 ? 2 : 1, b_b = a.prec_b == MI355_MOE_BF16 ? 2 : 1;
+        const int a_b = (a.prec_a == MI355_MOE_BF16 || a.prec_a == MI355_MOE_FP16) ? 2 : 1;
+        const int b_b = (a.prec_b == MI355_MOE_BF16 || a.prec_b == MI355_MOE_FP16) ? 2 : 1;
         const int k_eff = a.K - a.k_padded_zeros;
         if((k_eff * a_b) % 16 != 0 || (k_eff * b_b) % 16 != 0 || (f8 && k_eff % 32 != 0))
             return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: K - k_padded_zeros = %d must cover whole 16-byte pieces of A "
@@ -877,7 +880,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     if((w8 || f8) && (!a.scale_n || ((g1 || f8) && !a.scale_m)))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: quantised weights need scale_n, quantised activations scale_m");
     const int T = a.NumTokens, E = a.NumExperts, K = a.TopK, H = L.hidden, I = L.inter;
-    const int a_b = a.prec_a == MI355_MOE_BF16 ? 2 : 1, b_b = (w8 || f8) ? 1 : 2;
+    const int a_b = (a.prec_a == MI355_MOE_BF16 || a.prec_a == MI355_MOE_FP16) ? 2 : 1, b_b = (w8 || f8) ? 1 : 2;
     if(a.stride_A < a.K || a.stride_B != a.K || a.stride_C < (g1 ? I : H) || ((int64_t)a.stride_A * a_b) % 16 != 0 ||
        ((int64_t)a.stride_C * 2) % 16 != 0)
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: strides (A=%d B=%d C=%d): B must be [experts, N, K] with K "
@@ -937,7 +940,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     if(g1)
     {
         p.x_scale       = (w8 || f8) ? static_cast<const float*>(a.scale_m) : nullptr;
-        p.y_bf16        = 1; // C is bf16 whatever the operand type
+        p.y_bf16        = 1; // C is a 16-bit float whatever the operand type (fp16 with fp16 operands, else bf16)
         p.out           = static_cast<unsigned char*>(a.c_ptr);
         p.out_row_bytes = (int64_t)a.stride_C * 2;
         p.gate_only     = go;
@@ -965,7 +968,8 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
         hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + L.p_off, inv,
                            static_cast<const float*>(a.p_sorted_expert_weights), static_cast<unsigned char*>(a.c_ptr), K, H,
                            (int64_t)a.stride_C * 2, 1, f8 ? static_cast<const float*>(a.scale_m) : nullptr,
-                           static_cast<const float*>(a.exp_bias), static_cast<const int*>(a.p_sorted_expert_ids), a.block_m, 0);
+                           static_cast<const float*>(a.exp_bias), static_cast<const int*>(a.p_sorted_expert_ids), a.block_m,
+                           prec == MI355_MOE_FP16 ? 1 : 0);
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;

@@ -239,7 +239,7 @@ def _flatmm_args(kind, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens
     import torch
 
     experts, n, k = b.shape
-    dt = {torch.bfloat16: "bf16", torch.int8: "int8", torch.float8_e4m3fn: "fp8", torch.uint8: "fp8"}
+    dt = {torch.bfloat16: "bf16", torch.float16: "fp16", torch.int8: "int8", torch.float8_e4m3fn: "fp8", torch.uint8: "fp8"}
     return _lib.FlatmmArgs(_ptr(sorted_ids), _ptr(sorted_weights), _ptr(sorted_eid), _ptr(max_token_id), _ptr(a), _ptr(b),
                            _ptr(c), num_tokens, experts, topk, 1, sorted_ids.numel(), n, k, a.stride(0), k, c.stride(0),
                            n_padded_zeros, k_padded_zeros, _ptr(scale_m), _ptr(scale_n), _ptr(exp_bias),
