@@ -125,6 +125,31 @@ def test_decode_kernel_ragged(dtype):
     check(mi.MoeConfig("d", 40, 2080, 640, 64, 8, dtype, "sigmoid_renorm", unit=16), seed=3)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "int8"])
+def test_two_block_decode_tiles(dtype):
+    """28 .. 52 rows per expert with 16-bit or int8 operands: the decode kernel with two 32-row token blocks per
+    tile (64-row tiles).  Ragged K depths and column tails, experts with more than 64 rows (two tiles) and with
+    none, a sort unit that is not a multiple of 32, the expert mask, GELU and gate-only."""
+    import therock_amd as ta
+    chk = check_fp16 if dtype == "fp16" else check
+    for i, (T, H, I, E, K, router, unit) in enumerate(((160, 512, 256, 8, 2, "softmax_renorm", 32),
+                                                      (330, 1056, 288, 16, 2, "sigmoid_renorm", 16),
+                                                      (100, 480, 128, 6, 2, "softmax", 8),
+                                                      (640, 512, 256, 128, 8, "sigmoid_renorm", 32))):
+        cfg = mi.MoeConfig("d2", T, H, I, E, K, dtype, router, unit)
+        traits = ta.fused_moe_traits(prec_i=dtype, prec_w=dtype, prec_o="fp16" if dtype == "fp16" else "bf16", block_m=unit)
+        assert ta.fused_moe_tile_rows(traits, T, E, K, H, I) == 64, cfg
+        chk(cfg, seed=i)
+    cfg = mi.MoeConfig("d2", 160, 512, 256, 8, 2, dtype, "softmax_renorm")
+    chk(cfg, seed=5, activation=0)
+    chk(cfg, seed=6, gate_only=1)
+    if dtype != "fp16":
+        # 240 tokens over the five local experts of eight: about 36 rows each after the foreign slots drop out
+        check(mi.MoeConfig("d2", 144, 512, 256, 8, 2, dtype, "softmax_renorm"), seed=7, mask=np.array([1, 0, 1, 1, 0, 1, 0, 1], dtype=np.int32))
+    # a skewed routing: a few experts with several 64-row tiles, the tail with a handful of rows or none
+    chk(mi.MoeConfig("d2_zipf", 320, 512, 256, 16, 2, dtype, "zipf"), seed=8)
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 def test_many_rows_per_expert_with_small_sort_units(dtype):
     # hundreds of rows per expert, but expert boundaries on multiples of 8 or 24 rows only: the 320-row kernel
@@ -139,10 +164,10 @@ def test_many_rows_per_expert_with_small_sort_units(dtype):
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 def test_large_tile_kernel_partial_tiles(dtype):
-    # from about 28 rows per expert on, and with enough tiles to fill the chip, the 320-row kernel runs with
-    # mostly empty tiles: it then fetches only the 64-row slab groups a tile has (1 to 5 per step)
+    # from about 28 (fp8) or 53 (other types) rows per expert on, and with enough tiles to fill the chip, the 320-row
+    # kernel runs with mostly empty tiles: it then fetches only the 64-row slab groups a tile has (1 to 5 per step)
     import therock_amd as ta
-    for cfg, seed in ((mi.MoeConfig("p", 640, 256, 512, 64, 4, dtype, "softmax_renorm"), 1),
+    for cfg, seed in ((mi.MoeConfig("p", 640 if dtype == "fp8" else 900, 256, 512, 64, 4, dtype, "softmax_renorm"), 1),
                       (mi.MoeConfig("p", 1500, 256, 512, 64, 4, dtype, "zipf"), 2),
                       (mi.MoeConfig("p", 4000, 384, 512, 64, 6, dtype, "zipf", unit=64), 3)):
         traits = ta.fused_moe_traits(prec_i=dtype, prec_w=dtype, block_m=cfg.unit)

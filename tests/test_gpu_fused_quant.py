@@ -91,9 +91,11 @@ def run(cfg, fq, seed=0, mask=None):
     return got
 
 
-# 16 rows per expert: decode kernel; 128: 128-row tiles; 512 / 640: large-tile kernel (I % 128 == 0)
+# 16 rows per expert: decode kernel; 40: decode kernel with two token blocks per tile; 128: 128-row tiles;
+# 512 / 640: large-tile kernel (I % 128 == 0)
 SHAPES = [
     mi.MoeConfig("fq_decode", 64, 256, 256, 8, 2, "int8", "softmax_renorm"),
+    mi.MoeConfig("fq_decode_two_blocks", 160, 512, 256, 8, 2, "int8", "softmax_renorm"),
     mi.MoeConfig("fq_mid", 384, 512, 384, 8, 2, "int8", "softmax_renorm"),
     mi.MoeConfig("fq_big", 2048, 512, 256, 8, 2, "int8", "softmax_renorm"),
     mi.MoeConfig("fq_big_unit64", 640, 256, 1536, 4, 4, "int8", "sigmoid_renorm", 64),
@@ -110,12 +112,12 @@ def test_fused_quant_with_local_expert_mask():
     """A rank that owns some of the experts: the sort renumbers them, the re-quantisation pass and the down GEMM see
     local ids, slots of foreign experts drop out."""
     mask = np.array([1, 0, 1, 1, 0, 1, 0, 1], dtype=np.int32)
-    run(SHAPES[1], 2, mask=mask)
     run(SHAPES[2], 2, mask=mask)
+    run(SHAPES[3], 2, mask=mask)
 
 
 def test_fused_quant_is_deterministic():
-    cfg = SHAPES[2]
+    cfg = SHAPES[3]
     a = run(cfg, 2)
     b = run(cfg, 2)
     assert np.array_equal(a, b)

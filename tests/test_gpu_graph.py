@@ -11,6 +11,8 @@ pytestmark = pytest.mark.gpu
     ("cfg4_decode_int8_t64", dict(hidden=1024, inter=512), 0),
     ("cfg1_cpu_ref_bf16", {}, 0),
     ("cfg3_dsv3_fp8", dict(tokens=2048, hidden=512, inter=256, experts=8), 0),
+    # the decode kernel with two token blocks per tile (40 rows per expert)
+    ("cfg4_decode_int8_t64", dict(tokens=160, hidden=1024, inter=512, experts=32), 0),
     # with the re-quantisation pass between the GEMMs (decode kernel / large-tile kernel)
     ("cfg4_decode_int8_t64", dict(hidden=1024, inter=512), 2),
     ("cfg4_decode_int8_t64", dict(tokens=2048, hidden=512, inter=256, experts=8), 2)])

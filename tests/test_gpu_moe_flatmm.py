@@ -17,7 +17,8 @@ def _rel(a, b):
     return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
 
 
-# (tokens, experts, topk, hidden, inter, unit): decode kernel, 32-row tiles, 128-row tiles, large-tile kernel
+# (tokens, experts, topk, hidden, inter, unit): decode kernel, 128-row tiles, decode kernel with two token blocks
+# per tile (fp8: 64-row tiles), large-tile kernel
 SHAPES = [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (130, 6, 2, 1152, 256, 64), (1024, 4, 2, 512, 384, 32)]
 
 

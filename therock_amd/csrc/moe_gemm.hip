@@ -451,6 +451,16 @@ inline int y_bytes(const mi355_fused_moe_traits& t)
     return (t.prec_i == MI355_MOE_FP8 || (t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0)) ? 1 : 2;
 }
 
+// the decode kernel's variant with two 32-row token blocks per tile exists for every operand type; for fp8 the
+// other kernels are faster wherever it could run
+inline bool two_block_decode_ok(const mi355_fused_moe_traits& t) { return t.prec_i != MI355_MOE_FP8; }
+
+// the decode kernel takes tiles of this many 32-row blocks
+inline bool decode_tile(const mi355_fused_moe_traits& t, int mblk)
+{
+    return mblk == 1 || (mblk == 2 && two_block_decode_ok(t));
+}
+
 // 32-row blocks per M tile, from the expected rows per expert; big_tile_rows()/32 selects the
 // large-tile kernel
 inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
@@ -463,9 +473,16 @@ inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, 
     const int64_t max_pad = topk * tokens + (int64_t)experts * t.block_m - topk;
     const int64_t x_rows  = t.fused_quant == 1 ? tokens * topk : tokens; // smooth-quant: a row per (slot, token)
     const bool fits = (int64_t)2 * inter * hidden * eb < lim && max_pad * inter * y_b < lim && x_rows * hidden * eb < lim;
-    // Measured crossovers (fp8, 256 experts; bf16, 8 experts): the decode kernel wins up to about 24 rows per
-    // expert, the large-tile kernel from about 28 on - it streams every weight tile once whatever the row
-    // count and fetches only the token slabs a tile has - provided its tiles fill the chip.
+    // Measured crossovers (fp8, 256 experts; int8, 128 experts; bf16, 8 experts): the decode kernel with one
+    // token block per tile wins up to about 24 rows per expert.  From about 28 on an expert often has more
+    // than 32 rows and would stream its weights twice: with 16-bit and int8 operands the decode kernel with two
+    // token blocks (64-row tiles) is the fastest up to about 52 rows per expert (12 to 25 % ahead of the
+    // large-tile kernel, whose single workgroup per compute unit cannot hide a tile's prologue and epilogue
+    // behind another tile's weight stream); with fp8 operands, and from there on for all types, the large-tile
+    // kernel - it streams every weight tile once whatever the row count and fetches only the token slabs a
+    // tile has - provided its tiles fill the chip.
+    if(two_block_decode_ok(t) && fits && avg >= 28 && avg <= 52)
+        return 2;
     const int64_t big_tiles = (int64_t)experts * std::max<int64_t>(1, ceil_div<int64_t>(avg, big_tile_rows())) * ceil_div(inter, 128);
     // (its tiles start on whole 16-row slabs of Y: the sort unit must be a multiple of 16)
     const bool big_ok = t.block_m % 16 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b, y_b == 1);
@@ -503,7 +520,7 @@ int launch_gemm(int mblk, const GemmParams& p, int max_tiles, hipStream_t stream
 }
 
 // One grouped GEMM over the tile list: sets the column-tile count for the kernel family that runs this
-// tile size and launches it.  use_decode: the caller found the decode kernel applicable (one 32-row block per
+// tile size and launches it.  use_decode: the caller found the decode kernel applicable (one or two 32-row blocks per
 // tile, 32-bit offsets suffice).  The down GEMM of the int8 path multiplies bf16 Y by int8 weights, or, with
 // y_i8, int8 Y (scaled per row) by int8 weights on the i8 MFMAs.
 int launch_grouped_gemm(int prec, bool gemm0, int mblk, bool use_decode, GemmParams& p, int max_tiles, hipStream_t stream,
@@ -514,7 +531,7 @@ int launch_grouped_gemm(int prec, bool gemm0, int mblk, bool use_decode, GemmPar
     p.max_tiles    = max_tiles;
     p.n_ntiles     = ceil_div(p.n_out, (use_decode ? decode_tile_cols(false) : 256) / pair);
     if(use_decode)
-        return launch_gemm_decode(prec, gemm0, p, max_tiles, stream, y_i8);
+        return launch_gemm_decode(prec, gemm0, mblk, p, max_tiles, stream, y_i8);
     if(mblk > 4)
         return launch_gemm_big(prec, gemm0, p, max_tiles, stream, y_i8);
     if(prec == MI355_MOE_BF16)
@@ -722,8 +739,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.k_bytes_w       = H * eb;
     p.n_out           = I;
     p.n_total         = g_rows;
-    // decode-sized problems (one 32-row block per tile) have their own kernel
-    const bool decode = mblk == 1 && decode_supported((int64_t)T * (p.x_slot_major ? K : 1) * a.stride_token * eb,
+    // decode-sized problems (one or two 32-row blocks per tile) have their own kernel
+    const bool decode = decode_tile(t, mblk) && decode_supported((int64_t)T * (p.x_slot_major ? K : 1) * a.stride_token * eb,
                                                       ws.max_pad * (int64_t)I * y_b, (int64_t)2 * I * H * eb);
     // the two large-tile GEMMs hand Y over in the slab-major layout (the re-quantisation pass writes it when there
     // is one; gemm0 then stores plain rows)
@@ -936,7 +953,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     const int64_t a_rows = g1 ? T : (int64_t)T * K;
     if(a_rows * p.x_row_bytes >= ((int64_t)1 << 32) && mblk > 4)
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: A of 4 GiB or more is not supported at this problem size");
-    const bool decode = mblk == 1 && decode_supported(a_rows * p.x_row_bytes, a_rows * p.x_row_bytes, p.w_expert_bytes);
+    const bool decode = decode_tile(L.traits, mblk) && decode_supported(a_rows * p.x_row_bytes, a_rows * p.x_row_bytes, p.w_expert_bytes);
     if(g1)
     {
         p.x_scale       = (w8 || f8) ? static_cast<const float*>(a.scale_m) : nullptr;

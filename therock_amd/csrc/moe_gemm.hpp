@@ -55,10 +55,10 @@ int big_tile_rows();
 bool big_tile_supported(int prec, int k_bytes0, int k_bytes1, bool y_i8 = false);
 int launch_gemm_big(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream, bool y_i8 = false);
 
-// decode kernel (moe_gemm_decode.hip): tiles of one 32-row block x decode_tile_cols() output columns
+// decode kernel (moe_gemm_decode.hip): tiles of `blocks` (1 or 2) 32-row blocks x decode_tile_cols() output columns
 int decode_tile_cols(bool gemm0);
 bool decode_supported(int64_t x_bytes, int64_t y_bytes, int64_t w_expert_bytes);
-int launch_gemm_decode(int prec, bool gemm0, const gemm::GemmParams& p, int max_tiles, hipStream_t stream,
+int launch_gemm_decode(int prec, bool gemm0, int blocks, const gemm::GemmParams& p, int max_tiles, hipStream_t stream,
                        bool y_i8 = false);
 
 size_t moe_flatmm_workspace_bytes(int kind, const mi355_moe_flatmm_args& a);

@@ -1,4 +1,4 @@
-// Grouped GEMM for decode-sized expert batches (at most one 32-row block per expert tile; gfx950).
+// Grouped GEMM for decode-sized expert batches (one or two 32-row blocks per expert tile; gfx950).
 //
 // With a handful of tokens per expert the two GEMMs are pure weight streaming, and what decides
 // the rate is the shape of the HBM requests: 128-byte pieces of 256 different rows (the tile shape
@@ -9,7 +9,9 @@
 // partial accumulators are added through LDS at the end (in wave order, so the result is
 // deterministic).  Same MFMA orientation (weight rows on the M side), operand layouts and epilogues
 // as moe_gemm_kernel; operand tiles are staged through LDS with the next step prefetched into
-// registers, weights with non-temporal loads.
+// registers, weights with non-temporal loads.  NXB = 2 multiplies every weight tile with two token
+// blocks (tiles of up to 64 sorted rows), so that experts with 33 .. 64 rows still stream their
+// weights once.
 #include "moe_gemm_device.hpp"
 
 #include <algorithm>
@@ -22,8 +24,8 @@ namespace {
 constexpr int kDecWRows = 64;  // weight rows per workgroup
 constexpr int kDecWKB   = 512; // weight bytes per row and step
 
-template <int MODE, bool GEMM0>
-__global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) void moe_gemm_decode_kernel(const GemmParams p)
+template <int MODE, bool GEMM0, int NXB>
+__global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) void moe_gemm_decode_kernel(const GemmParams p)
 {
     using MT  = ModeTraits<MODE>;
     using Acc = typename MT::Acc;
@@ -35,7 +37,7 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
     constexpr int kWaveWB  = kDecWKB / 4;             // weight bytes of a row one wave multiplies per step
     constexpr int kSteps   = kWaveWB * kXMul / (2 * kOpB); // MFMAs along K per wave and step
     constexpr int kWLoads  = kDecWRows * (kDecWKB / 16) / kBlock; // 8
-    constexpr int kXLoads  = 32 * (kXKB / 16) / kBlock;           // 4 or 8
+    constexpr int kXLoads  = NXB * 32 * (kXKB / 16) / kBlock;     // 4 or 8 per token block
     constexpr int kWRowsPerPass = kBlock / (kDecWKB / 16);        // 8
     constexpr int kXRowsPerPass = kBlock / (kXKB / 16);
     constexpr bool kMx     = MODE == kFp8 && !GEMM0;
@@ -57,7 +59,7 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
     const int expert = tile.expert;
     const int row0   = tile.row0;
     const int nt     = tile.nt;
-    const int nrows  = min(tile.nrows, 32);
+    const int nrows  = min(tile.nrows, 32 * NXB);
     const bool paired = GEMM0 && !p.gate_only; // gate rows paired with up rows (see run_epilogue)
     const int n_base  = nt * (paired ? 32 : 64);
 
@@ -114,14 +116,17 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
     // takes to have enough bytes outstanding to cover the HBM latency
     uint4 xv_[2][kXLoads];
     uint4 wv_[2][kWLoads];
-    uint32_t ys_next_[2] = {0x7f7f7f7fu, 0x7f7f7f7fu}, ys_cur = 0x7f7f7f7fu;
+    uint32_t ys_next_[2][NXB], ys_cur[NXB];
+#pragma unroll
+    for(int i = 0; i < NXB; i++)
+        ys_next_[0][i] = ys_next_[1][i] = ys_cur[i] = 0x7f7f7f7fu;
     const uint4 zero4 = {0u, 0u, 0u, 0u};
 
     auto load_tiles = [&](int kt, auto buf_tag) __attribute__((always_inline)) {
         constexpr int B   = decltype(buf_tag)::value;
         auto& xv          = xv_[B];
         auto& wv          = wv_[B];
-        uint32_t& ys_next = ys_next_[B];
+        auto& ys_next     = ys_next_[B];
         const int kx = kt * kXKB + xchunk * 16;
 #pragma unroll
         for(int j = 0; j < kXLoads; j++)
@@ -144,24 +149,30 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
         }
         if constexpr(kMx)
         {
-            // the four e8m0 scales of this wave's 128 columns of the step
-            ys_next         = 0x7f7f7f7fu;
-            const int kb    = kt * (kDecWKB / 32) + wave * 4;
-            if(r32 < nrows && kb * 32 < p.k_bytes_x)
+            // the four e8m0 scales of this wave's 128 columns of the step, per token block
+            const int kb = kt * (kDecWKB / 32) + wave * 4;
+#pragma unroll
+            for(int i = 0; i < NXB; i++)
             {
-                const unsigned char* sp = p.y_scale + (int64_t)kb * p.ys_kb_stride + row0 + r32;
-                ys_next = sp[0] | (sp[p.ys_kb_stride] << 8) | (sp[2 * p.ys_kb_stride] << 16) |
-                          (static_cast<uint32_t>(sp[3 * p.ys_kb_stride]) << 24);
+                ys_next[i] = 0x7f7f7f7fu;
+                if(r32 + 32 * i < nrows && kb * 32 < p.k_bytes_x)
+                {
+                    const unsigned char* sp = p.y_scale + (int64_t)kb * p.ys_kb_stride + row0 + r32 + 32 * i;
+                    ys_next[i] = sp[0] | (sp[p.ys_kb_stride] << 8) | (sp[2 * p.ys_kb_stride] << 16) |
+                                 (static_cast<uint32_t>(sp[3 * p.ys_kb_stride]) << 24);
+                }
             }
         }
     };
 
-    Acc acc[1][2];
+    Acc acc[NXB][2];
 #pragma unroll
-    for(int b = 0; b < 2; b++)
+    for(int i = 0; i < NXB; i++)
 #pragma unroll
-        for(int v = 0; v < 16; v++)
-            acc[0][b][v] = 0;
+        for(int b = 0; b < 2; b++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                acc[i][b][v] = 0;
 
     const int kt_count = ceil_div(p.k_bytes_w, kDecWKB);
     auto k_step = [&](int kt, auto buf_tag) __attribute__((always_inline)) {
@@ -174,7 +185,9 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
 #pragma unroll
         for(int j = 0; j < kWLoads; j++)
             *reinterpret_cast<uint4*>(lds_w + (wrow + kWRowsPerPass * j) * kWStride + wchunk * 16) = wv[j];
-        ys_cur = ys_next_[B];
+#pragma unroll
+        for(int i = 0; i < NXB; i++)
+            ys_cur[i] = ys_next_[B][i];
         __syncthreads();
         if(kt + 2 < kt_count)
             load_tiles(kt + 2, buf_tag);
@@ -182,8 +195,7 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
 #pragma unroll
         for(int s = 0; s < kSteps; s++)
         {
-            Frag wf[2], xf;
-            uint32_t xs = 127;
+            Frag wf[2];
 #pragma unroll
             for(int b = 0; b < 2; b++)
             {
@@ -198,17 +210,24 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
                     wf[b].hi = *reinterpret_cast<const uint4*>(wp + (4 * s + 2 + kg) * 16);
                 }
             }
-            if constexpr(kOpB == 16)
-                xf.lo = *reinterpret_cast<const uint4*>(xp + (2 * s + kg) * 16);
-            else
+#pragma unroll
+            for(int i = 0; i < NXB; i++)
             {
-                xf.lo = *reinterpret_cast<const uint4*>(xp + (4 * s + kg) * 16);
-                xf.hi = *reinterpret_cast<const uint4*>(xp + (4 * s + 2 + kg) * 16);
-                if constexpr(kMx)
-                    xs = (ys_cur >> (8 * (2 * s + kg))) & 0xffu;
+                Frag xf;
+                uint32_t xs              = 127;
+                const unsigned char* xpi = xp + i * 32 * kXStride;
+                if constexpr(kOpB == 16)
+                    xf.lo = *reinterpret_cast<const uint4*>(xpi + (2 * s + kg) * 16);
+                else
+                {
+                    xf.lo = *reinterpret_cast<const uint4*>(xpi + (4 * s + kg) * 16);
+                    xf.hi = *reinterpret_cast<const uint4*>(xpi + (4 * s + 2 + kg) * 16);
+                    if constexpr(kMx)
+                        xs = (ys_cur[i] >> (8 * (2 * s + kg))) & 0xffu;
+                }
+                acc[i][0] = mfma<MODE>(wf[0], xf, xs, acc[i][0]);
+                acc[i][1] = mfma<MODE>(wf[1], xf, xs, acc[i][1]);
             }
-            acc[0][0] = mfma<MODE>(wf[0], xf, xs, acc[0][0]);
-            acc[0][1] = mfma<MODE>(wf[1], xf, xs, acc[0][1]);
         }
         __syncthreads();
     };
@@ -226,14 +245,16 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
 
     // ---- add the four K slices: waves 1..3 park their accumulators in LDS, wave 0 sums in wave order
     using AccElem   = decltype(acc[0][0][0] + acc[0][0][0]);
-    AccElem* red    = reinterpret_cast<AccElem*>(lds); // [3][2][16][64]
+    AccElem* red    = reinterpret_cast<AccElem*>(lds); // [3][NXB][2][16][64]
     if(wave > 0)
     {
 #pragma unroll
-        for(int b = 0; b < 2; b++)
+        for(int i = 0; i < NXB; i++)
 #pragma unroll
-            for(int v = 0; v < 16; v++)
-                red[(((wave - 1) * 2 + b) * 16 + v) * 64 + lane] = acc[0][b][v];
+            for(int b = 0; b < 2; b++)
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    red[((((wave - 1) * NXB + i) * 2 + b) * 16 + v) * 64 + lane] = acc[i][b][v];
     }
     __syncthreads();
     if(wave > 0)
@@ -243,28 +264,51 @@ __global__ __launch_bounds__(kBlock, (MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) 
 #pragma nounroll
     for(int w = 0; w < 3; w++)
 #pragma unroll
-        for(int b = 0; b < 2; b++)
+        for(int i = 0; i < NXB; i++)
 #pragma unroll
-            for(int v = 0; v < 16; v++)
-                acc[0][b][v] += red[((w * 2 + b) * 16 + v) * 64 + lane];
+            for(int b = 0; b < 2; b++)
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    acc[i][b][v] += red[(((w * NXB + i) * 2 + b) * 16 + v) * 64 + lane];
 
-    run_epilogue<MODE, GEMM0, 1, true>(p, acc, expert, row0, nrows, 0, 32, 1, n_base, 0, r32, kg);
+    run_epilogue<MODE, GEMM0, NXB, true>(p, acc, expert, row0, nrows, 0, 32, ceil_div(nrows, 32), n_base, 0, r32, kg);
 }
 
-template <int MODE, bool GEMM0>
-int launch_decode_t(const GemmParams& p, int max_tiles, hipStream_t stream)
+template <int MODE, bool GEMM0, int NXB>
+int launch_decode_n(const GemmParams& p, int max_tiles, hipStream_t stream)
 {
     using MT            = ModeTraits<MODE>;
     constexpr int kXMul = MT::kXKB / MT::kWKB;
-    const size_t lds    = kDecWRows * (kDecWKB + kPadB) + 32 * (kDecWKB * kXMul + kPadB);
-    static_assert(3 * 2 * 16 * 64 * 4 <= kDecWRows * (kDecWKB + kPadB), "reduction buffer fits in the weight tile");
+    constexpr size_t lds = kDecWRows * (kDecWKB + kPadB) + NXB * 32 * (kDecWKB * kXMul + kPadB);
+    static_assert(3 * NXB * 2 * 16 * 64 * 4 <= lds, "the reduction buffer fits in the operand tiles");
     const int grid = round_up(max_tiles * p.n_ntiles, 8);
     if(grid <= 0)
         return MI355_MOE_OK;
     KernelTimer timer(GEMM0 ? MI355_MOE_K_GEMM0 : MI355_MOE_K_GEMM1, stream);
-    hipLaunchKernelGGL((moe_gemm_decode_kernel<MODE, GEMM0>), dim3(grid), dim3(kBlock), lds, stream, p);
+    if constexpr(lds > 64 * 1024)
+    {
+        // the dynamic LDS limit is an attribute of the function on one device: set once per device
+        static bool attr_ok[64] = {};
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        if(dev < 0 || dev >= 64 || !attr_ok[dev])
+        {
+            MI355_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_decode_kernel<MODE, GEMM0, NXB>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            if(dev >= 0 && dev < 64)
+                attr_ok[dev] = true;
+        }
+    }
+    hipLaunchKernelGGL((moe_gemm_decode_kernel<MODE, GEMM0, NXB>), dim3(grid), dim3(kBlock), lds, stream, p);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
+}
+
+// blocks: 32-row token blocks per tile (1 or 2)
+template <int MODE, bool GEMM0>
+int launch_decode_t(int blocks, const GemmParams& p, int max_tiles, hipStream_t stream)
+{
+    return blocks == 1 ? launch_decode_n<MODE, GEMM0, 1>(p, max_tiles, stream) : launch_decode_n<MODE, GEMM0, 2>(p, max_tiles, stream);
 }
 
 } // namespace
@@ -278,18 +322,21 @@ bool decode_supported(int64_t x_bytes, int64_t y_bytes, int64_t w_expert_bytes)
     return x_bytes < lim && y_bytes < lim && w_expert_bytes < lim;
 }
 
-int launch_gemm_decode(int prec, bool gemm0, const GemmParams& p, int max_tiles, hipStream_t stream, bool y_i8)
+int launch_gemm_decode(int prec, bool gemm0, int blocks, const GemmParams& p, int max_tiles, hipStream_t stream, bool y_i8)
 {
+    if(blocks != 1 && blocks != 2)
+        return fail(MI355_MOE_E_UNSUPPORTED, "decode kernel: %d token blocks per tile", blocks);
+    const int b = blocks;
     if(prec == MI355_MOE_INT8 && !gemm0 && y_i8)
-        return launch_decode_t<kI8, false>(p, max_tiles, stream);
+        return launch_decode_t<kI8, false>(b, p, max_tiles, stream);
     if(prec == MI355_MOE_BF16)
-        return gemm0 ? launch_decode_t<kBf16, true>(p, max_tiles, stream) : launch_decode_t<kBf16, false>(p, max_tiles, stream);
+        return gemm0 ? launch_decode_t<kBf16, true>(b, p, max_tiles, stream) : launch_decode_t<kBf16, false>(b, p, max_tiles, stream);
     if(prec == MI355_MOE_FP16)
-        return gemm0 ? launch_decode_t<kF16, true>(p, max_tiles, stream) : launch_decode_t<kF16, false>(p, max_tiles, stream);
+        return gemm0 ? launch_decode_t<kF16, true>(b, p, max_tiles, stream) : launch_decode_t<kF16, false>(b, p, max_tiles, stream);
     if(prec == MI355_MOE_FP8)
-        return gemm0 ? launch_decode_t<kFp8, true>(p, max_tiles, stream) : launch_decode_t<kFp8, false>(p, max_tiles, stream);
+        return gemm0 ? launch_decode_t<kFp8, true>(b, p, max_tiles, stream) : launch_decode_t<kFp8, false>(b, p, max_tiles, stream);
     if(prec == MI355_MOE_INT8)
-        return gemm0 ? launch_decode_t<kI8, true>(p, max_tiles, stream) : launch_decode_t<kBf16W8, false>(p, max_tiles, stream);
+        return gemm0 ? launch_decode_t<kI8, true>(b, p, max_tiles, stream) : launch_decode_t<kBf16W8, false>(b, p, max_tiles, stream);
     return fail(MI355_MOE_E_UNSUPPORTED, "no decode kernel for precision %d", prec);
 }
 
