@@ -376,13 +376,17 @@ def main():
 
     # Beyond the benchmark configurations: the int8 model at a prefill-sized token count, with the intermediate
     # activations kept in bf16 (fused_quant 0) or re-quantised to int8 so that the down GEMM runs on int8 MFMAs
-    # (fused_quant 2), and decode-sized batches whose routing is skewed (Zipf; one expert in every token's top-k).
+    # (fused_quant 2), batches between decode and prefill (40 rows per expert), and decode-sized batches whose routing
+    # is skewed (Zipf; one expert in every token's top-k).
     extra = {}
     if not a.headline_only:
         i8 = mi.CONFIGS["cfg4_decode_int8_t256"]
         cases = {
             "cfg4_model_int8_t8192_fused_quant0": (i8.scaled(name="cfg4_model_int8_t8192", tokens=8192), {}),
             "cfg4_model_int8_t8192_fused_quant2": (i8.scaled(name="cfg4_model_int8_t8192", tokens=8192), {"fused_quant": 2}),
+            # 40 rows per expert: the decode kernel with two token blocks per tile
+            "cfg4_model_int8_t640": (i8.scaled(name="cfg4_model_int8_t640", tokens=640), {}),
+            "cfg2_mixtral_bf16_t160": (mi.CONFIGS["cfg2_mixtral_bf16"].scaled(name="cfg2_mixtral_bf16_t160", tokens=160), {}),
             "cfg4_decode_int8_t256_zipf": (i8.scaled(name="cfg4_decode_int8_t256_zipf", router="zipf"), {}),
             "cfg4_decode_int8_t256_hot_expert": (i8.scaled(name="cfg4_decode_int8_t256_hot_expert"), {"hot_expert": True}),
         }

@@ -526,6 +526,10 @@ int launch_gemm(int mblk, const GemmParams& p, int max_tiles, hipStream_t stream
 int launch_grouped_gemm(int prec, bool gemm0, int mblk, bool use_decode, GemmParams& p, int max_tiles, hipStream_t stream,
                         bool y_i8 = false)
 {
+    // (bf16 Y times int8 weights, the int8 path's down GEMM without re-quantisation: the decode kernel's variant with
+    // two token blocks would stage twice the bytes per weight byte and spills; the 64-row small tiles run instead)
+    if(mblk == 2 && prec == MI355_MOE_INT8 && !gemm0 && !y_i8)
+        use_decode = false;
     // output columns per tile: the tile's weight rows, halved where gate and up rows share them
     const int pair = gemm0 && !p.gate_only ? 2 : 1;
     p.max_tiles    = max_tiles;

@@ -60,6 +60,9 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
     const int row0   = tile.row0;
     const int nt     = tile.nt;
     const int nrows  = min(tile.nrows, 32 * NXB);
+    // a tile of at most 32 rows leaves the second token block out: no LDS traffic and no MFMAs for it (its loads are
+    // masked row by row anyway)
+    const bool two   = NXB > 1 && nrows > 32;
     const bool paired = GEMM0 && !p.gate_only; // gate rows paired with up rows (see run_epilogue)
     const int n_base  = nt * (paired ? 32 : 64);
 
@@ -181,7 +184,8 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
         auto& wv        = wv_[B];
 #pragma unroll
         for(int j = 0; j < kXLoads; j++)
-            *reinterpret_cast<uint4*>(lds_x + (xrow + kXRowsPerPass * j) * kXStride + xchunk * 16) = xv[j];
+            if(j < kXLoads / NXB || two)
+                *reinterpret_cast<uint4*>(lds_x + (xrow + kXRowsPerPass * j) * kXStride + xchunk * 16) = xv[j];
 #pragma unroll
         for(int j = 0; j < kWLoads; j++)
             *reinterpret_cast<uint4*>(lds_w + (wrow + kWRowsPerPass * j) * kWStride + wchunk * 16) = wv[j];
@@ -213,6 +217,8 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
 #pragma unroll
             for(int i = 0; i < NXB; i++)
             {
+                if(i > 0 && !two)
+                    continue;
                 Frag xf;
                 uint32_t xs              = 127;
                 const unsigned char* xpi = xp + i * 32 * kXStride;
@@ -250,11 +256,15 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
     {
 #pragma unroll
         for(int i = 0; i < NXB; i++)
+        {
+            if(i > 0 && !two)
+                continue;
 #pragma unroll
             for(int b = 0; b < 2; b++)
 #pragma unroll
                 for(int v = 0; v < 16; v++)
                     red[((((wave - 1) * NXB + i) * 2 + b) * 16 + v) * 64 + lane] = acc[i][b][v];
+        }
     }
     __syncthreads();
     if(wave > 0)
@@ -265,11 +275,15 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
     for(int w = 0; w < 3; w++)
 #pragma unroll
         for(int i = 0; i < NXB; i++)
+        {
+            if(i > 0 && !two)
+                continue;
 #pragma unroll
             for(int b = 0; b < 2; b++)
 #pragma unroll
                 for(int v = 0; v < 16; v++)
                     acc[i][b][v] += red[(((w * NXB + i) * 2 + b) * 16 + v) * 64 + lane];
+        }
 
     run_epilogue<MODE, GEMM0, NXB, true>(p, acc, expert, row0, nrows, 0, 32, ceil_div(nrows, 32), n_base, 0, r32, kg);
 }
@@ -335,9 +349,11 @@ int launch_gemm_decode(int prec, bool gemm0, int blocks, const GemmParams& p, in
         return gemm0 ? launch_decode_t<kF16, true>(b, p, max_tiles, stream) : launch_decode_t<kF16, false>(b, p, max_tiles, stream);
     if(prec == MI355_MOE_FP8)
         return gemm0 ? launch_decode_t<kFp8, true>(b, p, max_tiles, stream) : launch_decode_t<kFp8, false>(b, p, max_tiles, stream);
-    if(prec == MI355_MOE_INT8)
-        return gemm0 ? launch_decode_t<kI8, true>(b, p, max_tiles, stream) : launch_decode_t<kBf16W8, false>(b, p, max_tiles, stream);
-    return fail(MI355_MOE_E_UNSUPPORTED, "no decode kernel for precision %d", prec);
+    if(prec == MI355_MOE_INT8 && gemm0)
+        return launch_decode_t<kI8, true>(b, p, max_tiles, stream);
+    if(prec == MI355_MOE_INT8 && b == 1) // (two token blocks of bf16 Y per int8 weight tile do not fit the register budget)
+        return launch_decode_n<kBf16W8, false, 1>(p, max_tiles, stream);
+    return fail(MI355_MOE_E_UNSUPPORTED, "no decode kernel for precision %d with %d token blocks per tile", prec, b);
 }
 
 } // namespace mi355
