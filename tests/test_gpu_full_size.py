@@ -82,10 +82,16 @@ def sample_tokens(cfg, sort, n=64):
     return np.array(sorted(set(picked)), dtype=np.int64)
 
 
-@pytest.mark.parametrize("name", list(mi.CONFIGS))
+# the benchmark configurations, and the two models at 40 rows per expert (64-row tiles of the decode kernel)
+WORKLOADS = dict(mi.CONFIGS)
+WORKLOADS["cfg4_model_int8_t640"] = mi.CONFIGS["cfg4_decode_int8_t256"].scaled(name="cfg4_model_int8_t640", tokens=640)
+WORKLOADS["cfg2_mixtral_bf16_t160"] = mi.CONFIGS["cfg2_mixtral_bf16"].scaled(name="cfg2_mixtral_bf16_t160", tokens=160)
+
+
+@pytest.mark.parametrize("name", list(WORKLOADS))
 def test_full_size_workload(name):
     from tests.gpu_util import rel_l2
-    cfg = mi.CONFIGS[name]
+    cfg = WORKLOADS[name]
     print(f"full-size {cfg}", flush=True)
     inp = mi.make_inputs_torch(cfg, "cuda", seed=0)
     traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit)
