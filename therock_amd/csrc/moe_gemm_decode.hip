@@ -347,8 +347,8 @@ int launch_gemm_decode(int prec, bool gemm0, int blocks, const GemmParams& p, in
         return gemm0 ? launch_decode_t<kBf16, true>(b, p, max_tiles, stream) : launch_decode_t<kBf16, false>(b, p, max_tiles, stream);
     if(prec == MI355_MOE_FP16)
         return gemm0 ? launch_decode_t<kF16, true>(b, p, max_tiles, stream) : launch_decode_t<kF16, false>(b, p, max_tiles, stream);
-    if(prec == MI355_MOE_FP8)
-        return gemm0 ? launch_decode_t<kFp8, true>(b, p, max_tiles, stream) : launch_decode_t<kFp8, false>(b, p, max_tiles, stream);
+    if(prec == MI355_MOE_FP8 && b == 1) // (with two token blocks the fp8 kernels spill and the other families are faster)
+        return gemm0 ? launch_decode_n<kFp8, true, 1>(p, max_tiles, stream) : launch_decode_n<kFp8, false, 1>(p, max_tiles, stream);
     if(prec == MI355_MOE_INT8 && gemm0)
         return launch_decode_t<kI8, true>(b, p, max_tiles, stream);
     if(prec == MI355_MOE_INT8 && b == 1) // (two token blocks of bf16 Y per int8 weight tile do not fit the register budget)
