@@ -388,6 +388,8 @@ def main():
             "cfg4_model_int8_t640": (i8.scaled(name="cfg4_model_int8_t640", tokens=640), {}),
             "cfg2_mixtral_bf16_t160": (mi.CONFIGS["cfg2_mixtral_bf16"].scaled(name="cfg2_mixtral_bf16_t160", tokens=160), {}),
             "cfg4_decode_int8_t256_zipf": (i8.scaled(name="cfg4_decode_int8_t256_zipf", router="zipf"), {}),
+            # fp8: the sort sees ~40 active experts of ~70 rows and takes the 320-row tiles (the host's average says 8 rows)
+            "cfg3_dsv3_fp8_t256_zipf": (mi.CONFIGS["cfg3_dsv3_fp8"].scaled(name="cfg3_dsv3_fp8_t256_zipf", tokens=256, router="zipf"), {}),
             "cfg4_decode_int8_t256_hot_expert": (i8.scaled(name="cfg4_decode_int8_t256_hot_expert"), {"hot_expert": True}),
         }
         for name, (c, kw) in cases.items():

@@ -150,6 +150,51 @@ def test_two_block_decode_tiles(dtype):
     chk(mi.MoeConfig("d2_zipf", 320, 512, 256, 16, 2, dtype, "zipf"), seed=8)
 
 
+def test_skewed_fp8_batch_takes_the_large_tiles_on_the_device():
+    """fp8, 16 rows per expert on average: the host picks decode tiles.  With Zipf routing the experts that have
+    tokens hold 48 padded rows or more each, and the sort, which has the counts, builds the work list for the 320-row
+    tiles instead; both kernel families are launched and one of them finds nothing to do.  Same shapes with uniform
+    routing, and with too few active experts to fill the chip, stay on the decode tiles.  Parity either way, also
+    through the expert mask, gate-only weights and on a second call with another routing on the same workspace."""
+    import torch
+    import therock_amd as ta
+    from tests.gpu_util import rel_l2, run_fused_moe
+
+    def run(cfg, seed, want_rows, **kw):
+        inp = mi.make_inputs_np(cfg, seed)
+        mask = kw.get("mask")
+        if mask is not None:
+            nloc = int(mask.sum())
+            for k in ("g", "d", "g_scale", "d_scale"):
+                inp[k] = inp[k][:nloc]
+        if kw.get("gate_only"):
+            inp["g"] = np.ascontiguousarray(inp["g"][:, :cfg.inter])
+            inp["g_scale"] = np.ascontiguousarray(inp["g_scale"][:, :cfg.inter])
+        print(f"fused_moe {cfg} seed={seed} {kw}", flush=True)
+        got, buf = run_fused_moe(cfg, inp, **kw)
+        traits = ta.fused_moe_traits(prec_i="fp8", prec_w="fp8", block_m=cfg.unit, local_expert_masking=mask is not None,
+                                     gate_only=kw.get("gate_only", 0))
+        shape = (cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter)
+        assert ta.fused_moe_tile_rows(traits, *shape) == 32
+        rows = ta.fused_moe_chosen_tile_rows(traits, buf, *shape)
+        ref, s = oracle_out(cfg, inp, mask, 1, kw.get("gate_only", 0))
+        active = len(set(s[2][:s[3] // cfg.unit].tolist()))
+        print(f"  tile rows chosen on the device: {rows}; {active} active experts, {s[3]} padded rows", flush=True)
+        assert rows == want_rows
+        assert np.array_equal(buf.sorted_ids[:s[3]].cpu().numpy(), s[0][:s[3]])
+        err = rel_l2(oracle.bf16_to_f32(got), ref)
+        print(f"  rel-L2 = {err:.3e} (tolerance {TOL['fp8']:.0e})", flush=True)
+        assert np.all(np.isfinite(oracle.bf16_to_f32(got))) and err <= TOL["fp8"]
+
+    zipf = mi.MoeConfig("skew", 256, 512, 2048, 64, 4, "fp8", "zipf")
+    run(zipf, 1, 320)
+    run(mi.MoeConfig("skew", 256, 512, 2048, 64, 4, "fp8", "softmax_renorm"), 2, 32)   # uniform: 16 rows per expert
+    run(mi.MoeConfig("skew", 256, 512, 256, 64, 4, "fp8", "zipf"), 3, 32)              # two column tiles per expert: too few
+    run(mi.MoeConfig("skew", 192, 512, 2048, 64, 4, "fp8", "zipf", unit=16), 4, 320)   # 16-row sort units, ragged tiles
+    run(mi.MoeConfig("skew", 256, 512, 4096, 64, 4, "fp8", "zipf"), 5, 320, gate_only=1)  # (half the column tiles per expert)
+    run(zipf, 6, 320, mask=np.array(([1, 1, 1, 1, 1, 1, 1, 0] * 8), dtype=np.int32))
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 def test_many_rows_per_expert_with_small_sort_units(dtype):
     # hundreds of rows per expert, but expert boundaries on multiples of 8 or 24 rows only: the 320-row kernel

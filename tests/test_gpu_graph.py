@@ -11,6 +11,8 @@ pytestmark = pytest.mark.gpu
     ("cfg4_decode_int8_t64", dict(hidden=1024, inter=512), 0),
     ("cfg1_cpu_ref_bf16", {}, 0),
     ("cfg3_dsv3_fp8", dict(tokens=2048, hidden=512, inter=256, experts=8), 0),
+    # fp8 with skewed routing: two kernel families per GEMM, the sort decides on the device which one has work
+    ("cfg3_dsv3_fp8", dict(tokens=256, hidden=512, inter=2048, experts=64, topk=4, router="zipf"), 0),
     # the decode kernel with two token blocks per tile (40 rows per expert)
     ("cfg4_decode_int8_t64", dict(tokens=160, hidden=1024, inter=512, experts=32), 0),
     # with the re-quantisation pass between the GEMMs (decode kernel / large-tile kernel)

@@ -104,6 +104,7 @@ PROTOTYPES = {
     "mi355_fused_moe_supported": (C.c_int, [C.POINTER(FusedMoeTraits)]),
     "mi355_fused_moe_workspace_size": (C.c_size_t, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
     "mi355_fused_moe_tile_rows": (C.c_int32, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
+    "mi355_fused_moe_chosen_tile_rows": (C.c_int32, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5 + [C.POINTER(Workspace), C.c_void_p]),
     "mi355_fused_moegemm": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeGemmArgs), C.POINTER(Workspace),
                                       C.c_void_p]),
     "mi355_fused_moe": (C.c_int, [C.POINTER(FusedMoeTraits), C.POINTER(FusedMoeArgs), C.POINTER(Workspace), C.c_void_p]),

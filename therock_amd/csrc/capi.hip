@@ -45,6 +45,7 @@ struct ProfileState
 {
     bool enabled  = false;
     uint32_t mask = 0xffffffffu; // kernel kinds that are timed
+    uint32_t held = 0;           // kinds whose launches are inside an enclosing event pair (KernelTimerGroup)
     std::vector<hipEvent_t> pool; // events created so far
     size_t used = 0;
     struct Rec
@@ -69,7 +70,16 @@ struct ProfileState
 ProfileState g_prof;
 } // namespace
 
-bool profiling_enabled(int kind) { return g_prof.enabled && ((g_prof.mask >> kind) & 1u) != 0; }
+bool profiling_enabled(int kind)
+{
+    return g_prof.enabled && ((g_prof.mask >> kind) & 1u) != 0 && ((g_prof.held >> kind) & 1u) == 0;
+}
+
+void profile_hold(int kind, bool on)
+{
+    if(kind >= 0 && kind < 32)
+        g_prof.held = on ? (g_prof.held | (1u << kind)) : (g_prof.held & ~(1u << kind));
+}
 
 void profile_mark(int kind, hipStream_t stream, bool begin)
 {
@@ -152,6 +162,7 @@ __attribute__((visibility("default"))) int mi355_moe_profile_start(void)
 __attribute__((visibility("default"))) int mi355_moe_profile_start_kinds(uint32_t kind_mask)
 {
     g_prof.mask = kind_mask;
+    g_prof.held = 0;
     g_prof.used = 0;
     g_prof.recs.clear();
     for(auto& p : g_prof.pending)
@@ -233,6 +244,34 @@ mi355_fused_moe_tile_rows(const mi355_fused_moe_traits* traits, int32_t tokens, 
        !sizes_in_range(tokens, num_experts, topk, hidden_size, intermediate_size))
         return 0;
     return gemm_tile_rows(*traits, tokens, num_experts, topk, hidden_size, intermediate_size);
+}
+
+__attribute__((visibility("default"))) int32_t
+mi355_fused_moe_chosen_tile_rows(const mi355_fused_moe_traits* traits, int32_t tokens, int32_t num_experts, int32_t topk,
+                                 int32_t hidden_size, int32_t intermediate_size, const mi355_moe_workspace* ws, void* stream)
+{
+    if(traits == nullptr || check_traits(*traits) != MI355_MOE_OK ||
+       !sizes_in_range(tokens, num_experts, topk, hidden_size, intermediate_size))
+        return 0;
+    const int host_rows = gemm_tile_rows(*traits, tokens, num_experts, topk, hidden_size, intermediate_size);
+    if(gemm_alt_tile_rows(*traits, tokens, num_experts, topk, hidden_size, intermediate_size) == 0)
+        return host_rows;
+    const WorkspaceLayout L = workspace_layout(*traits, tokens, num_experts, topk, hidden_size, intermediate_size);
+    if(ws == nullptr || ws->ptr == nullptr || ws->bytes < L.total)
+    {
+        fail(MI355_MOE_E_WORKSPACE, "fused_moe_chosen_tile_rows: the workspace of the call is needed");
+        return 0;
+    }
+    int32_t rows = 0;
+    const hipStream_t s = static_cast<hipStream_t>(stream);
+    if(hipMemcpyAsync(&rows, static_cast<const unsigned char*>(ws->ptr) + L.map_off + sizeof(int32_t), sizeof(int32_t),
+                      hipMemcpyDeviceToHost, s) != hipSuccess ||
+       hipStreamSynchronize(s) != hipSuccess)
+    {
+        fail(MI355_MOE_E_HIP, "fused_moe_chosen_tile_rows: reading the work list failed");
+        return 0;
+    }
+    return rows;
 }
 
 __attribute__((visibility("default"))) int

@@ -73,7 +73,34 @@ struct KernelTimer
     }
 };
 
-// ---- work list of the grouped GEMMs: int32 [kMapHdr + kMapEnt * max_tiles]; [0] = live tiles, then per
+// One event pair around several launches that count as one kernel of kind `k` (two candidate kernels of which one
+// finds nothing to do): the launches' own timers stay off meanwhile.
+void profile_hold(int kind, bool on);
+struct KernelTimerGroup
+{
+    int kind;
+    hipStream_t stream;
+    bool on;
+    KernelTimerGroup(int k, hipStream_t s, bool wanted) : kind(k), stream(s), on(wanted && profiling_enabled(k))
+    {
+        if(on)
+        {
+            profile_mark(kind, stream, true);
+            profile_hold(kind, true);
+        }
+    }
+    ~KernelTimerGroup()
+    {
+        if(on)
+        {
+            profile_hold(kind, false);
+            profile_mark(kind, stream, false);
+        }
+    }
+};
+
+// ---- work list of the grouped GEMMs: int32 [kMapHdr + kMapEnt * max_tiles]; [0] = live tiles, [1] = the tile
+// height (rows) the list was built for when the sort chose between two (else 0), then per
 // tile (local expert id, first sorted row, rows, first tile of the expert, tiles of the expert, first sorted
 // row of the expert, rows of the expert, rows per tile of the expert): any tile of an expert can be worked
 // out from the entry of any other.  Entries are 32-byte aligned.
@@ -87,6 +114,12 @@ struct GemmPlan
     int rows_per_tile; // sorted rows per GEMM tile (multiple of 32)
     int max_tiles;     // capacity of tile_map
     int* inv;          // [tokens * topk]: sorted position of every (token, slot), -1 when dropped
+    // A second tile height the sort may choose instead, from what only the device knows: with skewed routing the
+    // experts that have tokens at all hold many more rows than tokens * topk / experts suggests.  Chosen when at least
+    // alt_min_active experts are active and their padded rows average alt_min_rows or more; 0 rows: no choice.
+    int alt_rows_per_tile;
+    int alt_min_rows;
+    int alt_min_active;
 };
 
 // ---- sorting launcher shared by the stand-alone and the fused entry points

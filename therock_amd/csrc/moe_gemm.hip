@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
 
     // ---- work item: XCD x gets a contiguous range of the work list (workgroup ids are dealt
     // round-robin to the 8 XCDs), and inside an expert the M tiles of one weight tile are adjacent
-    const TileRef tile = lookup_tile(p.tile_map, p.n_ntiles, p.max_tiles, blockIdx.x);
+    const TileRef tile = lookup_tile(p.tile_map, p.n_ntiles, p.max_tiles, blockIdx.x, p.tile_rows);
     if(!tile.ok)
         return;
     const int expert = tile.expert;
@@ -463,16 +463,31 @@ inline bool decode_tile(const mi355_fused_moe_traits& t, int mblk)
 
 // 32-row blocks per M tile, from the expected rows per expert; big_tile_rows()/32 selects the
 // large-tile kernel
-inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
+// every operand of the problem can be addressed as a base plus a 32-bit byte offset (the large-tile and decode kernels)
+inline bool offsets_fit(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
 {
-    const int64_t avg = tokens * topk / std::max(experts, 1);
     const int eb  = (t.prec_i == MI355_MOE_BF16 || t.prec_i == MI355_MOE_FP16) ? 2 : 1;
     const int y_b = y_bytes(t);
-    // the large-tile kernel addresses each operand as a base plus a 32-bit byte offset
     const int64_t lim     = (int64_t)1 << 32;
     const int64_t max_pad = topk * tokens + (int64_t)experts * t.block_m - topk;
     const int64_t x_rows  = t.fused_quant == 1 ? tokens * topk : tokens; // smooth-quant: a row per (slot, token)
-    const bool fits = (int64_t)2 * inter * hidden * eb < lim && max_pad * inter * y_b < lim && x_rows * hidden * eb < lim;
+    return (int64_t)2 * inter * hidden * eb < lim && max_pad * inter * y_b < lim && x_rows * hidden * eb < lim;
+}
+
+// the large-tile kernel can run this problem (its tiles start on whole 16-row slabs of Y: the sort unit must be a
+// multiple of 16)
+inline bool big_tile_ok(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
+{
+    const int eb  = (t.prec_i == MI355_MOE_BF16 || t.prec_i == MI355_MOE_FP16) ? 2 : 1;
+    const int y_b = y_bytes(t);
+    return t.block_m % 16 == 0 && offsets_fit(t, tokens, topk, experts, hidden, inter) &&
+           big_tile_supported(t.prec_i, hidden * eb, inter * y_b, y_b == 1);
+}
+
+inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
+{
+    const int64_t avg = tokens * topk / std::max(experts, 1);
+    const bool fits   = offsets_fit(t, tokens, topk, experts, hidden, inter);
     // Measured crossovers (fp8, 256 experts; int8, 128 experts; bf16, 8 experts): the decode kernel with one
     // token block per tile wins up to about 24 rows per expert.  From about 28 on an expert often has more
     // than 32 rows and would stream its weights twice: with 16-bit and int8 operands the decode kernel with two
@@ -484,8 +499,7 @@ inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, 
     if(two_block_decode_ok(t) && fits && avg >= 28 && avg <= 52)
         return 2;
     const int64_t big_tiles = (int64_t)experts * std::max<int64_t>(1, ceil_div<int64_t>(avg, big_tile_rows())) * ceil_div(inter, 128);
-    // (its tiles start on whole 16-row slabs of Y: the sort unit must be a multiple of 16)
-    const bool big_ok = t.block_m % 16 == 0 && fits && big_tile_supported(t.prec_i, hidden * eb, inter * y_b, y_b == 1);
+    const bool big_ok = big_tile_ok(t, tokens, topk, experts, hidden, inter);
     if(big_ok && (avg >= 160 || (avg >= 28 && big_tiles >= device_info().num_cu)))
         return big_tile_rows() / 32;
     if(avg <= 32)
@@ -494,6 +508,21 @@ inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, 
         return 2;
     return 4;
 }
+
+// Skewed routing: the tile height above comes from the average rows per expert, tokens * topk / experts, but the
+// experts that have tokens at all may hold several times that, and the decode tiles then stream a hot expert's
+// weights once per 32 rows.  Where it pays (fp8: a Zipf-routed batch of 256 / 512 tokens of the 256-expert model runs
+// 28 / 40 % faster on the large tiles; int8 and bf16 gain nothing up to the row counts where the average selects the
+// large tiles anyway) the sort chooses between the two tile heights from the counts it holds, and both kernel
+// families are launched: the workgroups of the one whose tile height was not chosen leave at once (two short empty
+// launches per pass).  Returns the second tile height in 32-row blocks, 0: no choice.
+inline int alt_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
+{
+    if(t.prec_i != MI355_MOE_FP8 || t.fused_quant != 0 || !big_tile_ok(t, tokens, topk, experts, hidden, inter))
+        return 0;
+    return pick_mblk(t, tokens, topk, experts, hidden, inter) <= 4 ? big_tile_rows() / 32 : 0;
+}
+constexpr int kAltMinRows = 48; // padded rows per active expert from which the large tiles are chosen
 
 template <int MODE, bool GEMM0>
 int launch_gemm(int mblk, const GemmParams& p, int max_tiles, hipStream_t stream)
@@ -588,6 +617,12 @@ int gemm_tile_rows(const mi355_fused_moe_traits& t, int32_t tokens, int32_t expe
     return pick_mblk(t, tokens, topk, experts, hidden, inter) * 32;
 }
 
+int gemm_alt_tile_rows(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk, int32_t hidden,
+                       int32_t inter)
+{
+    return alt_mblk(t, tokens, topk, experts, hidden, inter) * 32;
+}
+
 WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk,
                                  int32_t hidden, int32_t inter)
 {
@@ -626,6 +661,10 @@ GemmPlan make_gemm_plan(const mi355_fused_moe_traits& t, void* ws_ptr, int32_t t
     g.rows_per_tile = pick_mblk(t, tokens, topk, experts, hidden, inter) * 32;
     g.max_tiles     = ws.max_tiles;
     g.inv           = reinterpret_cast<int*>(wsb + ws.inv_off);
+    // the second candidate needs enough active experts for its gate+up tiles (256 weight rows each) to fill the chip
+    g.alt_rows_per_tile = alt_mblk(t, tokens, topk, experts, hidden, inter) * 32;
+    g.alt_min_rows      = kAltMinRows;
+    g.alt_min_active    = ceil_div(device_info().num_cu, ceil_div((t.gate_only ? 1 : 2) * inter, 256));
     return g;
 }
 
@@ -700,6 +739,9 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     int* inv           = reinterpret_cast<int*>(wsb + ws.inv_off);
     const int mblk     = pick_mblk(t, T, K, E, H, I);
     const int max_units = (int)ceil_div<int64_t>(ws.max_pad, t.block_m);
+    // the sort chose between two tile heights (see alt_mblk): both kernel families are launched for each GEMM
+    const int alt           = prep_done ? alt_mblk(t, T, K, E, H, I) : 0;
+    const int alt_max_tiles = alt ? (int)std::min<int64_t>(ws.max_tiles, E + ws.max_pad / (alt * 32) + 1) : 0;
 
     const int n_inv      = T * K;
     const int prep_grid  = 1 + std::min(ceil_div(n_inv, kPrepBlock * 4), 64);
@@ -722,6 +764,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.tokens     = T;
     p.y_scale    = wsb + ws.ys_off;
     p.ys_kb_stride = ws.ys_kb_stride;
+    p.tile_rows  = alt ? mblk * 32 : 0;
 
     // ---- gemm0: gate+up, SiLU*up
     const bool requant = t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0;
@@ -751,9 +794,22 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     const int yq_b   = requant ? 1 : y_b; // bytes per element of what the down GEMM reads
     const int y_slab = (mblk > 4 && ((int64_t)I * yq_b) % 64 == 0) ? (int)((int64_t)I * yq_b / 64) : 0;
     p.y_slab         = requant ? 0 : y_slab;
-    rc               = launch_grouped_gemm(t.prec_i, true, mblk, decode, p, ws.max_tiles, stream);
-    if(rc != MI355_MOE_OK)
-        return rc;
+    const int alt_y_slab = (alt && ((int64_t)I * y_b) % 64 == 0) ? (int)((int64_t)I * y_b / 64) : 0;
+    {
+        KernelTimerGroup both(MI355_MOE_K_GEMM0, stream, alt != 0);
+        rc = launch_grouped_gemm(t.prec_i, true, mblk, decode, p, ws.max_tiles, stream);
+        if(rc != MI355_MOE_OK)
+            return rc;
+        if(alt)
+        {
+            GemmParams pa = p;
+            pa.tile_rows  = alt * 32;
+            pa.y_slab     = alt_y_slab;
+            rc            = launch_grouped_gemm(t.prec_i, true, alt, false, pa, alt_max_tiles, stream);
+            if(rc != MI355_MOE_OK)
+                return rc;
+        }
+    }
     p.x_slot_major = 0;
     if(requant)
     {
@@ -781,10 +837,22 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.k_bytes_w      = I * eb;
     p.n_out          = H;
     p.n_total        = H;
-    rc = launch_grouped_gemm(t.prec_i, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p, ws.max_tiles,
-                             stream, requant);
-    if(rc != MI355_MOE_OK)
-        return rc;
+    {
+        KernelTimerGroup both(MI355_MOE_K_GEMM1, stream, alt != 0);
+        rc = launch_grouped_gemm(t.prec_i, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p,
+                                 ws.max_tiles, stream, requant);
+        if(rc != MI355_MOE_OK)
+            return rc;
+        if(alt)
+        {
+            GemmParams pa = p;
+            pa.tile_rows  = alt * 32;
+            pa.y_slab     = alt_y_slab;
+            rc            = launch_grouped_gemm(t.prec_i, false, alt, false, pa, alt_max_tiles, stream);
+            if(rc != MI355_MOE_OK)
+                return rc;
+        }
+    }
 
     // ---- combine
     {

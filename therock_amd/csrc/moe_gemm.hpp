@@ -28,6 +28,9 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
                                  int32_t topk, int32_t hidden, int32_t inter);
 
 // sorted rows per GEMM workgroup at this problem size
+// the second tile height the sort may choose on the device for this problem (0: none)
+int gemm_alt_tile_rows(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk, int32_t hidden,
+                       int32_t inter);
 int gemm_tile_rows(const mi355_fused_moe_traits& t, int32_t tokens, int32_t experts, int32_t topk, int32_t hidden,
                    int32_t inter);
 

@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     const int ww   = wave & 3;  // weight-row quarter
 
     // ---- work item (same XCD-aware order as moe_gemm_kernel)
-    const TileRef tile = lookup_tile<true>(p.tile_map, p.n_ntiles, p.max_tiles, blockIdx.x);
+    const TileRef tile = lookup_tile<true>(p.tile_map, p.n_ntiles, p.max_tiles, blockIdx.x, p.tile_rows);
     if(!tile.ok)
         return;
     const int expert = tile.expert;

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
     const int kg   = lane >> 5;
 
     // ---- work item (same XCD-aware order as moe_gemm_kernel)
-    const TileRef tile = lookup_tile(p.tile_map, p.n_ntiles, p.max_tiles, blockIdx.x);
+    const TileRef tile = lookup_tile(p.tile_map, p.n_ntiles, p.max_tiles, blockIdx.x, p.tile_rows);
     if(!tile.ok)
         return;
     const int expert = tile.expert;

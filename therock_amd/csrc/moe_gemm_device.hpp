@@ -64,6 +64,7 @@ struct GemmParams
     int act;
     // fp8 gate+up GEMM of the stand-alone entry point: write bf16 instead of e4m3 with block scales
     int y_bf16;
+    int tile_rows; // != 0: run only if the tile list was built for this tile height (see lookup_tile)
     int max_tiles; // entries the tile list has room for (upper bound of live tiles)
     // stand-alone GEMMs (ck_tile's MoeFlatmmHostArgs, moe_flatmm_kernel.hpp:17-31): expert bias [experts, n_total] added
     // to the scaled dot products (null: none); the last n_padded weight rows of every expert are padding and
@@ -110,10 +111,19 @@ struct TileRef
     int expert_tiles;            // row tiles of this expert (each of them re-reads the same weight tiles)
     bool ok;
 };
+// tile_rows != 0: the launch is one of two candidates and runs only if the sort built the list for its tile height
+// (tile_map[1]); the other candidate's workgroups all leave at once.
 template <bool CHUNKED = false>
-__device__ inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_ntiles, int max_tiles, int block)
+__device__ inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_ntiles, int max_tiles, int block,
+                                      int tile_rows = 0)
 {
     TileRef t;
+    if(tile_rows != 0 && tile_map[1] != tile_rows)
+    {
+        t.expert = t.row0 = t.nrows = t.nt = t.expert_tiles = 0;
+        t.ok = false;
+        return t;
+    }
     const int slot = block >> 3;
     int work, total;
     if constexpr(CHUNKED)

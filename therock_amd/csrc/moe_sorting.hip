@@ -215,7 +215,19 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
     if(plan.tile_map != nullptr)
     {
         const int rows = tid < E ? s.tiles[tid] * U : 0;
-        const int nt   = ceil_div(rows, plan.rows_per_tile);
+        int rows_per_tile = plan.rows_per_tile;
+        if(plan.alt_rows_per_tile > 0) // (uniform: every thread takes this branch or none)
+        {
+            int active;
+            (void)block_exclusive_scan<kScanWaves>(rows > 0 ? 1 : 0, s.wave, active);
+            if(active >= plan.alt_min_active && (int64_t)total_tiles * U >= (int64_t)plan.alt_min_rows * active)
+                rows_per_tile = plan.alt_rows_per_tile;
+            if(tid == 0)
+                plan.tile_map[1] = rows_per_tile;
+        }
+        else if(tid == 0)
+            plan.tile_map[1] = 0;
+        const int nt   = ceil_div(rows, rows_per_tile);
         int n_tiles;
         const int tb = block_exclusive_scan<kScanWaves>(nt, s.wave, n_tiles);
         if(nt > 0)

@@ -339,6 +339,16 @@ def fused_moe_tile_rows(traits: fused_moe_traits, tokens, num_experts, topk, hid
                                                      intermediate_size))
 
 
+def fused_moe_chosen_tile_rows(traits: fused_moe_traits, buf, tokens, num_experts, topk, hidden_size, intermediate_size,
+                               stream=None) -> int:
+    """The tile height the last fused_moe call on buf's workspace ran with (where the routing decides, the sort's
+    choice on the device, read back after a stream synchronisation; else fused_moe_tile_rows)."""
+    t = traits.pod()
+    ws = _workspace(buf.ws)
+    return int(_lib.load().mi355_fused_moe_chosen_tile_rows(C.byref(t), tokens, num_experts, topk, hidden_size,
+                                                            intermediate_size, C.byref(ws), _stream(stream)))
+
+
 class MoeBuffers:
     """Caller-side allocation of everything fused_moe needs (what CK's example main does with
     DeviceMem): sort outputs, workspace and the output tensor."""
