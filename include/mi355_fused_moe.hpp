@@ -265,13 +265,17 @@ struct fused_moe_traits
     int gate_only       = 0;
     int fused_quant     = 0; // 0: no-sweep, 1: smooth-dynamic-quant, 2: dynamic-quant
     bool local_expert_masking = false;
+    // FusedMoeGemmWeightPermuteEnum of the ck_tile kernel (a template argument there): 1 = g and d arrive in
+    // b_nr_kr_kw_nw_kv, as CK's example pre-shuffles them
+    int weight_permute = 0;
 
     mi355_fused_moe_traits pod() const
     {
         using detail::dtype_of;
         return mi355_fused_moe_traits{dtype_of(prec_i),  dtype_of(prec_w),  dtype_of(prec_o), dtype_of(prec_st),
                                       dtype_of(prec_sw), dtype_of(prec_sq), dtype_of(prec_kw), block_m,
-                                      activation,        gate_only,         fused_quant,       local_expert_masking ? 1 : 0};
+                                      activation,        gate_only,         fused_quant,       local_expert_masking ? 1 : 0,
+                                      weight_permute};
     }
 };
 

@@ -151,6 +151,13 @@ typedef struct mi355_fused_moe_traits
                             row per (slot, token), a [topk, tokens, stride_token], a_scale [topk, tokens]
                             (UseSmoothQuant of fused_moegemm_traits.hpp:19-35; layouts moe_sorting_kernel.hpp:82-83) */
     int32_t local_expert_masking; /* 1 = apply local_expert_mask_ptr in the sort */
+    int32_t weight_permute; /* layout of g and d, FusedMoeGemmWeightPermuteEnum (fused_moegemm_traits.hpp:10-17; a
+                               template argument of ck_tile's kernel, not a field of its example's traits): 0 =
+                               no_permute, rows of K elements as ck_tile's host reference takes them; 1 =
+                               b_nr_kr_kw_nw_kv, what ck_tile's device kernel takes and its example produces before
+                               the call: [e, n/16, k/(4 kv), 4, 16, kv] with kv = 16 bytes of elements (8 for bf16 and
+                               fp16, 16 for fp8 and int8); needs K rows that are multiples of 64 bytes.  The kernels
+                               read either layout in place (mi355_moe_permute_weights converts between them) */
 } mi355_fused_moe_traits;
 
 /* FusedMoeGemmHostArgs (fused_moegemm_kernel.hpp:97-120), field for field.  Weights are plain row-major,

@@ -39,12 +39,13 @@ def run_sorting(topk_ids, weights, experts, unit, mask=None, local_tokens=None, 
     return ids.cpu().numpy(), w.cpu().numpy(), eid.cpu().numpy(), total.cpu().numpy()
 
 
-def run_fused_moe(cfg, inp, mask=None, unfused=False, stride_pad=0, activation=1, gate_only=0):
+def run_fused_moe(cfg, inp, mask=None, unfused=False, stride_pad=0, activation=1, gate_only=0, weight_permute=0,
+                  fused_quant=0):
     """Runs mi355_fused_moe (or sorting + mi355_fused_moegemm) on numpy inputs of
     therock_amd.inputs.make_inputs_np.  Returns (out bf16 bits (fp16 bits for fp16 operands) [T,H] numpy, buffers)."""
     traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, prec_o="fp16" if cfg.dtype == "fp16" else "bf16",
                                  block_m=cfg.unit, local_expert_masking=mask is not None, activation=activation,
-                                 gate_only=gate_only)
+                                 gate_only=gate_only, weight_permute=weight_permute, fused_quant=fused_quant)
     buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, "cuda")
     view = TORCH_DT[cfg.dtype]
     a = dev(inp["a"]).view(view)
@@ -54,6 +55,8 @@ def run_fused_moe(cfg, inp, mask=None, unfused=False, stride_pad=0, activation=1
         a = wide[:, :cfg.hidden]
         buf.out = torch.zeros((cfg.tokens, cfg.hidden + stride_pad), dtype=buf.out.dtype, device="cuda")[:, :cfg.hidden]
     g, d = dev(inp["g"]).view(view), dev(inp["d"]).view(view)
+    if weight_permute:  # what ck_tile's example does before the call (b_nr_kr_kw_nw_kv, 16-byte kv)
+        g, d = ta.permute_weights(g), ta.permute_weights(d)
     sc = {k: (None if inp[k] is None else dev(inp[k])) for k in ("a_scale", "g_scale", "d_scale")}
     args = ta.make_args(traits, buf, a, g, d, dev(inp["topk_ids"]), dev(inp["topk_weight"]), a_scale=sc["a_scale"],
                         g_scale=sc["g_scale"], d_scale=sc["d_scale"],

@@ -157,6 +157,11 @@ def test_host_only_entry_points():
     for pi, po, ok in ((5, 5, 1), (5, 0, 0), (0, 5, 0)):
         t = _lib.FusedMoeTraits(pi, pi, po, 3, 3, 3, 3, 32, 1, 0, 0, 0)
         assert lib.mi355_fused_moe_supported(C.byref(t)) == ok
+    # weight layouts: FusedMoeGemmWeightPermuteEnum's two values, nothing else
+    for prec in (0, 1, 2):
+        for wp, ok in ((0, 1), (1, 1), (2, 0), (-1, 0)):
+            t = _lib.FusedMoeTraits(prec, prec, 0, 3, 3, 3, 3, 32, 1, 0, 0, 0, wp)
+            assert lib.mi355_fused_moe_supported(C.byref(t)) == ok
     # fused_quant 1 / 2 (re-quantised intermediate activations) exist for int8 only and need a larger workspace
     for prec, fq, ok in ((2, 1, 1), (2, 2, 1), (2, 3, 0), (0, 2, 0), (1, 1, 0)):
         t = _lib.FusedMoeTraits(prec, prec, 0, 3, 3, 3, 3, 32, 1, 0, fq, 0)

@@ -29,7 +29,7 @@ class SortingArgs(C.Structure):
 class FusedMoeTraits(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
         "prec_i", "prec_w", "prec_o", "prec_st", "prec_sw", "prec_sq", "prec_kw", "block_m", "activation",
-        "gate_only", "fused_quant", "local_expert_masking")]
+        "gate_only", "fused_quant", "local_expert_masking", "weight_permute")]
 
 
 class FusedMoeGemmArgs(C.Structure):

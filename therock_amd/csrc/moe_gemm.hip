@@ -98,11 +98,18 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
         }
     }
 
-    const int wchunk = tid % kWChunks;
-    const int wrow   = tid / kWChunks; // + kWRowsPerPass*j  (row of the LDS weight tile)
+    // (row of the LDS weight tile, + kWRowsPerPass * j, and 16-byte chunk of the 128-byte K window) a thread fetches.
+    // Row-major weights: 8 consecutive threads walk the 128 contiguous bytes of a row.  ck_tile's pre-shuffled layout
+    // (1 KiB blocks of 16 rows x 64 bytes, pieces ordered by chunk, then row): 16 consecutive threads take the 16 rows
+    // of a chunk, a wave one whole block - the rows whose channels, by chan_of_row(), are 16 (wave / 2) + tid % 16.
+    static_assert(kWChunks == 8 && kWRowsPerPass == 32, "the pre-shuffled assignment below covers 32 rows x 8 chunks per pass");
+    const bool wperm = p.w_permuted != 0;
+    const int wchunk = wperm ? ((wave & 1) << 2) | ((tid >> 4) & 3) : tid % kWChunks;
+    const int wrow   = wperm ? (((tid >> 3) & 1) << 4) | (((tid >> 2) & 1) << 3) | ((wave >> 1) << 2) | (tid & 3) : tid / kWChunks;
     const bool paired = GEMM0 && !p.gate_only; // gate rows paired with up rows (see run_epilogue)
     const int n_base  = nt * (paired ? 128 : 256);
-    const unsigned char* wbase = p.w + (int64_t)expert * p.w_expert_bytes + wchunk * 16;
+    const unsigned char* wbase = p.w + (int64_t)expert * p.w_expert_bytes;
+    const int w_kadv           = weight_k_advance(p, kWKB); // bytes between the K windows of two steps
     int64_t woff[kWLoads];
 #pragma unroll
     for(int j = 0; j < kWLoads; j++)
@@ -120,7 +127,8 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
         {
             grow = min(n_base + blk * 32 + c, p.n_total - 1);
         }
-        woff[j] = (int64_t)grow * p.w_row_bytes;
+        // (row-major rows may lie 4 GiB or more into the expert: 64-bit there)
+        woff[j] = wperm ? (int64_t)weight_offset(p, grow, wchunk) : (int64_t)grow * p.w_row_bytes + wchunk * 16;
     }
 
     uint4 xv[kXLoads];
@@ -146,7 +154,7 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
             {
                 // decode-sized tiles stream every weight exactly once: non-temporal loads reach a
                 // markedly higher HBM rate than cached ones
-                const uint4* src = reinterpret_cast<const uint4*>(wbase + woff[j] + kt * kWKB);
+                const uint4* src = reinterpret_cast<const uint4*>(wbase + woff[j] + kt * w_kadv);
                 if constexpr(MBLK == 1)
                 {
                     typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
@@ -608,6 +616,9 @@ int check_traits(const mi355_fused_moe_traits& t)
                     t.fused_quant, t.prec_i);
     if(t.block_m < 1 || t.block_m > 1024)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: block_m=%d", t.block_m);
+    if(t.weight_permute != 0 && t.weight_permute != 1)
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: weight_permute=%d (0 = no_permute, 1 = b_nr_kr_kw_nw_kv)",
+                    t.weight_permute);
     return MI355_MOE_OK;
 }
 
@@ -714,6 +725,11 @@ int validate_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_mo
     for(const void* ptr : {a.a_ptr, a.g_ptr, a.d_ptr, static_cast<const void*>(a.o_ptr)})
         if(reinterpret_cast<uintptr_t>(ptr) % 16 != 0)
             return fail(MI355_MOE_E_INVALID, "fused_moegemm: a, g, d and o must be 16-byte aligned");
+    // pre-shuffled weights: blocks of 16 rows x 64 bytes of K, addressed with 32-bit offsets inside an expert
+    if(t.weight_permute != 0 && (((int64_t)H * eb) % 64 != 0 || ((int64_t)I * eb) % 64 != 0 ||
+                                 (int64_t)2 * I * H * eb >= ((int64_t)1 << 32)))
+        return fail(MI355_MOE_E_UNSUPPORTED, "fused_moegemm: pre-shuffled weights need rows of whole 64-byte blocks and "
+                                             "experts below 4 GiB (H=%d I=%d)", H, I);
     const int mblk = pick_mblk(t, T, K, E, H, I);
     // (smooth-quant activations hold a row per (slot, token))
     if(mblk > 4 && (int64_t)T * (t.fused_quant == 1 ? K : 1) * a.stride_token * eb >= ((int64_t)1 << 32))
@@ -765,6 +781,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.y_scale    = wsb + ws.ys_off;
     p.ys_kb_stride = ws.ys_kb_stride;
     p.tile_rows  = alt ? mblk * 32 : 0;
+    p.w_permuted = t.weight_permute;
 
     // ---- gemm0: gate+up, SiLU*up
     const bool requant = t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0;

@@ -20,8 +20,11 @@
 //     not overtake them, so the token stream costs its stand-alone time on top of the weight stream (about
 //     19 bytes per clock together; a step of this tile needs up to 36.9 KB for 1400 clocks of MFMA work).
 //   * LDS rows are swizzled: 64-byte token rows keep chunk c of row r at c ^ ((r >> 2) & 3), 128-byte
-//     weight rows at c ^ ((r >> 1) & 7); both the linear DMA writes and the ds_read_b128 operand
-//     fetches are then conflict-free on the 64-bank LDS.  Token rows past the tile's last row inside a
+//     token rows at c ^ ((r >> 1) & 7), 128-byte weight rows at c ^ weight_row_swizzle(r); both the linear DMA
+//     writes and the ds_read_b128 operand fetches are then conflict-free on the 64-bank LDS.  Weight rows sit in
+//     LDS in channel order (row r of a 32-row block = channel r; the lane whose MFMA row is m reads row
+//     chan_of_row(m)), so that the eight rows of a DMA instruction are eight consecutive channels: eight full
+//     128-byte lines in the row-major layout and in ck_tile's pre-shuffled one alike.  Token rows past the tile's last row inside a
 //     fetched 64-row group (and padding ids) fetch some real row instead - their MFMA columns are never
 //     stored; whole groups the tile does not have are not fetched.
 //   * The K loop is specialised on the number of token blocks a wave owns, on the number of 64-row token
@@ -66,6 +69,11 @@ constexpr int kLdsBytesPair = kXOffsetPair + 2 * kXPairBytes;
 static_assert(kLdsBytesPair <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 
 typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
+
+// Chunk swizzle of the 128-byte weight rows in LDS.  The 16 lanes that a ds_read_b128 serves together read the rows
+// chan_of_row(16 i .. 16 i + 15) = {0..3, 16..19, 4..7, 20..23} (+ 8 for i = 1): among the rows of equal parity (two
+// rows span the 64 banks) bits 1, 2 and 4 of the row number take all eight values.
+__device__ __host__ constexpr int weight_row_swizzle(int r) { return ((r >> 1) & 3) | (((r >> 4) & 1) << 2); }
 
 
 __device__ inline uint32_t lds_offset(const void* p)
@@ -188,17 +196,17 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
 #pragma unroll
             for(int j = 0; j < 4; j++)
             {
-                const int rih    = (q4 + 4 * j) * 8 + (lane >> 3); // row inside the half
+                const int rih    = (q4 + 4 * j) * 8 + (lane >> 3); // LDS row inside the half
                 const int trow   = h * kWHalfRows + rih;
                 const int blk    = trow >> 5;
-                const int c      = chan_of_row(trow & 31);
-                const int cchunk = (lane & 7) ^ ((rih >> 1) & 7);
+                const int c      = trow & 31; // LDS row r of a 32-row block holds weight channel r (see weight_row_swizzle)
+                const int cchunk = (lane & 7) ^ weight_row_swizzle(rih);
                 int grow;
                 if(paired)
                     grow = (blk & 1) * p.n_out + min(n_base + (blk >> 1) * 32 + c, p.n_out - 1);
                 else
                     grow = min(n_base + blk * 32 + c, p.n_total - 1);
-                doff[h * 4 + j] = (uint32_t)grow * (uint32_t)p.w_row_bytes + cchunk * 16;
+                doff[h * 4 + j] = weight_offset(p, grow, cchunk);
             }
     }
     else
@@ -259,13 +267,14 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     // re-reads should hit L2, and non-temporal fetches cost 3 % there.  NT is a template argument like the
     // slab-group count, for the same reason.
     const bool w_nt = tile.expert_tiles == 1;
+    const int w_kadv = weight_k_advance(p, 2 * kStepKB); // bytes between the 128-byte K windows of two weight units
     auto issue_w = [&](int u, auto half_tag, auto nt_tag) __attribute__((always_inline)) {
         constexpr int H = decltype(half_tag)::value;
         constexpr bool NT = decltype(nt_tag)::value;
         if(u >= n_wunits)
             return;
         const uint32_t sbase     = lds_base + (u % kWS) * kWUnitBytes + q4 * 1024;
-        const unsigned char* src = dbase + (u >> 1) * (2 * kStepKB);
+        const unsigned char* src = dbase + (u >> 1) * w_kadv;
 #pragma unroll
         for(int j = 0; j < 4; j++)
         {
@@ -362,9 +371,11 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     }
 
     // per-lane LDS read offsets (swizzled chunk positions are per-lane constants)
-    const int sw_w  = (r32 >> 1) & 7; // 128-byte weight rows
+    const int sw_w  = (r32 >> 1) & 7; // 128-byte token rows of the gate+up GEMM
+    const int w_row = chan_of_row(r32); // LDS row that holds the channel of this lane's MFMA row
+    const int sw_wr = weight_row_swizzle(w_row);
     const int sw_x  = (r32 >> 2) & 3; // 64-byte token rows
-    const int w_off = ((ww & 1) * 64 + r32) * (2 * kStepKB);
+    const int w_off = ((ww & 1) * 64 + w_row) * (2 * kStepKB);
     const int w_h   = ww >> 1;
     const int x_off = kXOffset + (wt * 32 + r32) * kStepKB;
 
@@ -384,8 +395,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 constexpr int P          = decltype(p_tag)::value;
                 constexpr int kh         = P * 4; // first chunk of the step inside the 128-byte weight row
                 const unsigned char* wp  = lds + (((kk & ~1) + w_h) % kWS) * kWUnitBytes + w_off + b * 32 * (2 * kStepKB);
-                const int cw_lo          = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_w) * 16 : ((kh + kg) ^ sw_w) * 16;
-                const int cw_hi          = ((kh + 2 + kg) ^ sw_w) * 16;
+                const int cw_lo          = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_wr) * 16 : ((kh + kg) ^ sw_wr) * 16;
+                const int cw_hi          = ((kh + 2 + kg) ^ sw_wr) * 16;
                 Frag f;
                 f.lo = *reinterpret_cast<const uint4*>(wp + cw_lo);
                 if constexpr(kOpB == 32)
@@ -580,8 +591,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 uint32_t xs[NF];
                 const int cx_lo = kOpB == 16 ? ((2 * s + kg) ^ sw_x) * 16 : (kg ^ sw_x) * 16;
                 const int cx_hi = ((2 + kg) ^ sw_x) * 16;
-                const int cw_lo = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_w) * 16 : ((kh + kg) ^ sw_w) * 16;
-                const int cw_hi = ((kh + 2 + kg) ^ sw_w) * 16;
+                const int cw_lo = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_wr) * 16 : ((kh + kg) ^ sw_wr) * 16;
+                const int cw_hi = ((kh + 2 + kg) ^ sw_wr) * 16;
 #pragma unroll
                 for(int b = 0; b < 2; b++)
                 {
@@ -589,7 +600,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                     if constexpr(kW8)
                     {
                         // 8 int8 of this lane's K group: 16-byte chunk (k & 3) * 2 + s of the row, half kg
-                        const int c8 = ((((k & 3) << 1) + s) ^ sw_w) * 16 + kg * 8;
+                        const int c8 = ((((k & 3) << 1) + s) ^ sw_wr) * 16 + kg * 8;
                         wf[b].lo     = int8x8_to_bf16x8(*reinterpret_cast<const uint2*>(wp + c8));
                     }
                     else

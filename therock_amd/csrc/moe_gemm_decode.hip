@@ -24,7 +24,7 @@ namespace {
 constexpr int kDecWRows = 64;  // weight rows per workgroup
 constexpr int kDecWKB   = 512; // weight bytes per row and step
 
-template <int MODE, bool GEMM0, int NXB>
+template <int MODE, bool GEMM0, int NXB, bool WPERM>
 __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8) ? 2 : 3) void moe_gemm_decode_kernel(const GemmParams p)
 {
     using MT  = ModeTraits<MODE>;
@@ -97,14 +97,27 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
             xoff[j] = (uint32_t)src * (uint32_t)p.x_row_bytes + xchunk * 16;
         }
     }
-    const int wchunk = tid % (kDecWKB / 16);
-    const int wrow   = tid / (kDecWKB / 16);
+    // Which 16 bytes of the 64 x 512-byte weight tile thread `tid` fetches with load j, as (tile row, 16-byte chunk) =
+    // (w_row0 + w_row_add(j), w_chunk0 + w_chunk_add(j)).  Row-major weights: 32 consecutive threads walk the 512
+    // contiguous bytes of a row.  ck_tile's pre-shuffled layout (16 rows x 64 bytes per 1 KiB block, the 16-byte
+    // pieces of a block ordered by chunk, then row): 16 consecutive threads take the 16 rows of one chunk, 64 a
+    // whole block, the four waves four consecutive blocks - a wave's load is 1 KiB of contiguous memory there too.
+    // (Bits of the row: 0-1 = tid bits 0-1, 2 = j bit 1, 3-4 = tid bits 2-3, 5 = j bit 2, so that the channels
+    // chan_of_row() gives the rows are 16 (j bit 1) + tid % 16; chunk: 0-3 = tid bits 4-7, 4 = j bit 0.)
+    // (a template argument: chosen at run time the per-load offsets stop being constants, which costs the registers
+    // that three workgroups per compute unit leave no room for)
+    constexpr bool wperm = WPERM;
+    const int w_chunk0 = wperm ? ((tid >> 6) << 2) | ((tid >> 4) & 3) : tid % (kDecWKB / 16);
+    const int w_row0   = wperm ? (((tid >> 3) & 1) << 4) | (((tid >> 2) & 1) << 3) | (tid & 3) : tid / (kDecWKB / 16);
+    auto w_row_add     = [&](int j) { return wperm ? ((j >> 2) << 5) | (((j >> 1) & 1) << 2) : kWRowsPerPass * j; };
+    auto w_chunk_add   = [&](int j) { return wperm ? (j & 1) << 4 : 0; };
+    static_assert(kWLoads == 8 && kWRowsPerPass == 8, "the assignments above cover 64 rows x 32 chunks with 8 loads of 256 threads");
     const unsigned char* wbase = p.w + (int64_t)expert * p.w_expert_bytes;
     uint32_t woff[kWLoads];
 #pragma unroll
     for(int j = 0; j < kWLoads; j++)
     {
-        const int lrow = wrow + kWRowsPerPass * j;
+        const int lrow = w_row0 + w_row_add(j);
         const int blk  = lrow >> 5;
         const int c    = chan_of_row(lrow & 31);
         int grow;
@@ -112,9 +125,10 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
             grow = blk * p.n_out + min(n_base + c, p.n_out - 1);
         else
             grow = min(n_base + blk * 32 + c, p.n_total - 1);
-        woff[j] = (uint32_t)grow * (uint32_t)p.w_row_bytes + wchunk * 16;
+        woff[j] = weight_offset(p, grow, w_chunk0 + w_chunk_add(j));
     }
 
+    const int w_kadv = weight_k_advance(p, kDecWKB); // bytes between the K windows of two steps
     // two steps are kept in flight per workgroup: with three workgroups on a compute unit that is what it
     // takes to have enough bytes outstanding to cover the HBM latency
     uint4 xv_[2][kXLoads];
@@ -138,15 +152,15 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
             if(xvalid[j] && kx < p.k_bytes_x)
                 xv[j] = *reinterpret_cast<const uint4*>(p.x + (xoff[j] + (uint32_t)(kt * kXKB)));
         }
-        const int kw = kt * kDecWKB + wchunk * 16;
+        const int kw = kt * kDecWKB + w_chunk0 * 16;
 #pragma unroll
         for(int j = 0; j < kWLoads; j++)
         {
             wv[j] = zero4;
-            if(kw < p.k_bytes_w)
+            if(kw + w_chunk_add(j) * 16 < p.k_bytes_w)
             {
                 typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
-                const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wbase + (woff[j] + (uint32_t)(kt * kDecWKB))));
+                const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wbase + (woff[j] + (uint32_t)(kt * w_kadv))));
                 wv[j]           = make_uint4(t[0], t[1], t[2], t[3]);
             }
         }
@@ -188,7 +202,7 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
                 *reinterpret_cast<uint4*>(lds_x + (xrow + kXRowsPerPass * j) * kXStride + xchunk * 16) = xv[j];
 #pragma unroll
         for(int j = 0; j < kWLoads; j++)
-            *reinterpret_cast<uint4*>(lds_w + (wrow + kWRowsPerPass * j) * kWStride + wchunk * 16) = wv[j];
+            *reinterpret_cast<uint4*>(lds_w + (w_row0 + w_row_add(j)) * kWStride + (w_chunk0 + w_chunk_add(j)) * 16) = wv[j];
 #pragma unroll
         for(int i = 0; i < NXB; i++)
             ys_cur[i] = ys_next_[B][i];
@@ -288,8 +302,8 @@ __global__ __launch_bounds__(kBlock, (NXB > 1 || MODE == kBf16W8 || MODE == kFp8
     run_epilogue<MODE, GEMM0, NXB, true>(p, acc, expert, row0, nrows, 0, 32, ceil_div(nrows, 32), n_base, 0, r32, kg);
 }
 
-template <int MODE, bool GEMM0, int NXB>
-int launch_decode_n(const GemmParams& p, int max_tiles, hipStream_t stream)
+template <int MODE, bool GEMM0, int NXB, bool WPERM>
+int launch_decode_w(const GemmParams& p, int max_tiles, hipStream_t stream)
 {
     using MT            = ModeTraits<MODE>;
     constexpr int kXMul = MT::kXKB / MT::kWKB;
@@ -307,15 +321,22 @@ int launch_decode_n(const GemmParams& p, int max_tiles, hipStream_t stream)
         (void)hipGetDevice(&dev);
         if(dev < 0 || dev >= 64 || !attr_ok[dev])
         {
-            MI355_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_decode_kernel<MODE, GEMM0, NXB>),
+            MI355_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_decode_kernel<MODE, GEMM0, NXB, WPERM>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             if(dev >= 0 && dev < 64)
                 attr_ok[dev] = true;
         }
     }
-    hipLaunchKernelGGL((moe_gemm_decode_kernel<MODE, GEMM0, NXB>), dim3(grid), dim3(kBlock), lds, stream, p);
+    hipLaunchKernelGGL((moe_gemm_decode_kernel<MODE, GEMM0, NXB, WPERM>), dim3(grid), dim3(kBlock), lds, stream, p);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
+}
+
+template <int MODE, bool GEMM0, int NXB>
+int launch_decode_n(const GemmParams& p, int max_tiles, hipStream_t stream)
+{
+    return p.w_permuted ? launch_decode_w<MODE, GEMM0, NXB, true>(p, max_tiles, stream)
+                        : launch_decode_w<MODE, GEMM0, NXB, false>(p, max_tiles, stream);
 }
 
 // blocks: 32-row token blocks per tile (1 or 2)

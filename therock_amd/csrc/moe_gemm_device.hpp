@@ -40,6 +40,10 @@ struct GemmParams
     unsigned char* y_scale;  // e8m0 block scales of Y (fp8 path): written by gemm0, read by gemm1
     int64_t x_row_bytes;
     int64_t w_row_bytes;
+    // weight layout: 0 = rows of K bytes ([experts, n, k], FusedMoeGemmWeightPermuteEnum::no_permute); 1 = ck_tile's
+    // pre-shuffled b_nr_kr_kw_nw_kv (fused_moegemm_traits.hpp:10-17): blocks of 16 rows x 64 bytes of K, 1 KiB each,
+    // ordered [n / 16][k bytes / 64]; inside a block the 16-byte piece c of row r sits at 256 c + 16 r
+    int w_permuted;
     int64_t w_expert_bytes;
     int64_t out_row_bytes;
     int64_t ys_kb_stride;    // bytes between consecutive 32-column blocks of y_scale ([inter/32][rows])
@@ -97,6 +101,18 @@ __device__ inline int64_t slot_row(int sid, int topk)
 {
     return (int64_t)(sid & 0xffffff) * topk + static_cast<int>(static_cast<uint32_t>(sid) >> 24);
 }
+
+// Byte offset, inside one expert's weight matrix, of the 16 bytes of row `row` that start `chunk16` 16-byte pieces
+// into a window of K that begins on a multiple of 64 bytes; and what moving that window by `bytes` (a multiple of
+// 64) adds to it.  Row-major: row * row_bytes + 16 * chunk16, + bytes.  Pre-shuffled: the row's block row, the block
+// (chunk16 / 4) of the window, the piece inside the block; a window 64 bytes further on is the next 1 KiB block.
+__device__ inline uint32_t weight_offset(const GemmParams& p, int row, int chunk16)
+{
+    if(p.w_permuted == 0)
+        return (uint32_t)row * (uint32_t)p.w_row_bytes + chunk16 * 16;
+    return (uint32_t)(row >> 4) * (uint32_t)(p.w_row_bytes * 16) + (chunk16 >> 2) * 1024 + (chunk16 & 3) * 256 + (row & 15) * 16;
+}
+__device__ inline int weight_k_advance(const GemmParams& p, int bytes) { return p.w_permuted == 0 ? bytes : bytes * 16; }
 
 // Work item -> tile.  Workgroup ids are dealt round-robin to the 8 XCDs; inside an expert the row tiles of one
 // weight tile are adjacent.  One entry of the list describes the whole expert, so a single load resolves any of

@@ -30,6 +30,7 @@ class fused_moe_traits:
     gate_only: int = 0
     fused_quant: int = 0
     local_expert_masking: bool = False
+    weight_permute: int = 0  # 1: g and d in ck_tile's pre-shuffled layout b_nr_kr_kw_nw_kv
 
     def pod(self) -> _lib.FusedMoeTraits:
         d = _lib.DTYPES
@@ -38,7 +39,7 @@ class fused_moe_traits:
                 raise ValueError(f"unknown precision {getattr(self, k)!r} for {k}")
         return _lib.FusedMoeTraits(d[self.prec_i], d[self.prec_w], d[self.prec_o], d[self.prec_st], d[self.prec_sw],
                                    d[self.prec_sq], d[self.prec_kw], self.block_m, self.activation, self.gate_only,
-                                   self.fused_quant, int(self.local_expert_masking))
+                                   self.fused_quant, int(self.local_expert_masking), int(self.weight_permute))
 
 
 @dataclass
