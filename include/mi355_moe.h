@@ -335,7 +335,7 @@ typedef struct mi355_moe_flatmm_args
     const void* p_sorted_expert_ids;
     const void* p_max_token_id;          /* [1] int32: rows after padding (p_total_tokens_post_pad) */
     const void* a_ptr;    /* gate+up: [NumTokens, stride_A]; down: [NumTokens * TopK, stride_A] */
-    const void* b_ptr;    /* [NumExperts, N, K], K contiguous (stride_B = K) */
+    const void* b_ptr;    /* [NumExperts, N, K], K contiguous (stride_B = K), or pre-shuffled (b_shuffle) */
     void* c_ptr;          /* bf16 (fp16 with fp16 operands); gate+up: [NumTokens * TopK, stride_C] (N/2 columns); down: [NumTokens, stride_C] */
     int32_t NumTokens;
     int32_t NumExperts;
@@ -358,6 +358,11 @@ typedef struct mi355_moe_flatmm_args
     int32_t activation;   /* mi355_moe_flatmm_activation (gate GEMMs) */
     float swiglu_alpha;   /* 1.702 in ck_tile's default */
     float swiglu_limit;   /* 7.0 in ck_tile's default */
+    int32_t b_shuffle;    /* layout of B: 0 = rows of K elements; 1 = what ck_tile::shuffle_b gives a flatmm kernel with
+                             N_Warp_Tile = 16 and 64 bytes of K per warp tile (host/tensor_shuffle_utils.hpp:26-68:
+                             [n/16][k bytes/64][4][16][16 bytes], the b_nr_kr_kw_nw_kv of the fused kernel), read in
+                             place; needs K rows of whole 64-byte blocks, N a multiple of 16 and no k_padded_zeros.
+                             Other warp tiles: convert once with mi355_moe_permute_weights */
 } mi355_moe_flatmm_args;
 
 /* bytes of the mi355_moe_workspace for this call; 0 when the arguments have no kernel */

@@ -78,6 +78,13 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     assert np.isnan(yg[T * K:]).all() and not np.isnan(yg[:T * K]).any()
     assert _rel(yg[:T * K], oracle.to_f32(y_ref, odt)) <= tol
 
+    # the same with B as ck_tile::shuffle_b hands it to a flatmm kernel (16-row warp tiles): read in place, same bits
+    y2 = torch.full_like(y, float("nan"))
+    assert ta.moe_flatmm(ta.GEMM1_GATE_UP, x, ta.permute_weights(g), y2, d_ids, d_eid, d_tot, T, K, unit, scale_m=d_sa,
+                         scale_n=d_sg, b_shuffle=1) == 0.0
+    torch.cuda.synchronize()
+    assert torch.equal(y[:T * K].view(torch.int16), y2[:T * K].view(torch.int16))
+
     # gate only: the gate half of the same weights on their own, c = silu(a b^T)
     g_only = g[:, :I].contiguous()
     yo = torch.full((T * K + 3, I), float("nan"), dtype=cdt, device="cuda")
@@ -102,10 +109,15 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     c0 = (rng.standard_normal((T, H)) * 0.1).astype(np.float32)
     c = bf(c0)
     c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, a_ref, dr, _bits(c).copy(), T, K, s_m, sd, c_dtype=odt)
+    c2 = c.clone()
     assert ta.moe_flatmm(ta.GEMM2, y_in, d, c, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w, scale_m=d_sm,
                          scale_n=d_sd) == 0.0
     torch.cuda.synchronize()
     assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, odt)) <= tol
+    assert ta.moe_flatmm(ta.GEMM2, y_in, ta.permute_weights(d), c2, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w,
+                         scale_m=d_sm, scale_n=d_sd, b_shuffle=1) == 0.0
+    torch.cuda.synchronize()
+    assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
 
 
 @pytest.mark.parametrize("T,E,K,H,I,unit", [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (1024, 4, 2, 512, 384, 32)])

@@ -79,7 +79,7 @@ class FlatmmArgs(C.Structure):
         ("stride_C", C.c_int32), ("n_padded_zeros", C.c_int32), ("k_padded_zeros", C.c_int32),
         ("scale_m", C.c_void_p), ("scale_n", C.c_void_p), ("exp_bias", C.c_void_p), ("prec_a", C.c_int32),
         ("prec_b", C.c_int32), ("block_m", C.c_int32), ("activation", C.c_int32), ("swiglu_alpha", C.c_float),
-        ("swiglu_limit", C.c_float),
+        ("swiglu_limit", C.c_float), ("b_shuffle", C.c_int32),
     ]
 
 

@@ -920,6 +920,14 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
                     a.k_padded_zeros, a.K);
     if(a.activation != MI355_MOE_ACT_SILU && a.activation != MI355_MOE_ACT_SWIGLU)
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: activation %d (0 = MoeSilu, 1 = Swiglu)", a.activation);
+    {
+        const int64_t b_b = (a.prec_b == MI355_MOE_BF16 || a.prec_b == MI355_MOE_FP16) ? 2 : 1;
+        if(a.b_shuffle != 0 && (a.b_shuffle != 1 || (a.K * b_b) % 64 != 0 || a.N % 16 != 0 || a.k_padded_zeros != 0 ||
+                                (int64_t)a.N * a.K * b_b >= ((int64_t)1 << 32)))
+            return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: b_shuffle=%d needs K rows of whole 64-byte blocks, N a "
+                                                 "multiple of 16, no k_padded_zeros and experts below 4 GiB (N=%d K=%d)",
+                        a.b_shuffle, a.N, a.K);
+    }
     L.hidden = g1 ? a.K : a.N;
     L.inter  = g1 ? (go ? a.N : a.N / 2) : a.K;
     if(L.hidden % 32 != 0 || L.inter % 32 != 0 || (f8 && !g1 && L.inter % 128 != 0))
@@ -1036,6 +1044,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     p.w              = static_cast<const unsigned char*>(a.b_ptr);
     p.w_row_bytes    = (int64_t)a.K * b_b;
     p.w_expert_bytes = (int64_t)a.N * a.K * b_b;
+    p.w_permuted     = a.b_shuffle;
     p.w_scale        = (w8 || f8) ? static_cast<const float*>(a.scale_n) : nullptr;
     p.k_bytes_x      = (a.K - a.k_padded_zeros) * a_b;
     p.k_bytes_w      = (a.K - a.k_padded_zeros) * b_b;

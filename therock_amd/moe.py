@@ -236,7 +236,8 @@ ACT_SILU, ACT_SWIGLU = 0, 1
 
 
 def _flatmm_args(kind, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens, topk, block_m, sorted_weights,
-                 scale_m, scale_n, exp_bias, activation, swiglu_alpha, swiglu_limit, n_padded_zeros, k_padded_zeros):
+                 scale_m, scale_n, exp_bias, activation, swiglu_alpha, swiglu_limit, n_padded_zeros, k_padded_zeros,
+                 b_shuffle=0):
     import torch
 
     experts, n, k = b.shape
@@ -245,7 +246,7 @@ def _flatmm_args(kind, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens
                            _ptr(c), num_tokens, experts, topk, 1, sorted_ids.numel(), n, k, a.stride(0), k, c.stride(0),
                            n_padded_zeros, k_padded_zeros, _ptr(scale_m), _ptr(scale_n), _ptr(exp_bias),
                            _lib.DTYPES[dt[a.dtype]], _lib.DTYPES[dt[b.dtype]], block_m, activation, swiglu_alpha,
-                           swiglu_limit)
+                           swiglu_limit, b_shuffle)
 
 
 def moe_flatmm_get_workspace_size(kind: int, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens: int, topk: int,
@@ -259,7 +260,7 @@ def moe_flatmm_get_workspace_size(kind: int, a, b, c, sorted_ids, sorted_eid, ma
 def moe_flatmm(kind: int, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens: int, topk: int, block_m: int,
                sorted_weights=None, scale_m=None, scale_n=None, exp_bias=None, activation: int = ACT_SILU,
                swiglu_alpha: float = 1.702, swiglu_limit: float = 7.0, n_padded_zeros: int = 0, k_padded_zeros: int = 0,
-               workspace=None, stream=None):
+               workspace=None, stream=None, b_shuffle: int = 0):
     """One grouped GEMM of the MoE layer as its own launch (ck_tile's MoeFlatmm conventions): kind
     GEMM1_GATE_UP writes c[token * topk + slot, :N/2] = act(gate, up), GEMM1_GATE_ONLY c[.., :N] = act(a b^T),
     kind GEMM2 adds the weighted down projection of a[token * topk + slot] to c[token].  b is [experts, N, K].
@@ -269,7 +270,8 @@ def moe_flatmm(kind: int, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tok
     import torch
 
     args = _flatmm_args(kind, a, b, c, sorted_ids, sorted_eid, max_token_id, num_tokens, topk, block_m, sorted_weights,
-                        scale_m, scale_n, exp_bias, activation, swiglu_alpha, swiglu_limit, n_padded_zeros, k_padded_zeros)
+                        scale_m, scale_n, exp_bias, activation, swiglu_alpha, swiglu_limit, n_padded_zeros, k_padded_zeros,
+                        b_shuffle)
     lib = _lib.load()
     if workspace is None:
         if stream is not None and _stream(stream) != _stream(None):
