@@ -195,6 +195,24 @@ def ck_permute_weights(w: np.ndarray, nw: int, kw: int, kv: int) -> np.ndarray:
     return out.view(w.dtype).reshape(e, n, k)
 
 
+def ck_shuffle_b(w, n_warp, k_warp):
+    """ck_tile::shuffle_b on every expert of w [e, n, k] (1- or 2-byte elements) for a GemmConfig with the warp tile
+    n_warp x k_warp (elements); None when oracle/_ref is not built."""
+    r = ck_ref()
+    if r is None:
+        return None
+    e, n, k = w.shape
+    b = np.ascontiguousarray(w)
+    out = np.empty_like(b)
+    for i in range(e):
+        src, dst = b[i], out[i]
+        rc = r.ck_ref_shuffle_b(_p(src), C.c_int32(n), C.c_int32(k), C.c_int32(w.itemsize), C.c_int32(n_warp),
+                                C.c_int32(k_warp), _p(dst))
+        if rc != 0:
+            raise ValueError("ck_ref_shuffle_b: no instance for this warp tile")
+    return out
+
+
 def smoothquant(x, smscale, topk_ids, dt):
     """MoE smooth-quant oracle: fp32 x [T,H], smscale [E,H], topk_ids [T,K] -> (qy [K,T,H], yscale [K,T])."""
     x, smscale, topk_ids = _c(x, np.float32), _c(smscale, np.float32), _c(topk_ids, np.int32)

@@ -21,6 +21,8 @@
 #include "ck_tile/host/reference/reference_topk.hpp"
 #include "ck_tile/host/reference/reference_rowwise_quantization2d.hpp"
 #include "ck_tile/host/reference/reference_permute.hpp"
+#include "ck_tile/host/device_prop.hpp"
+#include "ck_tile/host/tensor_shuffle_utils.hpp"
 
 
 using ck_tile::HostTensor;
@@ -70,6 +72,21 @@ int run_fused(const void* a, const void* g, const void* d, void* o_bf16,
         gate_only);
     std::memcpy(o_bf16, o_h.data(), sizeof(uint16_t) * (std::size_t)T * H);
     return 0;
+}
+
+template <int NW, int KW>
+struct WarpTile
+{
+    static constexpr int N_Warp_Tile = NW;
+    static constexpr int K_Warp_Tile = KW;
+};
+template <typename T, int NW, int KW>
+void shuffle_b_into(const void* x, int32_t n, int32_t k, void* y)
+{
+    // (shuffle_b reads the lengths as [k, n] and copies the elements in storage order, n-major)
+    auto t = make_tensor<T>({(std::size_t)k, (std::size_t)n}, x);
+    auto s = ck_tile::shuffle_b<WarpTile<NW, KW>>(t);
+    std::memcpy(y, s.data(), sizeof(T) * (std::size_t)n * k);
 }
 
 } // namespace
@@ -198,6 +215,23 @@ ck_ref_permute_b_nr_kr_kw_nw_kv(const uint8_t* x, int32_t e, int32_t nr, int32_t
                                      (std::size_t)kv_bytes}, x);
     auto y_h = ck_tile::reference_permute(x_h, {0, 1, 3, 4, 2, 5});
     std::memcpy(y, y_h.data(), (std::size_t)e * nr * nw * kr * kw * kv_bytes);
+    return 0;
+}
+
+// ck_tile::shuffle_b (host/tensor_shuffle_utils.hpp:26-68), what a flatmm caller applies to B before the call, for
+// one [n, k] matrix of 1-byte or 2-byte elements and a GemmConfig with the given warp tile (16 x 32 or 32 x 16
+// elements for 2-byte types, 16 x 64 for 1-byte types).  Without a device the gfx9 branch runs, which is gfx950's.
+__attribute__((visibility("default"))) int
+ck_ref_shuffle_b(const void* x, int32_t n, int32_t k, int32_t elem_bytes, int32_t n_warp, int32_t k_warp, void* y)
+{
+    if(elem_bytes == 2 && n_warp == 16 && k_warp == 32)
+        shuffle_b_into<uint16_t, 16, 32>(x, n, k, y);
+    else if(elem_bytes == 2 && n_warp == 32 && k_warp == 16)
+        shuffle_b_into<uint16_t, 32, 16>(x, n, k, y);
+    else if(elem_bytes == 1 && n_warp == 16 && k_warp == 64)
+        shuffle_b_into<uint8_t, 16, 64>(x, n, k, y);
+    else
+        return -1;
     return 0;
 }
 

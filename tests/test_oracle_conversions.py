@@ -217,3 +217,19 @@ def test_weight_permutation(dtype, nw, kw, kv):
     assert np.array_equal(oracle.permute_weights(p, nw, kw, kv, inverse=True), w)
     if oracle.ck_ref() is not None:
         assert np.array_equal(p, oracle.ck_permute_weights(w, nw, kw, kv))
+
+
+@pytest.mark.parametrize("dtype,n_warp,k_warp,view", [(np.uint16, 16, 32, (16, 4, 8)), (np.uint8, 16, 64, (16, 4, 16)),
+                                                      (np.uint16, 32, 16, (32, 2, 8))])
+def test_preshuffled_layout_is_ck_tile_shuffle_b(dtype, n_warp, k_warp, view):
+    """The layout the GEMM kernels read in place (weight_permute / b_shuffle = 1: nw 16, kw 4, 16-byte kv) is what
+    ck_tile::shuffle_b (host/tensor_shuffle_utils.hpp:26-68) produces for 16-row warp tiles with 64 bytes of K, for
+    2-byte and for 1-byte elements; a 32-row warp tile gives another member of the family (nw 32, kw 2), which the
+    permutation tool covers and the kernels do not read."""
+    rng = np.random.Generator(np.random.Philox(9))
+    w = rng.integers(0, np.iinfo(dtype).max, size=(3, 2 * n_warp * 2, 4 * k_warp * 4), dtype=dtype)
+    want = oracle.ck_shuffle_b(w, n_warp, k_warp)
+    if want is None:
+        pytest.skip("oracle/_ref/libck_ref.so not built (ck_tile headers absent)")
+    assert np.array_equal(oracle.permute_weights(w, *view), want)
+    assert not np.array_equal(want, w)
