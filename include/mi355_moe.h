@@ -160,9 +160,9 @@ typedef struct mi355_fused_moe_traits
                                read either layout in place (mi355_moe_permute_weights converts between them) */
 } mi355_fused_moe_traits;
 
-/* FusedMoeGemmHostArgs (fused_moegemm_kernel.hpp:97-120), field for field.  Weights are plain row-major,
- * K contiguous (what ck_tile's host reference takes; FusedMoeGemmWeightPermuteEnum::no_permute,
- * fused_moegemm_traits.hpp:10-17); mi355_moe_permute_weights converts pre-shuffled checkpoints. */
+/* FusedMoeGemmHostArgs (fused_moegemm_kernel.hpp:97-120), field for field.  g and d in the layout that
+ * mi355_fused_moe_traits.weight_permute names: rows of K elements (what ck_tile's host reference takes) or
+ * ck_tile's pre-shuffled b_nr_kr_kw_nw_kv (what its device kernel takes; fused_moegemm_traits.hpp:10-17). */
 typedef struct mi355_fused_moegemm_args
 {
     const void* a_ptr;              /* [tokens, stride_token] activations ([topk, tokens, stride_token] with fused_quant 1) */
