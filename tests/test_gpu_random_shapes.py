@@ -73,6 +73,20 @@ def test_random_shapes(dtype):
         check(cfg, seed=1000 + case, mask=mask, **kw)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
+def test_random_shapes_preshuffled_weights(dtype):
+    """The same draw with g and d in ck_tile's pre-shuffled layout (rows of whole 64-byte blocks), against the oracle."""
+    rng = np.random.default_rng({"bf16": 111, "fp8": 222, "int8": 333}[dtype])
+    for case in range(16):
+        cfg = (draw_many_rows if case % 4 == 3 else draw)(rng, dtype)
+        if dtype != "bf16":
+            cfg = cfg.scaled(hidden=(cfg.hidden + 63) // 64 * 64, inter=(cfg.inter + (127 if dtype == "fp8" else 63)) // (128 if dtype == "fp8" else 64) * (128 if dtype == "fp8" else 64))
+        if dtype == "fp8" and cfg.tokens * cfg.topk < 16:
+            cfg = cfg.scaled(tokens=max(cfg.tokens, 16 // cfg.topk + 1))
+        kw = {0: {}, 1: {"unfused": True}, 2: {"activation": 0}, 3: {"gate_only": 1}, 4: {"stride_pad": 64}}[int(rng.integers(0, 5))]
+        check(cfg, seed=5000 + case, weight_permute=1, **kw)
+
+
 def test_random_shapes_fp16():
     from tests.test_gpu_fused_moe import check_fp16
     rng = np.random.default_rng(404)
