@@ -193,6 +193,9 @@ def test_skewed_fp8_batch_takes_the_large_tiles_on_the_device():
     run(mi.MoeConfig("skew", 192, 512, 2048, 64, 4, "fp8", "zipf", unit=16), 4, 320)   # 16-row sort units, ragged tiles
     run(mi.MoeConfig("skew", 256, 512, 4096, 64, 4, "fp8", "zipf"), 5, 320, gate_only=1)  # (half the column tiles per expert)
     run(zipf, 6, 320, mask=np.array(([1, 1, 1, 1, 1, 1, 1, 0] * 8), dtype=np.int32))
+    # 512 experts: the multi-phase sort (count / scan / scatter kernels) makes the same choice
+    run(mi.MoeConfig("skew", 1024, 256, 2048, 512, 4, "fp8", "zipf"), 7, 320)
+    run(mi.MoeConfig("skew", 1024, 256, 2048, 512, 4, "fp8", "softmax_renorm"), 8, 32)
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
