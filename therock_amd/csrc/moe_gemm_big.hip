@@ -124,7 +124,14 @@ __device__ inline void wait_vmcnt()
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int MODE, bool GEMM0>
+// WPERM: the weights are in ck_tile's pre-shuffled layout, where 128 contiguous bytes are one 16-byte chunk of eight
+// consecutive rows.  The eight rows x eight chunks of a weight DMA instruction then sit in LDS chunk-major - lane
+// 8 c' + r fetches chunk c' ^ s of row r, s = bit 1 of the instruction's number, and lands at byte 128 c' + 16 r of
+// the instruction's 1 KiB - so that eight consecutive lanes fetch one whole line, as they do for row-major weights
+// in the row-major LDS layout (eight chunks of one row).  The operand fetches of sixteen lanes (rows 0..7 of one
+// instruction, rows 16..23 of the one two further on, same chunk) cover 256 contiguous bytes modulo the bank span
+// thanks to s.
+template <int MODE, bool GEMM0, bool WPERM>
 __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmParams p)
 {
     using MT  = ModeTraits<MODE>;
@@ -196,11 +203,12 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
 #pragma unroll
             for(int j = 0; j < 4; j++)
             {
-                const int rih    = (q4 + 4 * j) * 8 + (lane >> 3); // LDS row inside the half
+                const int inst   = q4 + 4 * j;                      // instruction of the unit: LDS rows 8 inst .. + 7
+                const int rih    = inst * 8 + (WPERM ? lane & 7 : lane >> 3); // LDS row inside the half
                 const int trow   = h * kWHalfRows + rih;
                 const int blk    = trow >> 5;
                 const int c      = trow & 31; // LDS row r of a 32-row block holds weight channel r (see weight_row_swizzle)
-                const int cchunk = (lane & 7) ^ weight_row_swizzle(rih);
+                const int cchunk = WPERM ? (lane >> 3) ^ ((inst >> 1) & 1) : (lane & 7) ^ weight_row_swizzle(rih);
                 int grow;
                 if(paired)
                     grow = (blk & 1) * p.n_out + min(n_base + (blk >> 1) * 32 + c, p.n_out - 1);
@@ -373,9 +381,10 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     // per-lane LDS read offsets (swizzled chunk positions are per-lane constants)
     const int sw_w  = (r32 >> 1) & 7; // 128-byte token rows of the gate+up GEMM
     const int w_row = chan_of_row(r32); // LDS row that holds the channel of this lane's MFMA row
-    const int sw_wr = weight_row_swizzle(w_row);
+    const int sw_wr = WPERM ? (w_row >> 4) & 1 : weight_row_swizzle(w_row);
+    constexpr int kWChunkB = WPERM ? 128 : 16; // LDS bytes between two chunks of a weight row
     const int sw_x  = (r32 >> 2) & 3; // 64-byte token rows
-    const int w_off = ((ww & 1) * 64 + w_row) * (2 * kStepKB);
+    const int w_off = WPERM ? ((ww & 1) * 8 + (w_row >> 3)) * 1024 + (w_row & 7) * 16 : ((ww & 1) * 64 + w_row) * (2 * kStepKB);
     const int w_h   = ww >> 1;
     const int x_off = kXOffset + (wt * 32 + r32) * kStepKB;
 
@@ -395,8 +404,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 constexpr int P          = decltype(p_tag)::value;
                 constexpr int kh         = P * 4; // first chunk of the step inside the 128-byte weight row
                 const unsigned char* wp  = lds + (((kk & ~1) + w_h) % kWS) * kWUnitBytes + w_off + b * 32 * (2 * kStepKB);
-                const int cw_lo          = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_wr) * 16 : ((kh + kg) ^ sw_wr) * 16;
-                const int cw_hi          = ((kh + 2 + kg) ^ sw_wr) * 16;
+                const int cw_lo          = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_wr) * kWChunkB : ((kh + kg) ^ sw_wr) * kWChunkB;
+                const int cw_hi          = ((kh + 2 + kg) ^ sw_wr) * kWChunkB;
                 Frag f;
                 f.lo = *reinterpret_cast<const uint4*>(wp + cw_lo);
                 if constexpr(kOpB == 32)
@@ -591,8 +600,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                 uint32_t xs[NF];
                 const int cx_lo = kOpB == 16 ? ((2 * s + kg) ^ sw_x) * 16 : (kg ^ sw_x) * 16;
                 const int cx_hi = ((2 + kg) ^ sw_x) * 16;
-                const int cw_lo = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_wr) * 16 : ((kh + kg) ^ sw_wr) * 16;
-                const int cw_hi = ((kh + 2 + kg) ^ sw_wr) * 16;
+                const int cw_lo = kOpB == 16 ? ((kh + 2 * s + kg) ^ sw_wr) * kWChunkB : ((kh + kg) ^ sw_wr) * kWChunkB;
+                const int cw_hi = ((kh + 2 + kg) ^ sw_wr) * kWChunkB;
 #pragma unroll
                 for(int b = 0; b < 2; b++)
                 {
@@ -600,7 +609,7 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
                     if constexpr(kW8)
                     {
                         // 8 int8 of this lane's K group: 16-byte chunk (k & 3) * 2 + s of the row, half kg
-                        const int c8 = ((((k & 3) << 1) + s) ^ sw_wr) * 16 + kg * 8;
+                        const int c8 = ((((k & 3) << 1) + s) ^ sw_wr) * kWChunkB + kg * 8;
                         wf[b].lo     = int8x8_to_bf16x8(*reinterpret_cast<const uint2*>(wp + c8));
                     }
                     else
@@ -677,8 +686,8 @@ __global__ __launch_bounds__(kBigThreads) void moe_gemm_big_kernel(const GemmPar
     run_epilogue<MODE, GEMM0, kMaxNB, false>(p, acc, expert, row0, nrows, wt * 32, 64, nb_w, n_base, ww, r32, kg);
 }
 
-template <int MODE, bool GEMM0>
-int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
+template <int MODE, bool GEMM0, bool WPERM>
+int launch_big_w(const GemmParams& p, int max_tiles, hipStream_t stream)
 {
     constexpr bool kMx  = MODE == kFp8 && !GEMM0;
     const size_t lds    = (GEMM0 && MODE != kBf16W8) ? kLdsBytesPair : kMx ? kLdsBytes : kYsOffset;
@@ -688,7 +697,7 @@ int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
     (void)hipGetDevice(&dev);
     if(dev < 0 || dev >= 64 || !attr_ok[dev])
     {
-        MI355_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_big_kernel<MODE, GEMM0>),
+        MI355_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_big_kernel<MODE, GEMM0, WPERM>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         if(dev >= 0 && dev < 64)
             attr_ok[dev] = true;
@@ -697,9 +706,15 @@ int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
     if(grid <= 0)
         return MI355_MOE_OK;
     KernelTimer timer(GEMM0 ? MI355_MOE_K_GEMM0 : MI355_MOE_K_GEMM1, stream);
-    hipLaunchKernelGGL((moe_gemm_big_kernel<MODE, GEMM0>), dim3(grid), dim3(kBigThreads), lds, stream, p);
+    hipLaunchKernelGGL((moe_gemm_big_kernel<MODE, GEMM0, WPERM>), dim3(grid), dim3(kBigThreads), lds, stream, p);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
+}
+
+template <int MODE, bool GEMM0>
+int launch_big_t(const GemmParams& p, int max_tiles, hipStream_t stream)
+{
+    return p.w_permuted ? launch_big_w<MODE, GEMM0, true>(p, max_tiles, stream) : launch_big_w<MODE, GEMM0, false>(p, max_tiles, stream);
 }
 
 } // namespace

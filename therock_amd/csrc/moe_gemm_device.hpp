@@ -7,6 +7,9 @@
 
 namespace mi355 {
 namespace gemm {
+// Every device function below is forced inline: with several instantiations of a kernel in one translation unit
+// the inliner leaves the larger ones out of line, and their array arguments (accumulators, GemmParams) then live
+// in scratch memory.
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
@@ -84,20 +87,20 @@ struct GemmParams
 };
 
 // row of the gate+up GEMM's activations (and index of its per-row scale) a sorted id refers to
-__device__ inline uint32_t token_row(const GemmParams& p, int sid)
+__device__ __attribute__((always_inline)) inline uint32_t token_row(const GemmParams& p, int sid)
 {
     const uint32_t tok = static_cast<uint32_t>(sid) & 0xffffffu;
     return p.x_slot_major ? (static_cast<uint32_t>(sid) >> 24) * static_cast<uint32_t>(p.tokens) + tok : tok;
 }
 
 // byte offset of K byte kb of row `row` in the slab-major Y layout
-__device__ inline int64_t y_slab_offset(int64_t row, int kb, int segs)
+__device__ __attribute__((always_inline)) inline int64_t y_slab_offset(int64_t row, int kb, int segs)
 {
     return (((row >> 4) * segs + (kb >> 6)) << 10) + ((row & 15) << 6) + (kb & 63);
 }
 
 // row of a [tokens * topk, .] buffer a sorted id refers to
-__device__ inline int64_t slot_row(int sid, int topk)
+__device__ __attribute__((always_inline)) inline int64_t slot_row(int sid, int topk)
 {
     return (int64_t)(sid & 0xffffff) * topk + static_cast<int>(static_cast<uint32_t>(sid) >> 24);
 }
@@ -106,13 +109,13 @@ __device__ inline int64_t slot_row(int sid, int topk)
 // into a window of K that begins on a multiple of 64 bytes; and what moving that window by `bytes` (a multiple of
 // 64) adds to it.  Row-major: row * row_bytes + 16 * chunk16, + bytes.  Pre-shuffled: the row's block row, the block
 // (chunk16 / 4) of the window, the piece inside the block; a window 64 bytes further on is the next 1 KiB block.
-__device__ inline uint32_t weight_offset(const GemmParams& p, int row, int chunk16)
+__device__ __attribute__((always_inline)) inline uint32_t weight_offset(const GemmParams& p, int row, int chunk16)
 {
     if(p.w_permuted == 0)
         return (uint32_t)row * (uint32_t)p.w_row_bytes + chunk16 * 16;
     return (uint32_t)(row >> 4) * (uint32_t)(p.w_row_bytes * 16) + (chunk16 >> 2) * 1024 + (chunk16 & 3) * 256 + (row & 15) * 16;
 }
-__device__ inline int weight_k_advance(const GemmParams& p, int bytes) { return p.w_permuted == 0 ? bytes : bytes * 16; }
+__device__ __attribute__((always_inline)) inline int weight_k_advance(const GemmParams& p, int bytes) { return p.w_permuted == 0 ? bytes : bytes * 16; }
 
 // Work item -> tile.  Workgroup ids are dealt round-robin to the 8 XCDs; inside an expert the row tiles of one
 // weight tile are adjacent.  One entry of the list describes the whole expert, so a single load resolves any of
@@ -130,7 +133,7 @@ struct TileRef
 // tile_rows != 0: the launch is one of two candidates and runs only if the sort built the list for its tile height
 // (tile_map[1]); the other candidate's workgroups all leave at once.
 template <bool CHUNKED = false>
-__device__ inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_ntiles, int max_tiles, int block,
+__device__ __attribute__((always_inline)) inline TileRef lookup_tile(const int* __restrict__ tile_map, int n_ntiles, int max_tiles, int block,
                                       int tile_rows = 0)
 {
     TileRef t;
@@ -217,11 +220,11 @@ struct ModeTraits<kBf16W8>
 // consecutive channels 16*(l/32) .. +15 of its token in registers 0..15.
 __device__ __host__ constexpr int chan_of_row(int m) { return 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3); }
 
-__device__ inline float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+__device__ __attribute__((always_inline)) inline float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 // Gelu in the erf form of ck_tile::element_wise::Gelu (unary_element_wise_operation.hpp:975-986):
 // x * Phi(x) with erfc(z) = poly(t) * exp(-z^2), t = 1 / (1 + 0.3275911 z) (Abramowitz & Stegun 7.1.26,
 // absolute error of erf <= 1.5e-7), branch-free and free of cancellation in the negative tail
-__device__ inline float gelu(float x)
+__device__ __attribute__((always_inline)) inline float gelu(float x)
 {
     const float z = fabsf(x) * 0.70710678118f;
     const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
@@ -231,7 +234,7 @@ __device__ inline float gelu(float x)
 }
 
 // 8 int8 (two dwords) -> 8 bf16 (exact: |v| <= 128 fits bf16's 8 significant bits)
-__device__ inline uint4 int8x8_to_bf16x8(uint2 v)
+__device__ __attribute__((always_inline)) inline uint4 int8x8_to_bf16x8(uint2 v)
 {
     uint4 r;
     uint32_t d[2] = {v.x, v.y};
@@ -255,7 +258,7 @@ __device__ inline uint4 int8x8_to_bf16x8(uint2 v)
 }
 
 template <typename To, typename From>
-__device__ inline To bit_cast_dev(const From& f)
+__device__ __attribute__((always_inline)) inline To bit_cast_dev(const From& f)
 {
     static_assert(sizeof(To) == sizeof(From), "size mismatch");
     To t;
@@ -269,7 +272,7 @@ struct Frag
 };
 
 template <int MODE>
-__device__ inline typename ModeTraits<MODE>::Acc mfma(const Frag& w, const Frag& x, uint32_t x_scale,
+__device__ __attribute__((always_inline)) inline typename ModeTraits<MODE>::Acc mfma(const Frag& w, const Frag& x, uint32_t x_scale,
                                                       typename ModeTraits<MODE>::Acc c)
 {
     if constexpr(MODE == kBf16 || MODE == kBf16W8)
@@ -302,7 +305,7 @@ __device__ inline typename ModeTraits<MODE>::Acc mfma(const Frag& w, const Frag&
 
 // e4m3 x e4m3 without block scales (both scale operands literal 0 select the unscaled encoding,
 // which issues faster than the scaled one)
-__device__ inline f32x16_t mfma_fp8_unscaled(const Frag& w, const Frag& x, f32x16_t c)
+__device__ __attribute__((always_inline)) inline f32x16_t mfma_fp8_unscaled(const Frag& w, const Frag& x, f32x16_t c)
 {
     i32x8_t a, b;
     a[0] = w.lo.x; a[1] = w.lo.y; a[2] = w.lo.z; a[3] = w.lo.w;
@@ -314,7 +317,7 @@ __device__ inline f32x16_t mfma_fp8_unscaled(const Frag& w, const Frag& x, f32x1
 
 // two results -> the 16-bit type the mode stores (fp16 for kF16, bf16 otherwise), both round to nearest even
 template <int MODE>
-__device__ inline uint32_t pack_out2(float lo, float hi)
+__device__ __attribute__((always_inline)) inline uint32_t pack_out2(float lo, float hi)
 {
     if constexpr(MODE == kF16)
         return pack_f16x2(lo, hi);
@@ -330,7 +333,7 @@ __device__ inline uint32_t pack_out2(float lo, float hi)
 // one batch right after the K loop, so that their latencies overlap instead of adding up.
 
 // per-channel scales of the 16 channels a lane owns (1.0 when the path is unscaled)
-__device__ inline void load_channel_scales(const float* scale, float (&out)[16])
+__device__ __attribute__((always_inline)) inline void load_channel_scales(const float* scale, float (&out)[16])
 {
     if(scale != nullptr)
     {
@@ -352,7 +355,7 @@ __device__ inline void load_channel_scales(const float* scale, float (&out)[16])
 
 // ck_tile::moe::Swiglu (moe_flatmm_kernel.hpp:149-183, device branch): gate' = min(gate, limit),
 // linear' = clamp(linear, -limit, limit), gate' * rcp(1 + exp(-alpha * gate')) * (linear' + 1)
-__device__ inline float swiglu(float gate, float linear, float alpha, float limit)
+__device__ __attribute__((always_inline)) inline float swiglu(float gate, float linear, float alpha, float limit)
 {
     gate   = fminf(gate, limit);
     linear = fminf(fmaxf(linear, -limit), limit);
@@ -363,7 +366,7 @@ __device__ inline float swiglu(float gate, float linear, float alpha, float limi
 // inside the expert's weight): v = dot * scale, then the padded channels lose their dot product and every
 // channel gains its bias.  Rare (a uniform branch at the call sites), so the bias is fetched here rather than
 // carried in registers beside the scales.
-__device__ inline void bias_and_padding(const GemmParams& p, float (&v)[16], int expert, int chan0)
+__device__ __attribute__((always_inline)) inline void bias_and_padding(const GemmParams& p, float (&v)[16], int expert, int chan0)
 {
     if(p.n_padded > 0)
     {
@@ -389,7 +392,7 @@ __device__ inline void bias_and_padding(const GemmParams& p, float (&v)[16], int
 // the writes.  single: gate-only weights, y = act(gate) (swiglu: act(gate, 1)) and the up operands are ignored.
 // col0: first of the lane's 16 output columns = first gate channel; the up channels are n_out + col0 ...
 template <int MODE>
-__device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc_gate,
+__device__ __attribute__((always_inline)) inline void epilogue_gemm0(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc_gate,
                                       const typename ModeTraits<MODE>::Acc& acc_up, const float (&gs)[16],
                                       const float (&us)[16], float sa, int64_t grow, bool store, int col0, int kg,
                                       bool single = false, int expert = 0)
@@ -491,7 +494,7 @@ __device__ inline void epilogue_gemm0(const GemmParams& p, const typename ModeTr
 // gemm1: * per-channel scale (+ expert bias), bf16 partial row in sorted-row order (the combine applies the top-k weight)
 // (sa: per-row scale of a quantised Y, 1 otherwise)
 template <int MODE>
-__device__ inline void epilogue_gemm1(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc,
+__device__ __attribute__((always_inline)) inline void epilogue_gemm1(const GemmParams& p, const typename ModeTraits<MODE>::Acc& acc,
                                       const float (&ds)[16], float sa, int64_t prow, bool store, int col0, int expert = 0)
 {
     float y[16];
@@ -540,7 +543,7 @@ struct EpilogueOperands
 };
 
 template <bool GEMM0>
-__device__ inline EpilogueColumns epilogue_columns(const GemmParams& p, int n_base, int wblk, int kg)
+__device__ __attribute__((always_inline)) inline EpilogueColumns epilogue_columns(const GemmParams& p, int n_base, int wblk, int kg)
 {
     // gate+up tiles pair weight block 2w (gate) with 2w+1 (up) on the same 32 columns; every other kind of
     // tile (down, gate-only) maps its blocks 2w and 2w+1 to consecutive groups of 32 columns
@@ -554,7 +557,7 @@ __device__ inline EpilogueColumns epilogue_columns(const GemmParams& p, int n_ba
 }
 
 template <int MODE, bool GEMM0, int NBLK, bool SKIP_PAD>
-__device__ inline void load_epilogue_rows(const GemmParams& p, EpilogueRows<NBLK>& o, int row0, int nrows, int first_row,
+__device__ __attribute__((always_inline)) inline void load_epilogue_rows(const GemmParams& p, EpilogueRows<NBLK>& o, int row0, int nrows, int first_row,
                                           int row_step, int r32)
 {
 #pragma unroll
@@ -587,7 +590,7 @@ __device__ inline void load_epilogue_rows(const GemmParams& p, EpilogueRows<NBLK
 }
 
 template <int NBLK>
-__device__ inline void pin_epilogue_rows(EpilogueRows<NBLK>& o)
+__device__ __attribute__((always_inline)) inline void pin_epilogue_rows(EpilogueRows<NBLK>& o)
 {
 #pragma unroll
     for(int i = 0; i < NBLK; i++)
@@ -599,7 +602,7 @@ __device__ inline void pin_epilogue_rows(EpilogueRows<NBLK>& o)
 }
 
 template <int MODE, bool GEMM0, int NBLK, bool SKIP_PAD>
-__device__ inline void load_epilogue(const GemmParams& p, EpilogueOperands<NBLK>& o, int expert, int row0, int nrows,
+__device__ __attribute__((always_inline)) inline void load_epilogue(const GemmParams& p, EpilogueOperands<NBLK>& o, int expert, int row0, int nrows,
                                      int first_row, int row_step, int n_base, int wblk, int r32, int kg)
 {
     o.cols             = epilogue_columns<GEMM0>(p, n_base, wblk, kg);
@@ -614,7 +617,7 @@ __device__ inline void load_epilogue(const GemmParams& p, EpilogueOperands<NBLK>
 // its result would make the compiler guard later register reuse with a wait for all vector memory
 // operations - inside the caller's K loop when the caller walks several tiles.
 template <int NBLK>
-__device__ inline void pin_epilogue(EpilogueOperands<NBLK>& o)
+__device__ __attribute__((always_inline)) inline void pin_epilogue(EpilogueOperands<NBLK>& o)
 {
 #pragma unroll
     for(int v = 0; v < 16; v++)
@@ -624,7 +627,7 @@ __device__ inline void pin_epilogue(EpilogueOperands<NBLK>& o)
 
 // one token block of a wave: scales, activation, packing, stores
 template <int MODE, bool GEMM0, int NBLK>
-__device__ inline void apply_epilogue_block(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[2],
+__device__ __attribute__((always_inline)) inline void apply_epilogue_block(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[2],
                                             const float (&sc0)[16], const float (&sc1)[16], const EpilogueRows<NBLK>& rows,
                                             const EpilogueColumns& c, int i, int row0, int nrows, int first_row,
                                             int row_step, int r32, int kg, int expert)
@@ -649,7 +652,7 @@ __device__ inline void apply_epilogue_block(const GemmParams& p, typename ModeTr
 }
 
 template <int MODE, bool GEMM0, int NBLK>
-__device__ inline void apply_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2],
+__device__ __attribute__((always_inline)) inline void apply_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2],
                                       const EpilogueOperands<NBLK>& o, int row0, int nrows, int first_row, int row_step,
                                       int nblk_live, int r32, int kg, int expert)
 {
@@ -666,7 +669,7 @@ __device__ inline void apply_epilogue(const GemmParams& p, typename ModeTraits<M
 }
 
 template <int MODE, bool GEMM0, int NBLK, bool SKIP_PAD>
-__device__ inline void run_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2], int expert,
+__device__ __attribute__((always_inline)) inline void run_epilogue(const GemmParams& p, typename ModeTraits<MODE>::Acc (&acc)[NBLK][2], int expert,
                                     int row0, int nrows, int first_row, int row_step, int nblk_live, int n_base,
                                     int wblk, int r32, int kg)
 {
