@@ -38,7 +38,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_workload(cfg, steps, warmup, seed=0, fused_quant=0, hot_expert=False):
+def run_workload(cfg, steps, warmup, seed=0, fused_quant=0, hot_expert=False, weight_permute=0):
     """Times `steps` passes of the path (fused_quant 2: the int8 path re-quantises the intermediate activations
     per row and runs the down GEMM on int8 MFMAs).  The dominant kernel's duration comes from HIP events the
     library records on the launch stream inside the timed region, the other kernels' from an untimed
@@ -55,7 +55,10 @@ def run_workload(cfg, steps, warmup, seed=0, fused_quant=0, hot_expert=False):
         ids = inp["topk_ids"].clone()
         ids[~(ids == 0).any(dim=1), cfg.topk - 1] = 0
         inp["topk_ids"] = ids.contiguous()
-    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit, fused_quant=fused_quant)
+    if weight_permute:  # g and d as ck_tile's example hands them to its kernel (b_nr_kr_kw_nw_kv), read in place
+        inp["g"], inp["d"] = ta.permute_weights(inp["g"]), ta.permute_weights(inp["d"])
+    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit, fused_quant=fused_quant,
+                                 weight_permute=weight_permute)
     buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, dev)
     args = ta.make_args(traits, buf, inp["a"], inp["g"], inp["d"], inp["topk_ids"], inp["topk_weight"],
                         a_scale=inp["a_scale"], g_scale=inp["g_scale"], d_scale=inp["d_scale"])
@@ -391,6 +394,10 @@ def main():
             # fp8: the sort sees ~40 active experts of ~70 rows and takes the 320-row tiles (the host's average says 8 rows)
             "cfg3_dsv3_fp8_t256_zipf": (mi.CONFIGS["cfg3_dsv3_fp8"].scaled(name="cfg3_dsv3_fp8_t256_zipf", tokens=256, router="zipf"), {}),
             "cfg4_decode_int8_t256_hot_expert": (i8.scaled(name="cfg4_decode_int8_t256_hot_expert"), {"hot_expert": True}),
+            # the headline workload and the decode workload with weights in ck_tile's pre-shuffled layout
+            "cfg3_dsv3_fp8_preshuffled": (mi.CONFIGS["cfg3_dsv3_fp8"].scaled(name="cfg3_dsv3_fp8_preshuffled"), {"weight_permute": 1}),
+            "cfg4_decode_int8_t64_preshuffled": (mi.CONFIGS["cfg4_decode_int8_t64"].scaled(name="cfg4_decode_int8_t64_preshuffled"),
+                                                 {"weight_permute": 1}),
         }
         for name, (c, kw) in cases.items():
             try:
