@@ -133,6 +133,18 @@ def test_flatmm_operand_types_on_the_host():
         assert b"operand types" in lib.mi355_moe_last_error()
     assert ws(1, "int8", "int8") > 0 and ws(2, "bf16", "int8") > 0 and ws(2, "int8", "int8") == 0
 
+    # B as ck_tile::shuffle_b lays it out for 16-row warp tiles: rows of whole 64-byte blocks, no padded K
+    def ws_shuffled(prec, K, b_shuffle=1, k_pad=0):
+        a = _lib.FlatmmArgs()
+        a.NumTokens, a.NumExperts, a.TopK, a.N, a.K, a.block_m, a.k_batch = 64, 4, 2, 256, K, 32, 1
+        a.prec_a = a.prec_b = D[prec]
+        a.b_shuffle, a.k_padded_zeros = b_shuffle, k_pad
+        return lib.mi355_moe_flatmm_workspace_size(1, C.byref(a))
+
+    assert ws_shuffled("bf16", 128) > 0 and ws_shuffled("int8", 128) > 0 and ws_shuffled("bf16", 96) > 0
+    assert ws_shuffled("int8", 96) == 0 and b"b_shuffle" in lib.mi355_moe_last_error()
+    assert ws_shuffled("bf16", 128, b_shuffle=2) == 0 and ws_shuffled("bf16", 128, k_pad=32) == 0
+
 
 def test_host_only_entry_points():
     lib = _lib.load()
