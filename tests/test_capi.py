@@ -188,10 +188,10 @@ def test_host_only_entry_points():
     assert rows(1, 32, 8192, 256, 8, 7168, 2048) == 320
     assert rows(1, 32, 1024, 256, 8, 7168, 2048) == 320 and rows(1, 32, 512, 256, 8, 7168, 2048) == 32
     assert rows(1, 8, 8192, 256, 8, 7168, 2048) == 128
-    # 28 .. 52 rows per expert: 64-row tiles of the decode kernel for 16-bit and int8 operands, 320-row tiles for fp8
+    # 28 .. 56 rows per expert: 64-row tiles of the decode kernel for 16-bit and int8 operands, 320-row tiles for fp8
     assert rows(2, 32, 640, 128, 8, 4096, 1536) == 64 and rows(0, 32, 160, 8, 2, 4096, 14336) == 64
     assert rows(2, 32, 448, 128, 8, 4096, 1536) == 64 and rows(2, 32, 432, 128, 8, 4096, 1536) == 32
-    assert rows(2, 32, 832, 128, 8, 4096, 1536) == 64 and rows(2, 32, 848, 128, 8, 4096, 1536) == 320
+    assert rows(2, 32, 896, 128, 8, 4096, 1536) == 64 and rows(2, 32, 912, 128, 8, 4096, 1536) == 320
     assert rows(1, 32, 1280, 256, 8, 7168, 2048) == 320
     assert rows(2, 32, 8192, 128, 8, 4096, 1536) == 320 and rows(2, 32, 8192, 128, 8, 4096, 1504) == 128
 

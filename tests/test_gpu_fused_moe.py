@@ -127,7 +127,7 @@ def test_decode_kernel_ragged(dtype):
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16", "int8"])
 def test_two_block_decode_tiles(dtype):
-    """28 .. 52 rows per expert with 16-bit or int8 operands: the decode kernel with two 32-row token blocks per
+    """28 .. 56 rows per expert with 16-bit or int8 operands: the decode kernel with two 32-row token blocks per
     tile (64-row tiles).  Ragged K depths and column tails, experts with more than 64 rows (two tiles) and with
     none, a sort unit that is not a multiple of 32, the expert mask, GELU and gate-only."""
     import therock_amd as ta
@@ -212,10 +212,10 @@ def test_many_rows_per_expert_with_small_sort_units(dtype):
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])
 def test_large_tile_kernel_partial_tiles(dtype):
-    # from about 28 (fp8) or 53 (other types) rows per expert on, and with enough tiles to fill the chip, the 320-row
+    # from about 28 (fp8) or 57 (other types) rows per expert on, and with enough tiles to fill the chip, the 320-row
     # kernel runs with mostly empty tiles: it then fetches only the 64-row slab groups a tile has (1 to 5 per step)
     import therock_amd as ta
-    for cfg, seed in ((mi.MoeConfig("p", 640 if dtype == "fp8" else 900, 256, 512, 64, 4, dtype, "softmax_renorm"), 1),
+    for cfg, seed in ((mi.MoeConfig("p", 640 if dtype == "fp8" else 960, 256, 512, 64, 4, dtype, "softmax_renorm"), 1),
                       (mi.MoeConfig("p", 1500, 256, 512, 64, 4, dtype, "zipf"), 2),
                       (mi.MoeConfig("p", 4000, 384, 512, 64, 6, dtype, "zipf", unit=64), 3)):
         traits = ta.fused_moe_traits(prec_i=dtype, prec_w=dtype, block_m=cfg.unit)

@@ -499,12 +499,12 @@ inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, 
     // Measured crossovers (fp8, 256 experts; int8, 128 experts; bf16, 8 experts): the decode kernel with one
     // token block per tile wins up to about 24 rows per expert.  From about 28 on an expert often has more
     // than 32 rows and would stream its weights twice: with 16-bit and int8 operands the decode kernel with two
-    // token blocks (64-row tiles) is the fastest up to about 52 rows per expert (12 to 25 % ahead of the
+    // token blocks (64-row tiles) is the fastest up to about 56 rows per expert (5 to 25 % ahead of the
     // large-tile kernel, whose single workgroup per compute unit cannot hide a tile's prologue and epilogue
     // behind another tile's weight stream); with fp8 operands, and from there on for all types, the large-tile
     // kernel - it streams every weight tile once whatever the row count and fetches only the token slabs a
     // tile has - provided its tiles fill the chip.
-    if(two_block_decode_ok(t) && fits && avg >= 28 && avg <= 52)
+    if(two_block_decode_ok(t) && fits && avg >= 28 && avg <= 56)
         return 2;
     const int64_t big_tiles = (int64_t)experts * std::max<int64_t>(1, ceil_div<int64_t>(avg, big_tile_rows())) * ceil_div(inter, 128);
     const bool big_ok = big_tile_ok(t, tokens, topk, experts, hidden, inter);
