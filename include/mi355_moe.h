@@ -30,7 +30,9 @@
 extern "C" {
 #endif
 
-#define MI355_MOE_VERSION 200
+/* 210: mi355_fused_moe_traits gained weight_permute and mi355_moe_flatmm_args gained b_shuffle (both appended; a
+ * caller built against 200 must be rebuilt), mi355_fused_moe_chosen_tile_rows added */
+#define MI355_MOE_VERSION 210
 
 enum mi355_moe_status
 {

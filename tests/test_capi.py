@@ -148,7 +148,7 @@ def test_flatmm_operand_types_on_the_host():
 
 def test_host_only_entry_points():
     lib = _lib.load()
-    assert lib.mi355_moe_version() == 200
+    assert lib.mi355_moe_version() == 210
     assert lib.mi355_moe_max_num_tokens_padded(128, 8, 2, 32) == 2 * 128 + 8 * 32 - 2
     assert lib.mi355_moe_sorting_workspace_size(64, 128, 8) == 0          # one workgroup, no workspace
     assert lib.mi355_moe_sorting_workspace_size(32768, 64, 6) >= 384 * 64 * 4
