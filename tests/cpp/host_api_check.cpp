@@ -43,6 +43,22 @@ static T* to_device(const std::vector<T>& v)
     return p;
 }
 
+// the host-side weight pre-shuffle of CK's fused-MoE example for 2-byte elements: the row-major [e, n, k] weight viewed
+// as [e, n/16, 16, k/32, 4, 8] and permuted to [e, n/16, k/32, 4, 16, 8] (b_nr_kr_kw_nw_kv)
+static std::vector<uint16_t> preshuffle(const std::vector<uint16_t>& w, int e, int n, int k)
+{
+    std::vector<uint16_t> out(w.size());
+    size_t o = 0;
+    for(int x = 0; x < e; x++)
+        for(int nr = 0; nr < n / 16; nr++)
+            for(int kr = 0; kr < k / 32; kr++)
+                for(int kw = 0; kw < 4; kw++)
+                    for(int nw = 0; nw < 16; nw++)
+                        for(int kv = 0; kv < 8; kv++)
+                            out[o++] = w[((size_t)x * n + nr * 16 + nw) * k + kr * 32 + kw * 8 + kv];
+    return out;
+}
+
 int main()
 {
     const int T = 70, H = 256, I = 192, E = 6, K = 2, U = 32;
@@ -107,6 +123,19 @@ int main()
         den += r * r;
     }
     const double err = std::sqrt(num / den);
+    // the same call with g and d pre-shuffled on the host the way CK's example does it before calling its kernel
+    mi355::fused_moe_traits shuffled = traits;
+    shuffled.weight_permute = 1;
+    mi355::fused_moe_args args2 = args;
+    args2.g_ptr = to_device(preshuffle(g, E, 2 * I, H));
+    args2.d_ptr = to_device(preshuffle(d, E, H, I));
+    std::vector<uint16_t> z_o2(T * H, 0);
+    args2.o_ptr = to_device(z_o2);
+    if(mi355::fused_moe(shuffled, args2, mi355::stream_config{}) != 0.f) { std::fprintf(stderr, "pre-shuffled call failed\n"); return 5; }
+    HIP_OK(hipDeviceSynchronize());
+    std::vector<uint16_t> o2(T * H);
+    HIP_OK(hipMemcpy(o2.data(), args2.o_ptr, o2.size() * 2, hipMemcpyDeviceToHost));
+    if(std::memcmp(o.data(), o2.data(), o.size() * 2) != 0) { std::fprintf(stderr, "pre-shuffled weights give other bits\n"); return 6; }
     // unsupported traits report -1 like CK's dispatcher; timing returns milliseconds
     mi355::fused_moe_traits bad = traits; bad.prec_i = "fp16"; bad.prec_w = "fp16";
     const float unsupported = mi355::fused_moe(bad, args);
