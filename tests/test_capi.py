@@ -77,7 +77,8 @@ def test_sizes_out_of_range_are_rejected_on_the_host():
     lib = _lib.load()
     t = _lib.FusedMoeTraits(0, 0, 0, 3, 3, 3, 3, 32, 1, 0, 0, 0)
     for shape in ((128, 0, 2, 1024, 1024), (128, 8, 0, 1024, 1024), (-1, 8, 2, 1024, 1024), (128, 8, 2, 0, 1024),
-                  (128, 8, 2, 1024, -4), (128, 2000, 2, 1024, 1024), (128, 8, 300, 1024, 1024)):
+                  (128, 8, 2, 1024, -4), (128, 2000, 2, 1024, 1024), (128, 8, 300, 1024, 1024),
+                  (1 << 24, 8, 2, 1024, 1024), (0xffffff, 8, 255, 1024, 1024)):  # 24-bit tokens, 32-bit row indices
         assert lib.mi355_fused_moe_workspace_size(C.byref(t), *shape) == 0, shape
         assert lib.mi355_fused_moe_tile_rows(C.byref(t), *shape) == 0, shape
         T, E, K, H, I = shape
@@ -132,6 +133,13 @@ def test_flatmm_operand_types_on_the_host():
         assert ws(kind, "bf16", "fp16") == 0 and ws(kind, "fp16", "bf16") == 0 and ws(kind, "fp16", "int8") == 0
         assert b"operand types" in lib.mi355_moe_last_error()
     assert ws(1, "int8", "int8") > 0 and ws(2, "bf16", "int8") > 0 and ws(2, "int8", "int8") == 0
+    # the same size limits as the fused entry points
+    for field, value in (("NumTokens", 1 << 24), ("NumExperts", 0), ("TopK", 256), ("N", 0), ("K", -8)):
+        a = _lib.FlatmmArgs()
+        a.NumTokens, a.NumExperts, a.TopK, a.N, a.K, a.block_m, a.k_batch = 64, 4, 2, 256, 128, 32, 1
+        a.prec_a = a.prec_b = D["bf16"]
+        setattr(a, field, value)
+        assert lib.mi355_moe_flatmm_workspace_size(1, C.byref(a)) == 0 and b"bad sizes" in lib.mi355_moe_last_error(), field
 
     # B as ck_tile::shuffle_b lays it out for 16-row warp tiles: rows of whole 64-byte blocks, no padded K
     def ws_shuffled(prec, K, b_shuffle=1, k_pad=0):

@@ -450,8 +450,6 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
     *reinterpret_cast<uint4*>(out + (int64_t)t * out_row_bytes + (int64_t)h0 * 2) = o;
 }
 
-// 32-row blocks per M tile, from the expected rows per expert; big_tile_rows()/32 selects the
-// large-tile kernel
 // bytes per element of the intermediate activations the down GEMM reads: e4m3 on the fp8 path, int8 when the
 // int8 path re-quantises them (fused_quant 1 / 2), bf16 otherwise
 inline int y_bytes(const mi355_fused_moe_traits& t)
@@ -469,8 +467,6 @@ inline bool decode_tile(const mi355_fused_moe_traits& t, int mblk)
     return mblk == 1 || (mblk == 2 && two_block_decode_ok(t));
 }
 
-// 32-row blocks per M tile, from the expected rows per expert; big_tile_rows()/32 selects the
-// large-tile kernel
 // every operand of the problem can be addressed as a base plus a 32-bit byte offset (the large-tile and decode kernels)
 inline bool offsets_fit(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
 {
@@ -492,6 +488,7 @@ inline bool big_tile_ok(const mi355_fused_moe_traits& t, int64_t tokens, int top
            big_tile_supported(t.prec_i, hidden * eb, inter * y_b, y_b == 1);
 }
 
+// 32-row blocks per M tile, from the expected rows per expert; big_tile_rows() / 32 selects the large-tile kernel
 inline int pick_mblk(const mi355_fused_moe_traits& t, int64_t tokens, int topk, int experts, int hidden, int inter)
 {
     const int64_t avg = tokens * topk / std::max(experts, 1);
@@ -681,8 +678,9 @@ GemmPlan make_gemm_plan(const mi355_fused_moe_traits& t, void* ws_ptr, int32_t t
 
 bool sizes_in_range(int32_t tokens, int32_t experts, int32_t topk, int32_t hidden, int32_t inter)
 {
+    // (sorted ids hold the token in 24 bits; row indices of the padded routing list are 32-bit integers)
     return tokens >= 0 && tokens <= 0xffffff && experts > 0 && experts <= 1024 && topk > 0 && topk <= 255 && hidden > 0 &&
-           inter > 0;
+           inter > 0 && (int64_t)tokens * topk + (int64_t)experts * 1024 < INT32_MAX;
 }
 
 // Everything that can be checked on the host before anything is launched: the fused entry point calls it ahead
@@ -911,7 +909,7 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: operand types a=%d b=%d (bf16 x bf16, fp16 x fp16, fp8 x fp8, "
                                              "int8 x int8 for the gate+up GEMM, bf16 x int8 for the down GEMM)", a.prec_a,
                     a.prec_b);
-    if(a.NumTokens < 0 || a.NumExperts <= 0 || a.NumExperts > 1024 || a.TopK <= 0 || a.TopK > 255 || a.N <= 0 || a.K <= 0 ||
+    if(!sizes_in_range(a.NumTokens, a.NumExperts, a.TopK, a.N, a.K) ||
        a.block_m < 1 || a.block_m > 1024 || a.k_batch > 1 || (g1 && !go && a.N % 2 != 0))
         return fail(MI355_MOE_E_INVALID, "moe_flatmm: bad sizes (tokens=%d experts=%d topk=%d N=%d K=%d block_m=%d k_batch=%d)",
                     a.NumTokens, a.NumExperts, a.TopK, a.N, a.K, a.block_m, a.k_batch);
@@ -1014,6 +1012,8 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     int* inv           = reinterpret_cast<int*>(wsb + L.inv_off);
     const int mblk     = L.mblk;
     const int prec     = L.traits.prec_i;
+    if((g1 ? T : (int64_t)T * K) * a.stride_A * a_b >= ((int64_t)1 << 32) && mblk > 4)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: A of 4 GiB or more is not supported at this problem size");
     {
         KernelTimer timer(MI355_MOE_K_PREP, stream);
         const int n_inv     = T * K;
@@ -1049,8 +1049,6 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     p.k_bytes_x      = (a.K - a.k_padded_zeros) * a_b;
     p.k_bytes_w      = (a.K - a.k_padded_zeros) * b_b;
     const int64_t a_rows = g1 ? T : (int64_t)T * K;
-    if(a_rows * p.x_row_bytes >= ((int64_t)1 << 32) && mblk > 4)
-        return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: A of 4 GiB or more is not supported at this problem size");
     const bool decode = decode_tile(L.traits, mblk) && decode_supported(a_rows * p.x_row_bytes, a_rows * p.x_row_bytes, p.w_expert_bytes);
     if(g1)
     {
