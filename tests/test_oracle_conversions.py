@@ -233,3 +233,33 @@ def test_preshuffled_layout_is_ck_tile_shuffle_b(dtype, n_warp, k_warp, view):
         pytest.skip("oracle/_ref/libck_ref.so not built (ck_tile headers absent)")
     assert np.array_equal(oracle.permute_weights(w, *view), want)
     assert not np.array_equal(want, w)
+
+
+def test_fp64_reciprocal_product_rounds_like_the_fp32_division():
+    """The quantisation kernels divide a row by its scale as fp32(fp64(x) * (1 / fp64(s))): a quotient of two fp32
+    numbers is at least 2^-49 (relative) away from every fp32 rounding boundary, the fp64 product at most 2^-51.9
+    from the quotient.  Checked on random pairs and on the cases a shortcut in fp32 gets wrong: divisors whose
+    significand is next to a power of two, quotients next to midpoints."""
+    rng = np.random.default_rng(7)
+    n = 2_000_000
+
+    def mismatches(x, s):
+        ref = x / s
+        alt = (x.astype(np.float64) * (1.0 / s.astype(np.float64))).astype(np.float32)
+        normal = np.abs(ref) >= np.float32(2.0 ** -126)
+        return int(((ref.view(np.uint32) != alt.view(np.uint32)) & normal).sum())
+
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    s = (np.abs(rng.standard_normal(n)) + 1e-3).astype(np.float32)
+    pow2 = (np.float32(2.0) ** rng.integers(-20, 20, n).astype(np.float32)).view(np.uint32).astype(np.int64)
+    below = (pow2 - rng.integers(1, 40, n)).astype(np.uint32).view(np.float32)
+    above = (pow2 + rng.integers(0, 40, n)).astype(np.uint32).view(np.float32)
+    midpoints = rng.integers(2 ** 23, 2 ** 24, n).astype(np.float64) + 0.5
+    assert mismatches(x, s) == 0 and mismatches(x, below) == 0 and mismatches(x, above) == 0
+    for div in (s, below, above):
+        assert mismatches((midpoints * div.astype(np.float64)).astype(np.float32), div) == 0
+    # a row of the smooth-quant shape: |x| <= amax, s = amax / 448 and amax / 127
+    amax = np.abs(x).max()
+    for qmax in (448.0, 127.0):
+        sc = np.full(n, np.float32(amax) / np.float32(qmax), np.float32)
+        assert mismatches(x, sc) == 0

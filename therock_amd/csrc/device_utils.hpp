@@ -66,7 +66,6 @@ __device__ inline uint32_t float_to_bf16_bits(float f)
     return u >> 16;
 }
 
-// two floats -> packed bf16 pair, round-to-nearest-even: a single v_cvt_pk_bf16_f32 on gfx950
 // two floats -> packed fp16 (round to nearest even, overflow to infinity: the IEEE conversion)
 __device__ inline uint32_t pack_f16x2(float lo, float hi)
 {
@@ -79,6 +78,7 @@ __device__ inline float f16_bits_to_float(uint32_t h)
     return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(h)));
 }
 
+// two floats -> packed bf16 pair, round-to-nearest-even: a single v_cvt_pk_bf16_f32 on gfx950
 __device__ inline uint32_t pack_bf16x2(float lo, float hi)
 {
     typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
@@ -88,6 +88,21 @@ __device__ inline uint32_t pack_bf16x2(float lo, float hi)
     uint32_t r;
     __builtin_memcpy(&r, &b, sizeof(r));
     return r;
+}
+
+// x / s for many dividends x and one divisor s (a row's quantisation scale), with the result of the fp32 division
+// and a third of its instructions: one fp64 reciprocal per row, then per element an fp64 product rounded to fp32.
+// Why the rounding agrees: the product is within 2^-51.9 (relative) of the real quotient z (two fp64 roundings).
+// The fp32 result can only differ if a midpoint m of two neighbouring fp32 numbers lies that close to z.  Write
+// x = X 2^a, s = S 2^c with 24-bit integers X, S and m = M 2^b with an odd 25-bit M: z - m = (X 2^a - M S 2^(b+c)) / s
+// is not zero (M S = X 2^k would need the odd M > 2^24 to divide X < 2^24), so it is at least one unit of that
+// integer difference, |z - m| >= m / (M S) > m 2^-49.  Below 2^-126 midpoints have fewer bits and a quotient can hit
+// one exactly; there the two results may be neighbouring subnormals of the same sign, which every quantiser here
+// turns into the same zero.  Infinities, NaNs and zeros behave as in the division (1 / inf = 0, inf * 0 = NaN).
+__device__ inline double row_reciprocal(float s) { return 1.0 / static_cast<double>(s); }
+__device__ inline float div_by_row_scale(float x, double s_reciprocal)
+{
+    return static_cast<float>(static_cast<double>(x) * s_reciprocal);
 }
 
 } // namespace mi355

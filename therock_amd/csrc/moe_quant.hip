@@ -96,11 +96,12 @@ __device__ inline float quantise_row(const uint16_t* __restrict__ xr, const floa
         const float s     = amax > 0.f ? s_out : 1.0f;
         if(threadIdx.x == 0)
             *scale_out = s_out;
+        const double s_rcp = row_reciprocal(s);
         auto store = [&](int c, const float (&o)[8]) {
             uint32_t w[2] = {0u, 0u};
 #pragma unroll
             for(int i = 0; i < 8; i++)
-                w[i >> 2] |= static_cast<uint32_t>(quantise_one<FP8>(o[i] / s)) << (8 * (i & 3));
+                w[i >> 2] |= static_cast<uint32_t>(quantise_one<FP8>(div_by_row_scale(o[i], s_rcp))) << (8 * (i & 3));
             *reinterpret_cast<uint2*>(qr + c * 8) = make_uint2(w[0], w[1]);
         };
 #pragma unroll
@@ -130,8 +131,9 @@ __device__ inline float quantise_row(const uint16_t* __restrict__ xr, const floa
         const float s     = amax > 0.f ? s_out : 1.0f;
         if(threadIdx.x == 0)
             *scale_out = s_out;
+        const double s_rcp = row_reciprocal(s);
         for(int c = threadIdx.x; c < cols; c += 256)
-            qr[c] = quantise_one<FP8>((bf16_bits_to_float(xr[c]) * (SMOOTH ? sr[c] : 1.0f)) / s);
+            qr[c] = quantise_one<FP8>(div_by_row_scale(bf16_bits_to_float(xr[c]) * (SMOOTH ? sr[c] : 1.0f), s_rcp));
         return amax;
     }
 }
@@ -238,11 +240,12 @@ __global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t
         if(threadIdx.x == 0)
             yscale[r] = ys_out;
         unsigned char* qr = qy + r * y_stride;
+        const double ys_rcp = row_reciprocal(ys);
         auto store = [&](int c, const float (&o)[8]) {
             uint32_t w[2] = {0u, 0u};
 #pragma unroll
             for(int i = 0; i < 8; i++)
-                w[i >> 2] |= static_cast<uint32_t>(quantise_one<FP8>(o[i] / ys)) << (8 * (i & 3));
+                w[i >> 2] |= static_cast<uint32_t>(quantise_one<FP8>(div_by_row_scale(o[i], ys_rcp))) << (8 * (i & 3));
             *reinterpret_cast<uint2*>(qr + c * 8) = make_uint2(w[0], w[1]);
         };
 #pragma unroll
@@ -341,11 +344,12 @@ __global__ __launch_bounds__(256) void moe_requant_y_kernel(const uint16_t* __re
     const float ys     = amax > 0.f ? ys_out : 1.0f; // a row of zeros: scale 0, codes 0
     if(lane == 0)
         yscale[row] = ys_out;
+    const double ys_rcp = row_reciprocal(ys);
     auto store = [&](int c, const float (&o)[8]) {
         uint32_t w[2] = {0u, 0u};
 #pragma unroll
         for(int i = 0; i < 8; i++)
-            w[i >> 2] |= (static_cast<uint32_t>(static_cast<int>(__builtin_rintf(o[i] / ys))) & 0xffu) << (8 * (i & 3));
+            w[i >> 2] |= (static_cast<uint32_t>(static_cast<int>(__builtin_rintf(div_by_row_scale(o[i], ys_rcp)))) & 0xffu) << (8 * (i & 3));
         *reinterpret_cast<uint2*>(dst(c)) = make_uint2(w[0], w[1]);
     };
 #pragma unroll
