@@ -26,6 +26,33 @@ __device__ inline unsigned char quantise_one(float v)
     }
 }
 
+// eight quotients o[i] * (1 / s) -> eight codes in two dwords.  e4m3: the conversion instruction packs two codes
+// into a chosen half of a dword, so four of them fill both dwords with no masking or shifting.
+template <bool FP8>
+__device__ inline uint2 quantise_8(const float (&o)[8], double s_rcp)
+{
+    if constexpr(FP8)
+    {
+        float c[8];
+#pragma unroll
+        for(int i = 0; i < 8; i++)
+            c[i] = fminf(fmaxf(div_by_row_scale(o[i], s_rcp), -448.f), 448.f);
+        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
+        w0     = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w0, true);
+        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(c[4], c[5], 0, false);
+        w1     = __builtin_amdgcn_cvt_pk_fp8_f32(c[6], c[7], w1, true);
+        return make_uint2(static_cast<uint32_t>(w0), static_cast<uint32_t>(w1));
+    }
+    else
+    {
+        uint32_t w[2] = {0u, 0u};
+#pragma unroll
+        for(int i = 0; i < 8; i++)
+            w[i >> 2] |= static_cast<uint32_t>(quantise_one<false>(div_by_row_scale(o[i], s_rcp))) << (8 * (i & 3));
+        return make_uint2(w[0], w[1]);
+    }
+}
+
 __device__ inline float block_max_256(float v, float* s_red)
 {
 #pragma unroll
@@ -97,13 +124,7 @@ __device__ inline float quantise_row(const uint16_t* __restrict__ xr, const floa
         if(threadIdx.x == 0)
             *scale_out = s_out;
         const double s_rcp = row_reciprocal(s);
-        auto store = [&](int c, const float (&o)[8]) {
-            uint32_t w[2] = {0u, 0u};
-#pragma unroll
-            for(int i = 0; i < 8; i++)
-                w[i >> 2] |= static_cast<uint32_t>(quantise_one<FP8>(div_by_row_scale(o[i], s_rcp))) << (8 * (i & 3));
-            *reinterpret_cast<uint2*>(qr + c * 8) = make_uint2(w[0], w[1]);
-        };
+        auto store = [&](int c, const float (&o)[8]) { *reinterpret_cast<uint2*>(qr + c * 8) = quantise_8<FP8>(o, s_rcp); };
 #pragma unroll
         for(int j = 0; j < kQuantCache; j++)
         {
@@ -200,16 +221,32 @@ __global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t
         o[0] = in[0] * s0.x; o[1] = in[1] * s0.y; o[2] = in[2] * s0.z; o[3] = in[3] * s0.w;
         o[4] = in[4] * s1.x; o[5] = in[5] * s1.y; o[6] = in[6] * s1.z; o[7] = in[7] * s1.w;
     };
+    auto scales_of_slot = [&](int k) {
+        const int e = topk_ids[(int64_t)t * topk + k];
+        return smscale + (int64_t)min(max(e, 0), experts - 1) * hidden;
+    };
+    // the smooth scales of the cached pieces, for the slot about to be processed: fetched one slot ahead, so that
+    // their latency passes under the previous slot's reduction, conversions and stores
+    float4 sm[kQuantCache][2];
+    auto fetch_scales = [&](const float* sr) {
+#pragma unroll
+        for(int j = 0; j < kQuantCache; j++)
+            if(threadIdx.x + 256 * j < chunks)
+            {
+                sm[j][0] = *reinterpret_cast<const float4*>(sr + (threadIdx.x + 256 * j) * 8);
+                sm[j][1] = *reinterpret_cast<const float4*>(sr + (threadIdx.x + 256 * j) * 8 + 4);
+            }
+    };
     float xv[kQuantCache][8];
 #pragma unroll
     for(int j = 0; j < kQuantCache; j++)
         if(threadIdx.x + 256 * j < chunks)
             load_x(threadIdx.x + 256 * j, xv[j]);
+    if(topk > 0)
+        fetch_scales(scales_of_slot(0));
     for(int k = 0; k < topk; k++)
     {
-        int e = topk_ids[(int64_t)t * topk + k];
-        e     = min(max(e, 0), experts - 1);
-        const float* sr = smscale + (int64_t)e * hidden;
+        const float* sr = scales_of_slot(k);
         float v[kQuantCache][8];
         float amax = 0.f;
 #pragma unroll
@@ -218,12 +255,16 @@ __global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t
             const int c = threadIdx.x + 256 * j;
             if(c < chunks)
             {
-                times_sm(sr, c, xv[j], v[j]);
+                const float4 s0 = sm[j][0], s1 = sm[j][1];
+                v[j][0] = xv[j][0] * s0.x; v[j][1] = xv[j][1] * s0.y; v[j][2] = xv[j][2] * s0.z; v[j][3] = xv[j][3] * s0.w;
+                v[j][4] = xv[j][4] * s1.x; v[j][5] = xv[j][5] * s1.y; v[j][6] = xv[j][6] * s1.z; v[j][7] = xv[j][7] * s1.w;
 #pragma unroll
                 for(int i = 0; i < 8; i++)
                     amax = fmaxf(amax, fabsf(v[j][i]));
             }
         }
+        if(k + 1 < topk)
+            fetch_scales(scales_of_slot(k + 1));
         for(int c = threadIdx.x + 256 * kQuantCache; c < chunks; c += 256)
         {
             float a[8], b[8];
@@ -241,13 +282,7 @@ __global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t
             yscale[r] = ys_out;
         unsigned char* qr = qy + r * y_stride;
         const double ys_rcp = row_reciprocal(ys);
-        auto store = [&](int c, const float (&o)[8]) {
-            uint32_t w[2] = {0u, 0u};
-#pragma unroll
-            for(int i = 0; i < 8; i++)
-                w[i >> 2] |= static_cast<uint32_t>(quantise_one<FP8>(div_by_row_scale(o[i], ys_rcp))) << (8 * (i & 3));
-            *reinterpret_cast<uint2*>(qr + c * 8) = make_uint2(w[0], w[1]);
-        };
+        auto store = [&](int c, const float (&o)[8]) { *reinterpret_cast<uint2*>(qr + c * 8) = quantise_8<FP8>(o, ys_rcp); };
 #pragma unroll
         for(int j = 0; j < kQuantCache; j++)
             if(threadIdx.x + 256 * j < chunks)
