@@ -305,6 +305,8 @@ def main():
     ap.add_argument("--headline-only", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="the named workload, the kernels either side of the path and the router only (profiling runs)")
     # variations of the named workload, for profiling runs of what `extra_workloads` reports
     ap.add_argument("--tokens", type=int, default=0, help="token count instead of the workload's own")
     ap.add_argument("--fused-quant", type=int, default=0, choices=(0, 2),
@@ -359,7 +361,7 @@ def main():
         router = {"error": repr(e)}
 
     others = {}
-    if not a.headline_only:
+    if not a.headline_only and not a.no_other_workloads:
         for name, c in mi.CONFIGS.items():
             if name == cfg.name:
                 continue
@@ -382,7 +384,7 @@ def main():
     # (fused_quant 2), batches between decode and prefill (40 rows per expert), and decode-sized batches whose routing
     # is skewed (Zipf; one expert in every token's top-k).
     extra = {}
-    if not a.headline_only:
+    if not a.headline_only and not a.no_other_workloads:
         i8 = mi.CONFIGS["cfg4_decode_int8_t256"]
         cases = {
             "cfg4_model_int8_t8192_fused_quant0": (i8.scaled(name="cfg4_model_int8_t8192", tokens=8192), {}),

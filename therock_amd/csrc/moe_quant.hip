@@ -282,7 +282,12 @@ __global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t
             yscale[r] = ys_out;
         unsigned char* qr = qy + r * y_stride;
         const double ys_rcp = row_reciprocal(ys);
-        auto store = [&](int c, const float (&o)[8]) { *reinterpret_cast<uint2*>(qr + c * 8) = quantise_8<FP8>(o, ys_rcp); };
+        // (streaming stores: the quantised rows are written once and should not push the experts' scales out of L2)
+        auto store = [&](int c, const float (&o)[8]) {
+            typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+            const uint2 q = quantise_8<FP8>(o, ys_rcp);
+            __builtin_nontemporal_store(u32x2_t{q.x, q.y}, reinterpret_cast<u32x2_t*>(qr + c * 8));
+        };
 #pragma unroll
         for(int j = 0; j < kQuantCache; j++)
             if(threadIdx.x + 256 * j < chunks)
