@@ -199,7 +199,8 @@ def run_neighbours(cfg, inp, buf, steps):
     out = {}
 
     def timed(fn, n):
-        fn()
+        for _ in range(3):  # (the first calls on freshly allocated outputs run up to 15 % slower)
+            fn()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -214,7 +215,7 @@ def run_neighbours(cfg, inp, buf, steps):
     ms = timed(lambda: ta.rowwise_quant(x, qd), steps)
     out["rowwise_quant"] = {"ms": ms, "GBps": T * H * 3 / ms / 1e6, "what": f"[{T}, {H}] bf16 -> {qd} + scale"}
     sm = torch.rand((E, H), device="cuda", generator=g) + 0.5
-    ms = timed(lambda: ta.moe_smoothquant(x, sm, inp["topk_ids"], qd), max(2, steps // 4))
+    ms = timed(lambda: ta.moe_smoothquant(x, sm, inp["topk_ids"], qd), max(3, steps // 2))
     out["moe_smoothquant"] = {"ms": ms, "GBps": (T * H * 2 + K * T * H) / ms / 1e6,
                               "what": f"[{T}, {H}] bf16 -> [{K}, {T}, {H}] {qd} + scales"}
     del sm
@@ -231,7 +232,7 @@ def run_neighbours(cfg, inp, buf, steps):
                           dtype=torch.uint8, device="cuda")
         ms = timed(lambda: ta.moe_flatmm(ta.GEMM1_GATE_UP, inp["a"], inp["g"], y, buf.sorted_ids, buf.sorted_eid, buf.total,
                                          T, K, cfg.unit, scale_m=inp["a_scale"], scale_n=inp["g_scale"], workspace=ws0),
-                   max(2, steps // 4))
+                   max(3, steps // 2))
         out["flatmm_gate_up"] = {"ms": ms, "tflops": 4.0 * T * K * H * I / ms / 1e9, "what": "stand-alone gate+up GEMM, bf16 C"}
         if cfg.dtype == "fp8":
             yq, ys = ta.rowwise_quant(y, "fp8")
@@ -243,7 +244,7 @@ def run_neighbours(cfg, inp, buf, steps):
                                                             buf.total, T, K, cfg.unit),), dtype=torch.uint8, device="cuda")
         ms = timed(lambda: ta.moe_flatmm(ta.GEMM2, yq, inp["d"], c, buf.sorted_ids, buf.sorted_eid, buf.total, T, K, cfg.unit,
                                          sorted_weights=buf.sorted_w, scale_m=ys, scale_n=inp["d_scale"], workspace=ws1),
-                   max(2, steps // 4))
+                   max(3, steps // 2))
         out["flatmm_down"] = {"ms": ms, "tflops": 2.0 * T * K * H * I / ms / 1e9,
                               "what": "stand-alone down GEMM + combine, added to bf16 C"}
     return out
