@@ -43,6 +43,25 @@ __device__ inline float wave_sum(float v)
     return v;
 }
 
+// Wave-wide maximum / minimum of a 32-bit unsigned value, the same in every lane afterwards.  Data-parallel
+// primitives instead of LDS-routed shuffles: an inclusive scan over each row of 16 lanes (row_shr 1, 2, 4, 8; lanes
+// shifted in from outside a row read the identity), then lane 15 of rows 0 and 2 is combined into rows 1 and 3
+// (row_bcast:15) and lane 31 into rows 2 and 3 (row_bcast:31): lane 63 holds the result.
+template <bool MAX>
+__device__ inline uint32_t wave_reduce_u32(uint32_t v)
+{
+    constexpr int ident = MAX ? 0 : -1;
+    auto combine = [](uint32_t a, uint32_t b) { return MAX ? max(a, b) : min(a, b); };
+    int x = static_cast<int>(v);
+    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x111, 0xf, 0xf, false))); // row_shr:1
+    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x112, 0xf, 0xf, false))); // row_shr:2
+    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x114, 0xf, 0xf, false))); // row_shr:4
+    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x118, 0xf, 0xf, false))); // row_shr:8
+    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x142, 0xa, 0xf, false))); // row_bcast:15
+    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x143, 0xc, 0xf, false))); // row_bcast:31
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(x, 63));
+}
+
 template <typename In, int PER_LANE>
 __global__ __launch_bounds__(kRouterBlock) void topk_softmax_kernel(const RouterParams p)
 {
@@ -91,41 +110,40 @@ __global__ __launch_bounds__(kRouterBlock) void topk_softmax_kernel(const Router
         for(int j = 0; j < PER_LANE; j++)
             v[j] = lane + j * kWave < p.experts ? v[j] / s : -INFINITY;
     }
-    // k rounds of arg-max; the winner is struck out of its lane's registers and kept by lane i
+    // k rounds of arg-max.  The probabilities are non-negative, so their bit patterns order like unsigned integers:
+    // key = bits + 1 for a live entry, 0 for one that is struck out or beyond the expert count.  A round is two
+    // wave reductions: the largest key, then the lowest expert id among the entries that hold it.  The winner is
+    // struck out of its lane's registers and kept by lane i.
+    uint32_t key[PER_LANE];
+#pragma unroll
+    for(int j = 0; j < PER_LANE; j++)
+        key[j] = v[j] >= 0.f ? __float_as_uint(v[j]) + 1u : 0u;
     float my_w = 0.f;
     int my_e   = 0;
     float sum  = 0.f;
     for(int i = 0; i < p.topk; i++)
     {
-        float best = -INFINITY;
-        int be     = 0x7fffffff;
+        uint32_t bk = 0u;
+        int be      = 0x7fffffff;
 #pragma unroll
         for(int j = 0; j < PER_LANE; j++)
-            if(v[j] > best)
+            if(key[j] > bk)
             {
-                best = v[j];
-                be   = lane + j * kWave;
+                bk = key[j];
+                be = lane + j * kWave;
             }
-#pragma unroll
-        for(int d = 32; d > 0; d >>= 1)
-        {
-            const float ob = __shfl_xor(best, d);
-            const int oe   = __shfl_xor(be, d);
-            if(ob > best || (ob == best && oe < be))
-            {
-                best = ob;
-                be   = oe;
-            }
-        }
+        const uint32_t top = wave_reduce_u32<true>(bk);
+        const int win      = static_cast<int>(wave_reduce_u32<false>(bk == top ? static_cast<uint32_t>(be) : 0x7fffffffu));
+        const float best   = top != 0u ? __uint_as_float(top - 1u) : -INFINITY;
 #pragma unroll
         for(int j = 0; j < PER_LANE; j++)
-            if(lane + j * kWave == be)
-                v[j] = -INFINITY;
+            if(lane + j * kWave == win)
+                key[j] = 0u;
         sum += best;
         if(lane == i)
         {
             my_w = best;
-            my_e = be;
+            my_e = win;
         }
     }
     if(lane < p.topk)
