@@ -137,10 +137,26 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
     const int s0    = part * spp;
     const int s1    = min(s0 + spp, nseg);
 
+    // (both walks over the thread's segments fetch eight counters at a time: one workgroup runs this pass, and a chain
+    // of dependent global loads, one per segment, would be most of its time)
+    constexpr int kBatch = 8;
     int sum = 0;
     if(e < E)
-        for(int sg = s0; sg < s1; sg++)
-            sum += counts[sg * E + e];
+    {
+        int sg0 = s0;
+        for(; sg0 + kBatch <= s1; sg0 += kBatch)
+        {
+            int c[kBatch];
+#pragma unroll
+            for(int u = 0; u < kBatch; u++)
+                c[u] = counts[(sg0 + u) * E + e];
+#pragma unroll
+            for(int u = 0; u < kBatch; u++)
+                sum += c[u];
+        }
+        for(; sg0 < s1; sg0++)
+            sum += counts[sg0 * E + e];
+    }
     s.part[part * Ep + e] = sum;
     __syncthreads();
     if(tid < Ep)
@@ -178,10 +194,25 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
     if(e < E)
     {
         int base = s.tiles[e] > 0 ? s.tbase[e] * U + s.part[part * Ep + e] : -1;
-        for(int sg = s0; sg < s1; sg++)
+        int sg0 = s0;
+        for(; sg0 + kBatch <= s1; sg0 += kBatch)
         {
-            const int c          = counts[sg * E + e];
-            counts[sg * E + e]   = base;
+            int c[kBatch];
+#pragma unroll
+            for(int u = 0; u < kBatch; u++)
+                c[u] = counts[(sg0 + u) * E + e];
+#pragma unroll
+            for(int u = 0; u < kBatch; u++)
+            {
+                counts[(sg0 + u) * E + e] = base;
+                if(base >= 0)
+                    base += c[u];
+            }
+        }
+        for(; sg0 < s1; sg0++)
+        {
+            const int c        = counts[sg0 * E + e];
+            counts[sg0 * E + e] = base;
             if(base >= 0)
                 base += c;
         }
@@ -299,28 +330,36 @@ __global__ __launch_bounds__(kScanBlock) void moe_sorting_oneshot_kernel(SortPar
         cnt[e] = 0;
     wave_sync();
     int* inv = p.plan.tile_map != nullptr ? p.plan.inv : nullptr;
-    if(seglen == kWave)
+    // The wave's entries are read once, all loads issued together, and stay in registers for both walks: fetched
+    // step by step they would be a chain of dependent global loads in the one workgroup that does all the work.
+    constexpr int kMaxSteps = kOneShotMaxEntries / kScanBlock;
+    int ev[kMaxSteps];
+    float wv[kMaxSteps];
+#pragma unroll
+    for(int u = 0; u < kMaxSteps; u++)
     {
-        // a single step per wave (at most 1024 entries: the decode regime): the entry is read once
-        // and stays in registers for both walks
-        const int i   = begin + lane;
-        const int e   = i < end ? p.ids[i] : -1;
-        const float w = i < end ? p.weights[i] : 0.f;
-        walk_step<false>(i, e, w, i < end, p.K, p.E, p.nbits, cnt, nullptr, nullptr, nullptr);
-        __syncthreads();
-        scan_phase(sh, dyn_lds, kScanWaves, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
-                   p.sorted_eid, p.total, p.plan);
-        __syncthreads();
-        if(begin < end)
-            walk_step<true>(i, e, w, i < end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w, inv);
-        return;
+        const int i = begin + u * kWave + lane;
+        ev[u]       = i < end ? p.ids[i] : -1;
+        wv[u]       = i < end ? p.weights[i] : 0.f;
     }
-    walk_segment<false>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, nullptr, nullptr);
+#pragma unroll
+    for(int u = 0; u < kMaxSteps; u++)
+        if(begin + u * kWave < end)
+        {
+            const int i = begin + u * kWave + lane;
+            walk_step<false>(i, ev[u], wv[u], i < end, p.K, p.E, p.nbits, cnt, nullptr, nullptr, nullptr);
+        }
     __syncthreads();
     scan_phase(sh, dyn_lds, kScanWaves, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
                p.sorted_eid, p.total, p.plan);
     __syncthreads();
-    walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w, inv);
+#pragma unroll
+    for(int u = 0; u < kMaxSteps; u++)
+        if(begin + u * kWave < end)
+        {
+            const int i = begin + u * kWave + lane;
+            walk_step<true>(i, ev[u], wv[u], i < end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w, inv);
+        }
 }
 
 // ---- pass 1: per-segment expert histogram; trailing blocks zero moe_buf
