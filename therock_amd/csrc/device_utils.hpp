@@ -12,6 +12,20 @@ __device__ inline void wave_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Inclusive prefix sum over the 64 lanes of a wave (every lane active), with data-parallel primitives instead of
+// LDS-routed shuffles: row_shr 1, 2, 4, 8 scan each row of 16 lanes (a lane shifted in from outside its row reads
+// 0), row_bcast:15 adds the total of rows 0 and 2 to rows 1 and 3, row_bcast:31 the total of rows 0-1 to rows 2-3.
+__device__ inline int wave_inclusive_scan(int x)
+{
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false); // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false); // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false); // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false); // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false); // row_bcast:15 into rows 1 and 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false); // row_bcast:31 into rows 2 and 3
+    return x;
+}
+
 // Exclusive scan of one int per thread over a block of NWAVES*64 threads.  s_wave needs
 // NWAVES+1 ints of LDS.  Every thread of the block must call it; `total` gets the block sum.
 template <int NWAVES>
@@ -20,28 +34,14 @@ __device__ inline int block_exclusive_scan(int v, int* s_wave, int& total)
     static_assert(NWAVES <= kWave, "one wave scans the wave totals");
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
-    int x          = v;
-#pragma unroll
-    for(int d = 1; d < kWave; d <<= 1)
-    {
-        const int y = __shfl_up(x, d);
-        if(lane >= d)
-            x += y;
-    }
+    const int x    = wave_inclusive_scan(v);
     if(lane == kWave - 1)
         s_wave[wave] = x;
     __syncthreads();
     if(wave == 0)
     {
-        const int w = lane < NWAVES ? s_wave[lane] : 0;
-        int xx      = w;
-#pragma unroll
-        for(int d = 1; d < NWAVES; d <<= 1)
-        {
-            const int y = __shfl_up(xx, d);
-            if(lane >= d)
-                xx += y;
-        }
+        const int w  = lane < NWAVES ? s_wave[lane] : 0;
+        const int xx = wave_inclusive_scan(w);
         if(lane < NWAVES)
             s_wave[lane] = xx - w;
         if(lane == NWAVES - 1)
