@@ -232,9 +232,10 @@ size_t mi355_fused_moe_workspace_size(const mi355_fused_moe_traits* traits, int3
 int32_t mi355_fused_moe_tile_rows(const mi355_fused_moe_traits* traits, int32_t tokens, int32_t num_experts,
                                   int32_t topk, int32_t hidden_size, int32_t intermediate_size);
 
-/* For harnesses and tests: the tile height the last mi355_fused_moe call on `ws` ran with.  Where the routing decides
- * (fp8 operands below about 28 rows per expert on average: a skewed batch whose active experts hold 48 padded rows
- * or more each runs on the 320-row tiles, chosen by the sort on the device) the value is read back from the work list
+/* For harnesses and tests: the tile height the last mi355_fused_moe or mi355_fused_moegemm call on `ws` ran with.  Where
+ * the routing decides (fp8 operands below about 28 rows per expert on average: a skewed batch whose active experts hold
+ * 48 padded rows or more each runs on the 320-row tiles, chosen on the device by the pass that builds the work list: the
+ * sort, or the GEMM entry point's own pass over sorted_expert_ids) the value is read back from the work list
  * in `ws`, after synchronising `stream`; everywhere else it is mi355_fused_moe_tile_rows().  No counterpart in ck_tile. */
 int32_t mi355_fused_moe_chosen_tile_rows(const mi355_fused_moe_traits* traits, int32_t tokens, int32_t num_experts,
                                          int32_t topk, int32_t hidden_size, int32_t intermediate_size,

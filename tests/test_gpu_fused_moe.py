@@ -171,7 +171,7 @@ def test_skewed_fp8_batch_takes_the_large_tiles_on_the_device():
             inp["g"] = np.ascontiguousarray(inp["g"][:, :cfg.inter])
             inp["g_scale"] = np.ascontiguousarray(inp["g_scale"][:, :cfg.inter])
         print(f"fused_moe {cfg} seed={seed} {kw}", flush=True)
-        got, buf = run_fused_moe(cfg, inp, **kw)
+        got, buf = run_fused_moe(cfg, inp, **kw)  # (unfused: mi355_moe_sorting + mi355_fused_moegemm, whose tile-list pass chooses)
         traits = ta.fused_moe_traits(prec_i="fp8", prec_w="fp8", block_m=cfg.unit, local_expert_masking=mask is not None,
                                      gate_only=kw.get("gate_only", 0))
         shape = (cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter)
@@ -196,6 +196,10 @@ def test_skewed_fp8_batch_takes_the_large_tiles_on_the_device():
     # 512 experts: the multi-phase sort (count / scan / scatter kernels) makes the same choice
     run(mi.MoeConfig("skew", 1024, 256, 2048, 512, 4, "fp8", "zipf"), 7, 320)
     run(mi.MoeConfig("skew", 1024, 256, 2048, 512, 4, "fp8", "softmax_renorm"), 8, 32)
+    # the sort and the grouped GEMMs as two calls: the GEMM entry point's own tile-list pass makes the same choice
+    run(zipf, 9, 320, unfused=True)
+    run(mi.MoeConfig("skew", 256, 512, 2048, 64, 4, "fp8", "softmax_renorm"), 10, 32, unfused=True)
+    run(zipf, 11, 320, unfused=True, mask=np.array(([1, 1, 1, 1, 1, 1, 1, 0] * 8), dtype=np.int32))
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp8", "int8"])

@@ -289,7 +289,8 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
                                                                const int* __restrict__ post_pad_ptr, int unit,
                                                                int experts, int rows_per_tile, int max_units,
                                                                int max_tiles, int* __restrict__ tile_map,
-                                                               int* __restrict__ inv, int n_inv)
+                                                               int* __restrict__ inv, int n_inv, int alt_rows_per_tile,
+                                                               int alt_min_rows, int alt_min_active)
 {
     for(int i = blockIdx.x * kPrepBlock + threadIdx.x; i < n_inv; i += gridDim.x * kPrepBlock)
         inv[i] = -1;
@@ -310,6 +311,19 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
             hi = lower_bound_dev(sorted_eid, nunits, e + 1);
         }
         const int rows = (hi - lo) * unit;
+        // the same choice between two tile heights as the sort makes in the fused entry point (see alt_mblk), from
+        // the rows per active expert; 0 in the header: no choice, the kernels do not look
+        if(alt_rows_per_tile > 0) // (uniform; experts <= 1024 = one pass of this loop)
+        {
+            int active;
+            (void)block_exclusive_scan<kPrepWaves>(rows > 0 ? 1 : 0, s_wave, active);
+            if(active >= alt_min_active && (int64_t)nunits * unit >= (int64_t)alt_min_rows * active)
+                rows_per_tile = alt_rows_per_tile;
+            if(threadIdx.x == 0)
+                tile_map[1] = rows_per_tile;
+        }
+        else if(threadIdx.x == 0)
+            tile_map[1] = 0;
         const int nt   = ceil_div(rows, rows_per_tile);
         int sum;
         const int tb   = total + block_exclusive_scan<kPrepWaves>(nt, s_wave, sum);
@@ -754,7 +768,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     const int mblk     = pick_mblk(t, T, K, E, H, I);
     const int max_units = (int)ceil_div<int64_t>(ws.max_pad, t.block_m);
     // the sort chose between two tile heights (see alt_mblk): both kernel families are launched for each GEMM
-    const int alt           = prep_done ? alt_mblk(t, T, K, E, H, I) : 0;
+    const int alt           = alt_mblk(t, T, K, E, H, I);
     const int alt_max_tiles = alt ? (int)std::min<int64_t>(ws.max_tiles, E + ws.max_pad / (alt * 32) + 1) : 0;
 
     const int n_inv      = T * K;
@@ -765,7 +779,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
         hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
                            static_cast<const int*>(a.sorted_expert_ids_ptr),
                            static_cast<const int*>(a.num_sorted_tiles_ptr), t.block_m, E, mblk * 32, max_units,
-                           ws.max_tiles, tile_map, inv, n_inv);
+                           ws.max_tiles, tile_map, inv, n_inv, alt * 32, kAltMinRows,
+                           ceil_div(device_info().num_cu, ceil_div((t.gate_only ? 1 : 2) * I, 256)));
         hipLaunchKernelGGL(moe_inv_kernel, dim3(std::min<int>(ceil_div<int64_t>(ws.max_pad, 256), 1024)), dim3(256), 0,
                            stream, static_cast<const int*>(a.sorted_token_ids_ptr),
                            static_cast<const int*>(a.num_sorted_tiles_ptr), (int)ws.max_pad, T, K, inv);
@@ -1021,7 +1036,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
         hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
                            static_cast<const int*>(a.p_sorted_expert_ids), static_cast<const int*>(a.p_max_token_id),
                            a.block_m, E, mblk * 32, (int)ceil_div<int64_t>(L.max_pad, a.block_m), L.max_tiles, tile_map,
-                           inv, n_inv);
+                           inv, n_inv, 0, 0, 0);
         if(!g1)
             hipLaunchKernelGGL(moe_inv_kernel, dim3(std::min<int>(ceil_div<int64_t>(L.max_pad, 256), 1024)), dim3(256), 0,
                                stream, static_cast<const int*>(a.p_sorted_token_ids),
