@@ -45,15 +45,20 @@ def test_rowwise_quant(rows, cols, kind):
     assert np.array_equal(s2.cpu().numpy(), rs) and np.array_equal(_raw(q2), rq)
 
 
+# second line: scale tables larger than an XCD's L2, short and long rows, many slots
 @pytest.mark.parametrize("tokens,hidden,experts,topk", [(1, 64, 4, 2), (64, 4096, 128, 8), (300, 1024, 8, 2), (17, 7168, 256, 8),
-                                                         (9, 10240, 4, 3), (5, 100, 3, 2)])
+                                                         (9, 10240, 4, 3), (5, 100, 3, 2),
+                                                         (33, 2048, 512, 5), (5, 16400, 64, 3), (40, 7184, 128, 64),
+                                                         (3, 7168, 128, 65)])
 @pytest.mark.parametrize("kind", ["int8", "fp8"])
 def test_moe_smoothquant(tokens, hidden, experts, topk, kind):
     import torch
     import therock_amd as ta
 
     rng = np.random.default_rng(tokens * 7 + hidden)
-    x = _bf16(rng.standard_normal((tokens, hidden)).astype(np.float32))
+    x = _bf16((rng.standard_normal((tokens, hidden)) * rng.choice([1e-2, 1, 30], size=(tokens, 1))).astype(np.float32))
+    if tokens > 2:
+        x[tokens // 2] = 0  # a row of zeros: scale 0, codes 0
     sm = torch.from_numpy((0.25 + rng.random((experts, hidden)) * 2).astype(np.float32)).cuda()
     ids = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int32)
     qy, ys = ta.moe_smoothquant(x, sm, torch.from_numpy(ids).cuda(), kind)
@@ -62,6 +67,10 @@ def test_moe_smoothquant(tokens, hidden, experts, topk, kind):
     rq, rs = oracle.smoothquant(x.float().cpu().numpy(), sm.cpu().numpy(), ids, dt)
     assert np.array_equal(ys.cpu().numpy(), rs)
     assert np.array_equal(_raw(qy), rq)
+    # a second call into the same outputs
+    ta.moe_smoothquant(x, sm, torch.from_numpy(ids).cuda(), kind, out=(qy, ys))
+    torch.cuda.synchronize()
+    assert np.array_equal(ys.cpu().numpy(), rs) and np.array_equal(_raw(qy), rq)
 
 
 @pytest.mark.parametrize("kind", ["int8", "fp8"])

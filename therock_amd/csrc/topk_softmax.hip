@@ -43,25 +43,6 @@ __device__ inline float wave_sum(float v)
     return v;
 }
 
-// Wave-wide maximum / minimum of a 32-bit unsigned value, the same in every lane afterwards.  Data-parallel
-// primitives instead of LDS-routed shuffles: an inclusive scan over each row of 16 lanes (row_shr 1, 2, 4, 8; lanes
-// shifted in from outside a row read the identity), then lane 15 of rows 0 and 2 is combined into rows 1 and 3
-// (row_bcast:15) and lane 31 into rows 2 and 3 (row_bcast:31): lane 63 holds the result.
-template <bool MAX>
-__device__ inline uint32_t wave_reduce_u32(uint32_t v)
-{
-    constexpr int ident = MAX ? 0 : -1;
-    auto combine = [](uint32_t a, uint32_t b) { return MAX ? max(a, b) : min(a, b); };
-    int x = static_cast<int>(v);
-    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x111, 0xf, 0xf, false))); // row_shr:1
-    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x112, 0xf, 0xf, false))); // row_shr:2
-    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x114, 0xf, 0xf, false))); // row_shr:4
-    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x118, 0xf, 0xf, false))); // row_shr:8
-    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x142, 0xa, 0xf, false))); // row_bcast:15
-    x = static_cast<int>(combine(x, __builtin_amdgcn_update_dpp(ident, x, 0x143, 0xc, 0xf, false))); // row_bcast:31
-    return static_cast<uint32_t>(__builtin_amdgcn_readlane(x, 63));
-}
-
 template <typename In, int PER_LANE>
 __global__ __launch_bounds__(kRouterBlock) void topk_softmax_kernel(const RouterParams p)
 {

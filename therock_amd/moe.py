@@ -300,16 +300,22 @@ def permute_weights(w, nw: int = 16, kw: int = 4, kv: int | None = None, inverse
     return out
 
 
-def moe_smoothquant(x, smscale, topk_ids, q_dtype: str = "int8", stream=None):
+def moe_smoothquant(x, smscale, topk_ids, q_dtype: str = "int8", stream=None, out=None):
     """CK's moe_smoothquant(traits, args, stream): x [tokens, hidden] bf16, smscale [experts, hidden] fp32,
-    topk_ids [tokens, topk] int32 -> (qy [topk, tokens, hidden] int8 / e4m3, yscale [topk, tokens] fp32)."""
+    topk_ids [tokens, topk] int32 -> (qy [topk, tokens, hidden] int8 / e4m3, yscale [topk, tokens] fp32).
+    out: a (qy, yscale) pair of contiguous tensors to write into instead of new ones."""
     import torch
 
     tokens, hidden = x.shape
     experts, topk = smscale.shape[0], topk_ids.shape[1]
     st = {"fp8": torch.float8_e4m3fn, "int8": torch.int8}[q_dtype]
-    qy = torch.empty((topk, tokens, hidden), dtype=st, device=x.device)
-    ys = torch.empty((topk, tokens), dtype=torch.float32, device=x.device)
+    if out is not None:
+        qy, ys = out
+        assert qy.shape == (topk, tokens, hidden) and qy.dtype == st and qy.is_contiguous()
+        assert ys.shape == (topk, tokens) and ys.dtype == torch.float32 and ys.is_contiguous()
+    else:
+        qy = torch.empty((topk, tokens, hidden), dtype=st, device=x.device)
+        ys = torch.empty((topk, tokens), dtype=torch.float32, device=x.device)
     a = _lib.SmoothquantArgs(_ptr(x), _ptr(smscale), _ptr(topk_ids), _ptr(ys), _ptr(qy), tokens, hidden, experts, topk,
                              x.stride(0) if tokens else hidden, hidden)
     _check(_lib.load().mi355_moe_smoothquant(C.byref(a), _lib.DTYPES[q_dtype], _stream(stream)), "moe_smoothquant")
