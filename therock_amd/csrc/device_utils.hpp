@@ -73,6 +73,45 @@ __device__ inline int block_exclusive_scan(int v, int* s_wave, int& total)
     return r;
 }
 
+// N such scans at once (N values per thread), sharing the three barriers.  s_wave: N x (NWAVES + 1) ints of LDS.
+template <int NWAVES, int N>
+__device__ inline void block_exclusive_scan_n(const int (&v)[N], int (*s_wave)[NWAVES + 1], int (&excl)[N], int (&total)[N])
+{
+    static_assert(NWAVES <= kWave, "one wave scans the wave totals");
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    int x[N];
+#pragma unroll
+    for(int q = 0; q < N; q++)
+    {
+        x[q] = wave_inclusive_scan(v[q]);
+        if(lane == kWave - 1)
+            s_wave[q][wave] = x[q];
+    }
+    __syncthreads();
+    if(wave == 0)
+    {
+#pragma unroll
+        for(int q = 0; q < N; q++)
+        {
+            const int w  = lane < NWAVES ? s_wave[q][lane] : 0;
+            const int xx = wave_inclusive_scan(w);
+            if(lane < NWAVES)
+                s_wave[q][lane] = xx - w;
+            if(lane == NWAVES - 1)
+                s_wave[q][NWAVES] = xx;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for(int q = 0; q < N; q++)
+    {
+        excl[q]  = s_wave[q][wave] + x[q] - v[q];
+        total[q] = s_wave[q][NWAVES];
+    }
+    __syncthreads();
+}
+
 __device__ inline float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
 
 // round-to-nearest-even float -> bf16 bits (NaN stays NaN)

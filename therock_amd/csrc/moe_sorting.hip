@@ -119,6 +119,7 @@ struct ScanShared
     int tbase[kMaxExperts]; // first output tile of the expert
     int oeid[kMaxExperts];  // expert id written to sorted_expert_ids
     int wave[kScanWaves + 1];
+    int wave3[3][kScanWaves + 1];
 };
 
 // Pass 2, run by one 1024-thread block.  counts is [nseg][E] (global or LDS): on entry the
@@ -179,10 +180,13 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
     const bool on_rank = tid < E && (mask == nullptr || mask[tid] != 0);
     const int my_cnt   = tid < E ? s.cnt[tid] : 0;
     const int my_tiles = on_rank ? ceil_div(my_cnt, U) : 0;
-    int total_tiles, total_ids;
-    const int tbase = block_exclusive_scan<kScanWaves>(my_tiles, s.wave, total_tiles);
-    const int oeid  = block_exclusive_scan<kScanWaves>(on_rank ? 1 : 0, s.wave, total_ids);
-    (void)total_ids;
+    // one pass of block scans for the first output tile of each expert, the output expert ids and the number of
+    // experts that have tokens
+    const int scan_in[3] = {my_tiles, on_rank ? 1 : 0, my_tiles > 0 ? 1 : 0};
+    int scan_ex[3], scan_total[3];
+    block_exclusive_scan_n<kScanWaves, 3>(scan_in, s.wave3, scan_ex, scan_total);
+    const int tbase = scan_ex[0], oeid = scan_ex[1];
+    const int total_tiles = scan_total[0], active = scan_total[2];
     if(tid < kMaxExperts)
     {
         s.tiles[tid] = my_tiles;
@@ -221,6 +225,41 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const int pad  = mock_id(T, K);
+    if((int64_t)E * U <= 65536)
+    {
+        // The usual sizes, flat over the whole block (this pass is one workgroup; a wave per expert walking its
+        // tiles and pad cells in turn was a third of the one-workgroup sort's time at decode sizes).  An expert has
+        // fewer than U pad cells: candidate (expert, o) is one of them when o < tiles * U - count.
+        for(int idx = tid; idx < E * U; idx += kScanBlock)
+        {
+            const int ex = idx / U;
+            const int o  = idx - ex * U;
+            const int tl = s.tiles[ex];
+            const int c  = s.cnt[ex];
+            if(tl > 0 && o < tl * U - c)
+            {
+                const int pos   = s.tbase[ex] * U + c + o;
+                sorted_ids[pos] = pad;
+                sorted_w[pos]   = 0.f;
+            }
+        }
+        // the expert of output tile t: the last one whose first tile is at or before t (experts without tiles share
+        // their first-tile index with the next expert that has some, and come before it)
+        for(int t = tid; t < total_tiles; t += kScanBlock)
+        {
+            int lo = 0, hi = E; // first expert with tbase > t
+            while(lo < hi)
+            {
+                const int mid = (lo + hi) >> 1;
+                if(s.tbase[mid] <= t)
+                    lo = mid + 1;
+                else
+                    hi = mid;
+            }
+            sorted_eid[t] = s.oeid[lo - 1];
+        }
+    }
+    else
     for(int ex = wave; ex < E; ex += kScanWaves)
     {
         const int tl = s.tiles[ex];
@@ -249,8 +288,6 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
         int rows_per_tile = plan.rows_per_tile;
         if(plan.alt_rows_per_tile > 0) // (uniform: every thread takes this branch or none)
         {
-            int active;
-            (void)block_exclusive_scan<kScanWaves>(rows > 0 ? 1 : 0, s.wave, active);
             if(active >= plan.alt_min_active && (int64_t)total_tiles * U >= (int64_t)plan.alt_min_rows * active)
                 rows_per_tile = plan.alt_rows_per_tile;
             if(tid == 0)
