@@ -102,12 +102,27 @@ __device__ inline void walk_segment(const int* __restrict__ ids, const float* __
                                     int* __restrict__ inv = nullptr)
 {
     const int lane = threadIdx.x & (kWave - 1);
-    for(int i0 = begin; i0 < end; i0 += kWave)
+    // eight steps' entries are fetched together (a segment of the multi-phase passes is eight steps): one load
+    // latency per segment instead of one per step
+    constexpr int kAhead = 8;
+    for(int i0 = begin; i0 < end; i0 += kAhead * kWave)
     {
-        const int i   = i0 + lane;
-        const int e   = i < end ? ids[i] : -1;
-        const float w = SCATTER && i < end ? weights[i] : 0.f;
-        walk_step<SCATTER>(i, e, w, i < end, K, E, nbits, cnt, out_ids, out_w, inv);
+        int ev[kAhead];
+        float wv[kAhead];
+#pragma unroll
+        for(int u = 0; u < kAhead; u++)
+        {
+            const int i = i0 + u * kWave + lane;
+            ev[u]       = i < end ? ids[i] : -1;
+            wv[u]       = SCATTER && i < end ? weights[i] : 0.f;
+        }
+#pragma unroll
+        for(int u = 0; u < kAhead; u++)
+            if(i0 + u * kWave < end)
+            {
+                const int i = i0 + u * kWave + lane;
+                walk_step<SCATTER>(i, ev[u], wv[u], i < end, K, E, nbits, cnt, out_ids, out_w, inv);
+            }
     }
 }
 
