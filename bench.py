@@ -258,9 +258,9 @@ def run_neighbours(cfg, inp, buf, steps):
     return out
 
 
-def cpu_baseline(cfg, inp, max_rows=256):
+def cpu_baseline(cfg, inp, max_rows=256, n_experts=3):
     """ck_tile's own host reference (oracle/_ref) timed on this machine's cores on a bounded
-    sample of the workload: every row routed to one expert (T'=rows, E'=1, K'=1), operands
+    sample of the workload: every row routed to each of a few experts (T'=rows, E'=1, K'=1 per expert), operands
     de-quantised to fp32 because the reference ignores scale tensors.  Falls back to the C
     restatement when oracle/_ref is not built."""
     import numpy as np
@@ -268,10 +268,6 @@ def cpu_baseline(cfg, inp, max_rows=256):
 
     import oracle
 
-    e0 = int(inp["topk_ids"][0, 0])
-    t_idx, k_idx = torch.nonzero(inp["topk_ids"] == e0, as_tuple=True)
-    t_idx, k_idx = t_idx[:max_rows], k_idx[:max_rows]
-    n = int(t_idx.numel())
     H, I = cfg.hidden, cfg.inter
 
     def deq(x, scale):
@@ -281,26 +277,39 @@ def cpu_baseline(cfg, inp, max_rows=256):
     def rows(x, idx):  # row gather that also works for 8-bit float storage
         return x.view(torch.uint8)[idx].view(x.dtype) if x.element_size() == 1 else x[idx]
 
-    a = deq(rows(inp["a"], t_idx), None if inp["a_scale"] is None else inp["a_scale"][t_idx]).cpu().numpy()
-    g = deq(inp["g"][e0], None if inp["g_scale"] is None else inp["g_scale"][e0]).cpu().numpy()[None]
-    d = deq(inp["d"][e0], None if inp["d_scale"] is None else inp["d_scale"][e0]).cpu().numpy()[None]
-    ids = np.zeros((n, 1), dtype=np.int32)
-    w = inp["topk_weight"][t_idx, k_idx].cpu().numpy().reshape(n, 1)
-    flops = 6.0 * n * H * I
-    sample = (f"the {n} rows routed to expert {e0} of {cfg.name} as a T'={n}, E'=1, K'=1 problem "
-              f"(same H={H}, I={I}), de-quantised fp32 operands")
-    if oracle.ck_ref() is not None:
+    # the experts of the first token's first slots, one E'=1 problem each: 10 to 20 s of CPU work on the headline workload
+    experts = []
+    for e in inp["topk_ids"][0].tolist():
+        if e not in experts:
+            experts.append(int(e))
+    experts = experts[:n_experts]
+    use_ref = oracle.ck_ref() is not None
+    flops, dt, n_rows = 0.0, 0.0, []
+    for e0 in experts:
+        t_idx, k_idx = torch.nonzero(inp["topk_ids"] == e0, as_tuple=True)
+        t_idx, k_idx = t_idx[:max_rows], k_idx[:max_rows]
+        n = int(t_idx.numel())
+        a = deq(rows(inp["a"], t_idx), None if inp["a_scale"] is None else inp["a_scale"][t_idx]).cpu().numpy()
+        g = deq(inp["g"][e0], None if inp["g_scale"] is None else inp["g_scale"][e0]).cpu().numpy()[None]
+        d = deq(inp["d"][e0], None if inp["d_scale"] is None else inp["d_scale"][e0]).cpu().numpy()[None]
+        ids = np.zeros((n, 1), dtype=np.int32)
+        w = inp["topk_weight"][t_idx, k_idx].cpu().numpy().reshape(n, 1)
         t0 = time.perf_counter()
-        s = oracle.ck_moe_sorting(ids, w, 1, cfg.unit)
-        oracle.ck_fused_moe(a, g, d, *s, cfg.unit, n, 1, H, I, 1, f32_inputs=True)
-        dt = time.perf_counter() - t0
+        if use_ref:
+            s = oracle.ck_moe_sorting(ids, w, 1, cfg.unit)
+            oracle.ck_fused_moe(a, g, d, *s, cfg.unit, n, 1, H, I, 1, f32_inputs=True)
+        else:
+            s = oracle.moe_sorting(ids, w, 1, cfg.unit)
+            oracle.fused_moe(a, oracle.DT_F32, g, oracle.DT_F32, d, oracle.DT_F32, *s, cfg.unit, n, 1, H, I, 1)
+        dt += time.perf_counter() - t0
+        flops += 6.0 * n * H * I
+        n_rows.append(n)
+    sample = (f"the rows routed to experts {experts} of {cfg.name} ({n_rows} rows), each as a T'=rows, E'=1, K'=1 problem "
+              f"(same H={H}, I={I}), de-quantised fp32 operands")
+    if use_ref:
         return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "reference", "seconds": dt,
                 "sample": sample + "; ck_tile::reference_moe_sorting + reference_fused_moe (GEMM phase is "
                 "single-threaded by construction, the final top-k reduce uses all cores)"}
-    t0 = time.perf_counter()
-    s = oracle.moe_sorting(ids, w, 1, cfg.unit)
-    oracle.fused_moe(a, oracle.DT_F32, g, oracle.DT_F32, d, oracle.DT_F32, *s, cfg.unit, n, 1, H, I, 1)
-    dt = time.perf_counter() - t0
     return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
             "seconds": dt, "sample": sample + "; C restatement of the ck_tile reference (oracle/moe_oracle.c)"}
 
