@@ -271,20 +271,6 @@ __global__ __launch_bounds__(kBlock, 2) void moe_gemm_kernel(const GemmParams p)
 constexpr int kPrepBlock = 1024;
 constexpr int kPrepWaves = kPrepBlock / kWave;
 
-__device__ inline int lower_bound_dev(const int* a, int n, int key)
-{
-    int lo = 0, hi = n;
-    while(lo < hi)
-    {
-        const int mid = (lo + hi) >> 1;
-        if(a[mid] < key)
-            lo = mid + 1;
-        else
-            hi = mid;
-    }
-    return lo;
-}
-
 __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restrict__ sorted_eid,
                                                                const int* __restrict__ post_pad_ptr, int unit,
                                                                int experts, int rows_per_tile, int max_units,
@@ -297,9 +283,29 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
     if(blockIdx.x != 0)
         return;
     __shared__ int s_wave[kPrepWaves + 1];
+    __shared__ int s_lo[kPrepBlock], s_hi[kPrepBlock]; // first and one-past-last sort unit of each expert
     const int post_pad = post_pad_ptr[0];
     int nunits         = post_pad / unit;
     nunits             = max(0, min(nunits, max_units));
+    // sorted_expert_ids is non-decreasing: the units of an expert form one run, found by looking at each unit's
+    // neighbours - independent loads, where a binary search per expert is a chain of a dozen dependent ones
+    s_lo[threadIdx.x] = 0;
+    s_hi[threadIdx.x] = 0;
+    __syncthreads();
+    for(int u = threadIdx.x; u < nunits; u += kPrepBlock)
+    {
+        const int e    = sorted_eid[u];
+        const int prev = u > 0 ? sorted_eid[u - 1] : -1;
+        const int next = u + 1 < nunits ? sorted_eid[u + 1] : -1;
+        if(e >= 0 && e < experts)
+        {
+            if(prev != e)
+                s_lo[e] = u;
+            if(next != e)
+                s_hi[e] = u + 1;
+        }
+    }
+    __syncthreads();
     int total          = 0;
     for(int e0 = 0; e0 < experts; e0 += kPrepBlock) // experts <= 1024: one pass
     {
@@ -307,8 +313,8 @@ __global__ __launch_bounds__(kPrepBlock) void moe_prep_kernel(const int* __restr
         int lo = 0, hi = 0;
         if(e < experts)
         {
-            lo = lower_bound_dev(sorted_eid, nunits, e);
-            hi = lower_bound_dev(sorted_eid, nunits, e + 1);
+            lo = s_lo[e];
+            hi = max(s_hi[e], lo);
         }
         const int rows = (hi - lo) * unit;
         // the same choice between two tile heights as the sort makes in the fused entry point (see alt_mblk), from
