@@ -314,6 +314,67 @@ def cpu_baseline(cfg, inp, max_rows=256, n_experts=3):
             "seconds": dt, "sample": sample + "; C restatement of the ck_tile reference (oracle/moe_oracle.c)"}
 
 
+MAX_LINE_BYTES = 4096  # the one JSON line on stdout stays below this; everything else goes to stderr
+
+
+def _r(x, n=4):
+    return None if x is None else float(f"{x:.{n}g}")
+
+
+def _roof_short(r):
+    """The roofline fields a reader of the one-line result needs (the long form is printed on stderr)."""
+    if not r:
+        return None
+    out = {"kernel": r["kernel"], "bound": r["bound"], "achieved": _r(r["achieved"], 5), "peak": r["peak"],
+           "unit": r["unit"], "frac": _r(r["frac"]), "traffic": r.get("traffic"),
+           "avg_launch_ms": _r(r["avg_launch_ms"], 5), "algorithmic_bytes": r.get("algorithmic_bytes"),
+           "algorithmic_flop": r.get("algorithmic_flop")}
+    return out
+
+
+def _workload_short(r):
+    """ms per pass, the rate the workload is graded on and its fraction of that peak."""
+    if "error" in r:
+        return {"error": r["error"][:80]}
+    rows_per_expert = r["tokens"] * r["topk"] / r["experts"]
+    if rows_per_expert >= 64:
+        return {"ms": _r(r["ms_per_step"]), "rate": _r(r["tflops"]), "unit": "TFLOP/s", "frac": _r(r["frac_mfma_peak"], 3)}
+    return {"ms": _r(r["ms_per_step"]), "rate": _r(r["hbm_GBps"]), "unit": "GB/s", "frac": _r(r["frac_hbm_peak"], 3)}
+
+
+def build_line(cfg, steps, warmup, res, roof, roof1, cpu, router, neighbours, workloads):
+    """The one JSON line of the result: headline fields, the two roofline entries, the CPU baseline and one short
+    record per other workload.  Kept under MAX_LINE_BYTES: readers that keep only the tail of stdout must still
+    see a whole line."""
+    if cpu:
+        cpu = {k: (_r(v, 5) if isinstance(v, float) else v) for k, v in cpu.items()}
+        if len(cpu.get("sample", "")) > 300:
+            cpu["sample"] = cpu["sample"][:297] + "..."
+    line = {
+        "metric": METRIC, "value": _r(res["tflops"], 6), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": _r(res["ms_per_step"], 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": {"bf16": "bf16", "fp8": "fp8_e4m3", "int8": "int8"}[cfg.dtype],
+        "data": "synthetic (seeded N(0,1) activations, N(0,0.02) weights, pre-quantised, resident in HBM)",
+        "config": {"workload": f"{cfg.name}: tokens={cfg.tokens} hidden={cfg.hidden} inter={cfg.inter} "
+                               f"experts={cfg.experts} topk={cfg.topk} block_m={cfg.unit} router={cfg.router}",
+                   "path": "moe_sorting + gemm0(gate,up,SiLU*up) + gemm1(down) + combine, one stream"},
+        "frac_of_mfma_peak": _r(res["frac_mfma_peak"]), "tokens_per_s": _r(res["tokens_per_s"], 6),
+        "hbm_GBps": _r(res["hbm_GBps"], 5), "kernel_avg_ms": {k: _r(v, 4) for k, v in res["kernel_avg_ms"].items()},
+        "roofline": _roof_short(roof), "roofline_gemm1": _roof_short(roof1), "cpu_baseline": cpu,
+    }
+    if router and "avg_launch_ms" in router:
+        line["router_ms"] = _r(router["avg_launch_ms"])
+    if neighbours and "error" not in neighbours:
+        line["neighbours_ms"] = {k: _r(v["ms"]) for k, v in neighbours.items()}
+    line["workloads"] = {name: _workload_short(r) for name, r in workloads.items()}
+    # never let the line outgrow what a tail of stdout holds: drop the optional parts, longest first
+    for key in ("workloads", "neighbours_ms", "kernel_avg_ms"):
+        if len(json.dumps(line, separators=(",", ":"))) < MAX_LINE_BYTES:
+            break
+        line.pop(key, None)
+    return line
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -433,21 +494,14 @@ def main():
                 log(f"[bench] {name} failed: {e!r}")
                 extra[name] = {"error": repr(e)}
 
-    line = {
-        "metric": METRIC, "value": res["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
-        "warmup": a.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": {"bf16": "bf16", "fp8": "fp8_e4m3", "int8": "int8"}[cfg.dtype],
-        "data": "synthetic (seeded N(0,1) activations, N(0,0.02) weights, pre-quantised, resident in HBM)",
-        "config": {"workload": f"{cfg.name}: tokens={cfg.tokens} hidden={cfg.hidden} inter={cfg.inter} "
-                               f"experts={cfg.experts} topk={cfg.topk} block_m={cfg.unit} router={cfg.router}",
-                   "path": "moe_sorting + gemm0(gate,up,SiLU*up) + gemm1(down) + combine, one stream"},
-        "frac_of_mfma_peak": res["frac_mfma_peak"], "tokens_per_s": res["tokens_per_s"],
-        "hbm_GBps": res["hbm_GBps"], "kernel_avg_ms": res["kernel_avg_ms"], "gemm0_tflops": res["gemm0_tflops"],
-        "gemm1_tflops": res["gemm1_tflops"], "roofline": roof, "roofline_gemm1": roofline_of(cfg, res, 1),
-        "cpu_baseline": cpu, "router": router, "neighbours": neighbours, "workloads": others,
-        "extra_workloads": extra,
-    }
-    print(json.dumps(line), flush=True)
+    for group, items in (("workloads", others), ("extra_workloads", extra)):
+        for name, r in items.items():  # the full per-workload records go to stderr, one JSON object per line
+            log("[bench-detail] " + json.dumps({"group": group, "name": name, **r}))
+    log("[bench-detail] " + json.dumps({"group": "headline", "name": cfg.name, **res, "router": router,
+                                        "neighbours": neighbours}))
+    line = build_line(cfg, a.steps, a.warmup, res, roof, roofline_of(cfg, res, 1), cpu, router, neighbours,
+                      {**others, **extra})
+    print(json.dumps(line, separators=(",", ":")), flush=True)
 
 
 if __name__ == "__main__":

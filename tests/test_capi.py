@@ -156,7 +156,7 @@ def test_flatmm_operand_types_on_the_host():
 
 def test_host_only_entry_points():
     lib = _lib.load()
-    assert lib.mi355_moe_version() == 210
+    assert lib.mi355_moe_version() == _lib.header_version() >= 210
     assert lib.mi355_moe_max_num_tokens_padded(128, 8, 2, 32) == 2 * 128 + 8 * 32 - 2
     assert lib.mi355_moe_sorting_workspace_size(64, 128, 8) == 0          # one workgroup, no workspace
     assert lib.mi355_moe_sorting_workspace_size(32768, 64, 6) >= 384 * 64 * 4
@@ -220,6 +220,15 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
         ta.moe_sorting_get_workspace_size(64, 8, 2)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ta.fused_moe(ta.fused_moe_traits(), ta.fused_moe_args())
+
+
+def test_build_entry_compares_the_library_with_the_header():
+    """build() must take the expected version from the header, never from a literal of its own."""
+    src = open(os.path.join(ROOT, "__graft_entry__.py")).read()
+    body = src[src.index("def build()"):src.index("def smoke()")]
+    assert "header_version()" in body
+    import re
+    assert not re.search(r"mi355_moe_version\(\)\s*[=!]=\s*\d", body)
 
 
 def test_bench_refuses_more_than_one_gpu():

@@ -127,6 +127,14 @@ PROTOTYPES = {
 _lib = None
 
 
+def header_version() -> int:
+    """MI355_MOE_VERSION as include/mi355_moe.h defines it (what a freshly built library must report)."""
+    import re
+
+    text = open(os.path.join(os.path.dirname(_HERE), "include", "mi355_moe.h")).read()
+    return int(re.search(r"^#define\s+MI355_MOE_VERSION\s+(\d+)", text, re.M).group(1))
+
+
 def load():
     """dlopen the HIP library; raises RuntimeError when it has not been built."""
     global _lib
