@@ -2,7 +2,7 @@
 """Benchmark of the fused-MoE path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--headline-only] [--no-cpu-baseline]
-                    [--calibrate-copy]
+                    [--calibrate-copy] [--no-sustained]
 
 One "step" is one pass of the whole path (moe_sorting + gate/up GEMM with SiLU*up + down GEMM +
 top-k combine) over one batch of synthetic, already-quantised inputs resident in HBM.  The headline
@@ -168,6 +168,18 @@ def roofline_of(cfg, res, gemm=0):
             "algorithmic_flop": flop, "mfma_TFLOPs": tflops, "mfma_frac": tflops / PEAK_MFMA[cfg.dtype]}
 
 
+def run_sustained(dtype):
+    """The matrix-core rate this device sustains for the workload's MFMA instruction on register operands, with no
+    memory traffic at all: with operands that toggle like real data (the ceiling of any kernel on this box, set by
+    the package's power limit) and with zeros (where the published peak is reached)."""
+    from therock_amd import _lib
+
+    rnd = _lib.mfma_sustained(dtype, 1600, False)
+    zer = _lib.mfma_sustained(dtype, 600, True)
+    return {"random_operands": rnd, "zero_operands": zer, "unit": "TFLOP/s",
+            "what": "independent MFMAs on register operands, 2 waves per SIMD, no memory traffic; measured live"}
+
+
 def run_router(cfg, steps, warmup):
     """Router front-end of the same workload (softmax or sigmoid over [tokens, experts] fp32 logits,
     top-k): an HBM-bound pass over the logits, reported beside the path it feeds."""
@@ -329,6 +341,9 @@ def _roof_short(r):
            "unit": r["unit"], "frac": _r(r["frac"]), "traffic": r.get("traffic"),
            "avg_launch_ms": _r(r["avg_launch_ms"], 5), "algorithmic_bytes": r.get("algorithmic_bytes"),
            "algorithmic_flop": r.get("algorithmic_flop")}
+    if "sustained_peak" in r:  # the rate this device sustains for the same MFMA on register operands, measured live
+        out["sustained_peak"] = _r(r["sustained_peak"], 5)
+        out["frac_of_sustained"] = _r(r["frac_of_sustained"])
     return out
 
 
@@ -342,7 +357,7 @@ def _workload_short(r):
     return {"ms": _r(r["ms_per_step"]), "rate": _r(r["hbm_GBps"]), "unit": "GB/s", "frac": _r(r["frac_hbm_peak"], 3)}
 
 
-def build_line(cfg, steps, warmup, res, roof, roof1, cpu, router, neighbours, workloads):
+def build_line(cfg, steps, warmup, res, roof, roof1, cpu, router, neighbours, workloads, sustained=None):
     """The one JSON line of the result: headline fields, the two roofline entries, the CPU baseline and one short
     record per other workload.  Kept under MAX_LINE_BYTES: readers that keep only the tail of stdout must still
     see a whole line."""
@@ -362,6 +377,10 @@ def build_line(cfg, steps, warmup, res, roof, roof1, cpu, router, neighbours, wo
         "hbm_GBps": _r(res["hbm_GBps"], 5), "kernel_avg_ms": {k: _r(v, 4) for k, v in res["kernel_avg_ms"].items()},
         "roofline": _roof_short(roof), "roofline_gemm1": _roof_short(roof1), "cpu_baseline": cpu,
     }
+    if sustained:
+        line["mfma_sustained"] = {"random_operands": _r(sustained["random_operands"], 5),
+                                  "zero_operands": _r(sustained["zero_operands"], 5), "unit": sustained["unit"],
+                                  "frac_of_sustained": _r(res["tflops"] / sustained["random_operands"])}
     if router and "avg_launch_ms" in router:
         line["router_ms"] = _r(router["avg_launch_ms"])
     if neighbours and "error" not in neighbours:
@@ -384,6 +403,7 @@ def main():
     ap.add_argument("--headline-only", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true")
+    ap.add_argument("--no-sustained", action="store_true", help="skip the measurement of the sustained MFMA rate")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="the named workload, the kernels either side of the path and the router only (profiling runs)")
     # variations of the named workload, for profiling runs of what `extra_workloads` reports
@@ -417,6 +437,17 @@ def main():
         torch.cuda.synchronize()
         log(f"[bench] calibration copy: {src.numel() * 4} bytes read, {dst.numel() * 4} bytes written")
         del src, dst
+    sustained = None
+    if not a.no_sustained:
+        try:
+            sustained = run_sustained(cfg.dtype)
+            log(f"[bench] sustained MFMA rate: {sustained}")
+            for r in (roof,):
+                if r and r["bound"] == "mfma":
+                    r["sustained_peak"] = sustained["random_operands"]
+                    r["frac_of_sustained"] = r["achieved"] / sustained["random_operands"]
+        except Exception as e:
+            log(f"[bench] sustained MFMA rate failed: {e!r}")
     cpu = None
     if not a.no_cpu_baseline:
         try:
@@ -499,8 +530,11 @@ def main():
             log("[bench-detail] " + json.dumps({"group": group, "name": name, **r}))
     log("[bench-detail] " + json.dumps({"group": "headline", "name": cfg.name, **res, "router": router,
                                         "neighbours": neighbours}))
-    line = build_line(cfg, a.steps, a.warmup, res, roof, roofline_of(cfg, res, 1), cpu, router, neighbours,
-                      {**others, **extra})
+    roof1 = roofline_of(cfg, res, 1)
+    if sustained and roof1 and roof1["bound"] == "mfma":
+        roof1["sustained_peak"] = sustained["random_operands"]
+        roof1["frac_of_sustained"] = roof1["achieved"] / sustained["random_operands"]
+    line = build_line(cfg, a.steps, a.warmup, res, roof, roof1, cpu, router, neighbours, {**others, **extra}, sustained)
     print(json.dumps(line, separators=(",", ":")), flush=True)
 
 

@@ -44,6 +44,11 @@ struct moe_sorting_trait
     std::string index_type  = "int32";
     std::string weight_type = "fp32";
     bool local_expert_masking = false;
+    bool clear_workspace_inside_api = false; // accepted: the workspace never needs clearing
+    int dispatch_policy             = 0;     // 0 the library picks, 1 single kernel, 2 multi-launch passes
+    // MoeSortingProblemEx::SkipExpertsWithZeroTokens (ops/fused_moe/kernel/moe_sorting_problem.hpp:35), a template
+    // argument of ck_tile's kernel: false gives every expert of this rank that no token chose one unit of padding
+    bool skip_experts_with_zero_tokens = true;
 };
 
 // ck_tile::MoeSortingHostArgs (ops/fused_moe/kernel/moe_sorting_kernel.hpp:188-222)
@@ -51,9 +56,9 @@ struct moe_sorting_args : public mi355_moe_sorting_args
 {
 };
 
-inline int moe_sorting_get_workspace_size(int tokens, int num_experts, int topk, int /*dispatch_policy*/ = 0)
+inline int moe_sorting_get_workspace_size(int tokens, int num_experts, int topk, int dispatch_policy = 0)
 {
-    return static_cast<int>(mi355_moe_sorting_workspace_size(tokens, num_experts, topk));
+    return static_cast<int>(mi355_moe_sorting_workspace_size2(tokens, num_experts, topk, dispatch_policy));
 }
 
 namespace detail {
@@ -147,10 +152,11 @@ inline float moe_sorting(moe_sorting_trait t, moe_sorting_args a, stream_config 
 {
     if(t.index_type != "int32" || t.weight_type != "fp32")
         return -1.f;
-    if(!t.local_expert_masking)
-        a.p_local_expert_mask = nullptr;
+    const mi355_moe_sorting_traits ct{MI355_MOE_INT32, MI355_MOE_FP32, t.local_expert_masking ? 1 : 0,
+                                      t.clear_workspace_inside_api ? 1 : 0, t.dispatch_policy,
+                                      t.skip_experts_with_zero_tokens ? 1 : 0};
     return detail::run_timed(s, [&] {
-        const int rc = mi355_moe_sorting(&a, s.stream_id_);
+        const int rc = mi355_moe_sorting2(&ct, &a, s.stream_id_);
         detail::throw_on_error(rc, "moe_sorting");
         return rc;
     });

@@ -32,7 +32,7 @@ extern "C" {
 
 /* 210: mi355_fused_moe_traits gained weight_permute and mi355_moe_flatmm_args gained b_shuffle (both appended; a
  * caller built against 200 must be rebuilt), mi355_fused_moe_chosen_tile_rows added */
-#define MI355_MOE_VERSION 210
+#define MI355_MOE_VERSION 220
 
 enum mi355_moe_status
 {
@@ -97,9 +97,33 @@ int64_t mi355_moe_max_num_tokens_padded(int32_t tokens, int32_t num_experts, int
 /* replaces moe_sorting_get_workspace_size() (moe_sorting_kernel.hpp:1394-1438) */
 size_t mi355_moe_sorting_workspace_size(int32_t tokens, int32_t num_experts, int32_t topk);
 
+/* the same with ck_tile's fourth argument (moe_sorting_kernel.hpp:1407-1438): dispatch_policy 0 = the library picks
+ * the kernel (what the three-argument form returns), 1 = always the single kernel (0 bytes), 2 = always the
+ * multi-launch passes; other values return 0 */
+size_t mi355_moe_sorting_workspace_size2(int32_t tokens, int32_t num_experts, int32_t topk, int32_t dispatch_policy);
+
 /* replaces moe_sorting(moe_sorting_trait, moe_sorting_args, stream_config) of CK's
  * example/ck_tile/13_moe_sorting; index type int32 and weight type fp32 are the only ones CK has */
 int mi355_moe_sorting(const mi355_moe_sorting_args* args, void* stream);
+
+/* moe_sorting_trait of CK's example/ck_tile/13_moe_sorting (enums for its strings) plus the one switch of
+ * MoeSortingProblemEx / MoeSortingProblemMp that changes the output (moe_sorting_problem.hpp:35,60). */
+typedef struct mi355_moe_sorting_traits
+{
+    int32_t index_type;                 /* mi355_moe_dtype: INT32 */
+    int32_t weight_type;                /* FP32 */
+    int32_t local_expert_masking;       /* 0: p_local_expert_mask is ignored */
+    int32_t clear_workspace_inside_api; /* accepted; the workspace never needs clearing here */
+    int32_t dispatch_policy;            /* 0 | 1 | 2 as for mi355_moe_sorting_workspace_size2; with 1 p_ws may be NULL
+                                           whatever the size (one workgroup then walks the whole routing list) */
+    int32_t skip_experts_with_zero_tokens; /* 1 = ck_tile's default.  0: an expert of this rank that no token chose
+                                           still owns one unit of padding ids and its expert id in the outputs
+                                           (reference_moe_sorting's skip_experts_with_zero_token = false); the
+                                           output arrays then need topk*tokens + num_experts*unit_size cells */
+} mi355_moe_sorting_traits;
+
+/* mi355_moe_sorting with traits; returns MI355_MOE_E_UNSUPPORTED for index / weight types ck_tile has no kernel for */
+int mi355_moe_sorting2(const mi355_moe_sorting_traits* traits, const mi355_moe_sorting_args* args, void* stream);
 
 /* ----------------------------------------------------------------------------- topk_softmax
  * Router front-end.  Replaces ck_tile::TopkSoftmaxKernel behind TopkSoftmaxHostArgs
@@ -122,7 +146,8 @@ typedef struct mi355_topk_softmax_args
 /* topk_softmax_trait of CK's example/ck_tile/09_topk_softmax, enums for its strings */
 typedef struct mi355_topk_softmax_traits
 {
-    int32_t input_type;  /* mi355_moe_dtype: FP32 | BF16 */
+    int32_t input_type;  /* mi355_moe_dtype: FP32 | BF16 | FP16 (ck_tile's kernel is generic over InputType,
+                            topk_softmax_kernel.hpp:33); the arithmetic is fp32 for all three */
     int32_t weight_type; /* FP32 */
     int32_t experts;     /* CK selects an instance by this upper bound; here informational */
     int32_t activation;  /* 0 = softmax, 1 = sigmoid (TopkSoftmaxWarpPerRowProblem::ActivationIsSoftmax) */
@@ -200,8 +225,8 @@ typedef struct mi355_fused_moe_args
     const void* y_smooth_scale_ptr;
     const void* local_expert_mask_ptr; /* [experts] int32, used when traits.local_expert_masking */
     void* o_ptr;
-    void* ws_ptr;                      /* the example's sort workspace (mi355_moe_sorting_workspace_size() bytes);
-                                          may be NULL: the mi355_moe_workspace then holds it too */
+    void* ws_ptr;                      /* the example's sort workspace: accepted and never touched (it comes without
+                                          a size; the sort's counters live in the mi355_moe_workspace); may be NULL */
     const void* topk_ids_ptr;          /* [tokens, topk] int32 */
     const void* topk_weight_ptr;       /* [tokens, topk] fp32 */
     void* sorted_token_ids_ptr;        /* outputs of the sort, sized as for mi355_moe_sorting */
@@ -398,6 +423,15 @@ int mi355_moe_profile_start(void);
 int mi355_moe_profile_start_kinds(uint32_t kind_mask);
 int mi355_moe_profile_stop(double* ms, int32_t* launches);
 const char* mi355_moe_kernel_name(int32_t kind);
+
+/* ------------------------------------------------------------------- sustained matrix-core rate
+ * No counterpart in ck_tile: a measurement aid for benchmarks.  Runs, for about `milliseconds` on `stream`, a loop of
+ * independent MFMAs of the instruction the grouped GEMMs use for `prec` (mi355_moe_dtype: FP8, BF16, FP16, INT8) on
+ * register operands, without any memory traffic, and returns the rate in TFLOP/s (TOP/s for INT8) averaged over the
+ * second half of that time.  zero_operands = 0: operands with random signs, mantissas and exponents (what real
+ * tensors look like to the multipliers); 1: all zeros.  The two differ widely on a power-limited part: the published
+ * peak is reached on zeros only.  Blocks the calling thread until done; allocates nothing. */
+int mi355_moe_mfma_sustained(int32_t prec, int32_t milliseconds, int32_t zero_operands, double* tflops, void* stream);
 
 const char* mi355_moe_last_error(void);
 int mi355_moe_version(void);

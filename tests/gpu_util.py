@@ -15,15 +15,17 @@ def dev(x, view=None):
 
 
 def run_sorting(topk_ids, weights, experts, unit, mask=None, local_tokens=None, moe_buf=None,
-                fill=True):
+                fill=True, skip_empty=True, dispatch_policy=0):
     """Returns numpy (ids, w, eid, total[2]) with untouched cells holding -1 (when fill)."""
     T, K = topk_ids.shape
     mp = ta.moe_max_num_tokens_padded(T, experts, K, unit)
+    if not skip_empty:  # every expert owns a unit even when no token chose it
+        mp = T * K + experts * unit
     ids = torch.full((mp,), -1, dtype=torch.int32, device="cuda")
     w = torch.full((mp,), -1.0, dtype=torch.float32, device="cuda")
     eid = torch.full(((mp + unit - 1) // unit,), -1, dtype=torch.int32, device="cuda")
     total = torch.full((2,), -7, dtype=torch.int32, device="cuda")
-    ws_bytes = ta.moe_sorting_get_workspace_size(T, experts, K)
+    ws_bytes = ta.moe_sorting_get_workspace_size(T, experts, K, dispatch_policy)
     ws = torch.full((max(ws_bytes, 4),), 0x5A, dtype=torch.uint8, device="cuda")  # deliberately dirty
     args = ta.moe_sorting_args(
         p_topk_ids=dev(topk_ids.astype(np.int32)), p_weights=dev(weights.astype(np.float32)),
@@ -33,7 +35,8 @@ def run_sorting(topk_ids, weights, experts, unit, mask=None, local_tokens=None, 
         p_moe_buf=moe_buf, p_ws=ws if ws_bytes else None, tokens=T, unit_size=unit, num_experts=experts, topk=K,
         moe_buf_interm_dim=0 if moe_buf is None else moe_buf.shape[1],
         moe_buf_elem_bytes=0 if moe_buf is None else moe_buf.element_size())
-    rc = ta.moe_sorting(ta.moe_sorting_trait(local_expert_masking=mask is not None), args)
+    rc = ta.moe_sorting(ta.moe_sorting_trait(local_expert_masking=mask is not None, dispatch_policy=dispatch_policy,
+                                             skip_experts_with_zero_tokens=skip_empty), args)
     assert rc == 0.0
     torch.cuda.synchronize()
     return ids.cpu().numpy(), w.cpu().numpy(), eid.cpu().numpy(), total.cpu().numpy()

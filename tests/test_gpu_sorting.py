@@ -19,11 +19,12 @@ def routing(cfg, seed=1000):
     return mi.route_np(rng.standard_normal((cfg.tokens, cfg.experts), dtype=np.float32), cfg.topk, cfg.router)
 
 
-def check(ids, w, experts, unit, mask=None, local_tokens=None):
+def check(ids, w, experts, unit, mask=None, local_tokens=None, skip_empty=True, dispatch_policy=0):
     from tests.gpu_util import run_sorting
-    got = run_sorting(ids, w, experts, unit, mask=mask, local_tokens=local_tokens)
+    got = run_sorting(ids, w, experts, unit, mask=mask, local_tokens=local_tokens, skip_empty=skip_empty,
+                      dispatch_policy=dispatch_policy)
     T = ids.shape[0] if local_tokens is None else local_tokens
-    ref = oracle.moe_sorting(ids[:T], w[:T], experts, unit, local_expert_mask=mask)
+    ref = oracle.moe_sorting(ids[:T], w[:T], experts, unit, local_expert_mask=mask, skip_empty=skip_empty)
     pp = ref[3]
     print(f"sorting T={T} K={ids.shape[1]} E={experts} U={unit} post_pad={pp}", flush=True)
     assert got[3][0] == pp and got[3][1] == T
@@ -74,6 +75,47 @@ def test_empty_and_skew():
     T = 20000
     ids = np.tile(np.array([[5, 2]], dtype=np.int32), (T, 1))
     check(ids, np.ones((T, 2), np.float32), 64, 32)
+
+
+def test_experts_without_tokens_keep_a_unit_of_padding(golden_dir):
+    """SkipExpertsWithZeroTokens = false (moe_sorting_problem.hpp:35,60): the second worked example of
+    moe_sorting_kernel.hpp:55-117 (expert ids [0,1,2,3,3,4,5], 28 cells), then random shapes with masks, local
+    token counts and both kernels."""
+    g = np.load(os.path.join(golden_dir, "sorting_header_examples.npz"))
+    got = check(g["topk_ids"], g["topk_weight"], 6, 4, skip_empty=False)
+    assert got[3][0] == 28 and list(got[2][:7]) == [0, 1, 2, 3, 3, 4, 5]
+    assert np.array_equal(got[0][:28], g["noskip_ids"]) and np.array_equal(got[2][:7], g["noskip_eid"])
+    for seed in range(6):
+        rng = np.random.default_rng(100 + seed)
+        E = int(rng.choice([3, 64, 100, 256, 257, 1024]))
+        K = int(rng.integers(1, min(E, 8) + 1))
+        T = int(rng.choice([0, 1, 65, 513, 3000]))
+        U = int(rng.choice([1, 16, 32, 48]))
+        pool = rng.permutation(E)[:max(K, E // 3)]  # two thirds of the experts never get a token
+        ids = np.array([rng.permutation(pool)[:K] for _ in range(T)], dtype=np.int32).reshape(T, K)
+        w = rng.random((T, K), dtype=np.float32)
+        check(ids, w, E, U, skip_empty=False)
+        check(ids, w, E, U, skip_empty=False, mask=(rng.random(E) < 0.5).astype(np.int32))
+        check(ids, w, E, U, skip_empty=False, local_tokens=int(rng.integers(0, T + 1)))
+        check(ids, w, E, U, skip_empty=False, dispatch_policy=2)
+
+
+@pytest.mark.parametrize("policy", [1, 2])
+def test_dispatch_policy_forces_a_kernel(policy):
+    """dispatch_policy of moe_sorting_get_workspace_size / moe_sorting_trait (moe_sorting_kernel.hpp:1407-1438): 1 =
+    the single kernel whatever the size (no workspace), 2 = the multi-launch passes whatever the size."""
+    import therock_amd as ta
+    from therock_amd import _lib
+    for T, E, K in ((0, 8, 2), (5, 8, 2), (64, 128, 8), (8192, 256, 8), (3000, 1024, 4)):
+        cfg = mi.MoeConfig("z", max(T, 1), 0, 0, E, K, "bf16", "softmax")
+        ids, w = routing(cfg, 7)
+        ids, w = ids[:T], w[:T]
+        assert (ta.moe_sorting_get_workspace_size(T, E, K, policy) == 0) == (policy == 1)
+        _lib.profile_start()
+        check(ids, w, E, 32, dispatch_policy=policy)
+        kinds = set(_lib.profile_stop())
+        assert kinds == ({"moe_sorting_oneshot"} if policy == 1 else
+                         {"moe_sorting_count", "moe_sorting_scan", "moe_sorting_scatter"}), kinds
 
 
 def test_moe_buf_is_zeroed():

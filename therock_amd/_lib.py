@@ -26,6 +26,12 @@ class SortingArgs(C.Structure):
     ]
 
 
+class SortingTraits(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "index_type", "weight_type", "local_expert_masking", "clear_workspace_inside_api", "dispatch_policy",
+        "skip_experts_with_zero_tokens")]
+
+
 class FusedMoeTraits(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
         "prec_i", "prec_w", "prec_o", "prec_st", "prec_sw", "prec_sq", "prec_kw", "block_m", "activation",
@@ -99,7 +105,9 @@ class SmoothquantArgs(C.Structure):
 PROTOTYPES = {
     "mi355_moe_max_num_tokens_padded": (C.c_int64, [C.c_int32] * 4),
     "mi355_moe_sorting_workspace_size": (C.c_size_t, [C.c_int32] * 3),
+    "mi355_moe_sorting_workspace_size2": (C.c_size_t, [C.c_int32] * 4),
     "mi355_moe_sorting": (C.c_int, [C.POINTER(SortingArgs), C.c_void_p]),
+    "mi355_moe_sorting2": (C.c_int, [C.POINTER(SortingTraits), C.POINTER(SortingArgs), C.c_void_p]),
     "mi355_topk_softmax": (C.c_int, [C.POINTER(TopkSoftmaxTraits), C.POINTER(TopkSoftmaxArgs), C.c_void_p]),
     "mi355_fused_moe_supported": (C.c_int, [C.POINTER(FusedMoeTraits)]),
     "mi355_fused_moe_workspace_size": (C.c_size_t, [C.POINTER(FusedMoeTraits)] + [C.c_int32] * 5),
@@ -120,6 +128,7 @@ PROTOTYPES = {
     "mi355_moe_profile_start_kinds": (C.c_int, [C.c_uint32]),
     "mi355_moe_profile_stop": (C.c_int, [C.POINTER(C.c_double), C.POINTER(C.c_int32)]),
     "mi355_moe_kernel_name": (C.c_char_p, [C.c_int32]),
+    "mi355_moe_mfma_sustained": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]),
     "mi355_moe_last_error": (C.c_char_p, []),
     "mi355_moe_version": (C.c_int, []),
 }
@@ -182,6 +191,15 @@ def profile_stop() -> dict:
     if rc != OK:
         raise RuntimeError(f"profile_stop failed ({rc}): {last_error()}")
     return {lib.mi355_moe_kernel_name(k).decode(): (ms[k], n[k]) for k in range(NUM_KERNELS) if n[k] > 0}
+
+
+def mfma_sustained(prec: str, milliseconds: int = 1500, zero_operands: bool = False, stream=None) -> float:
+    """TFLOP/s (TOP/s for int8) a loop of independent MFMAs on register operands sustains on this device."""
+    out = C.c_double(0.0)
+    rc = load().mi355_moe_mfma_sustained(DTYPES[prec], int(milliseconds), int(bool(zero_operands)), C.byref(out), stream)
+    if rc != OK:
+        raise RuntimeError(f"mfma_sustained failed ({rc}): {last_error()}")
+    return out.value
 
 
 def last_error() -> str:

@@ -194,6 +194,12 @@ __attribute__((visibility("default"))) int mi355_moe_profile_stop(double* ms, in
     return MI355_MOE_OK;
 }
 
+__attribute__((visibility("default"))) int
+mi355_moe_mfma_sustained(int32_t prec, int32_t milliseconds, int32_t zero_operands, double* tflops, void* stream)
+{
+    return mfma_sustained(prec, milliseconds, zero_operands, tflops, static_cast<hipStream_t>(stream));
+}
+
 __attribute__((visibility("default"))) int64_t
 mi355_moe_max_num_tokens_padded(int32_t tokens, int32_t num_experts, int32_t topk, int32_t unit_size)
 {
@@ -206,11 +212,34 @@ mi355_moe_sorting_workspace_size(int32_t tokens, int32_t num_experts, int32_t to
     return sorting_workspace_bytes(tokens, num_experts, topk);
 }
 
+__attribute__((visibility("default"))) size_t
+mi355_moe_sorting_workspace_size2(int32_t tokens, int32_t num_experts, int32_t topk, int32_t dispatch_policy)
+{
+    if(dispatch_policy < 0 || dispatch_policy > 2)
+        return 0;
+    return sorting_workspace_bytes(tokens, num_experts, topk, dispatch_policy);
+}
+
 __attribute__((visibility("default"))) int mi355_moe_sorting(const mi355_moe_sorting_args* args, void* stream)
 {
     if(args == nullptr)
         return fail(MI355_MOE_E_INVALID, "moe_sorting: args is null");
     return launch_moe_sorting(*args, static_cast<hipStream_t>(stream));
+}
+
+__attribute__((visibility("default"))) int
+mi355_moe_sorting2(const mi355_moe_sorting_traits* traits, const mi355_moe_sorting_args* args, void* stream)
+{
+    if(traits == nullptr || args == nullptr)
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: traits or args is null");
+    if(traits->index_type != MI355_MOE_INT32 || traits->weight_type != MI355_MOE_FP32)
+        return fail(MI355_MOE_E_UNSUPPORTED, "moe_sorting: index type %d / weight type %d (int32 / fp32 only)",
+                    traits->index_type, traits->weight_type);
+    mi355_moe_sorting_args a = *args;
+    if(!traits->local_expert_masking)
+        a.p_local_expert_mask = nullptr;
+    return launch_moe_sorting(a, static_cast<hipStream_t>(stream), nullptr, traits->skip_experts_with_zero_tokens == 0,
+                              traits->dispatch_policy);
 }
 
 __attribute__((visibility("default"))) int
@@ -339,8 +368,10 @@ int run_fused_moe(const mi355_fused_moe_traits* traits, const mi355_fused_moe_ar
     s.p_sorted_expert_ids     = a->sorted_expert_ids_ptr;
     s.p_total_tokens_post_pad = a->num_sorted_tiles_ptr;
     s.p_moe_buf               = nullptr;
-    // the example's own sort workspace when the caller passes one, else the slice of the library workspace
-    s.p_ws                    = a->ws_ptr != nullptr ? a->ws_ptr : static_cast<char*>(ws_ptr) + wl.sort_off;
+    // Always the slice of the library workspace: args->ws_ptr (the example's own sort workspace) comes without a
+    // size, and one sized by another formula than mi355_moe_sorting_workspace_size() would be overrun.  It is
+    // accepted and not touched.
+    s.p_ws                    = static_cast<char*>(ws_ptr) + wl.sort_off;
     s.tokens                  = a->num_tokens;
     s.unit_size               = a->block_m;
     s.num_experts             = a->num_experts;

@@ -123,10 +123,16 @@ struct GemmPlan
 };
 
 // ---- sorting launcher shared by the stand-alone and the fused entry points
-int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, const GemmPlan* plan = nullptr);
+// keep_empty: experts without tokens own one tile of padding (ck_tile's SkipExpertsWithZeroTokens = false);
+// dispatch_policy: 0 = the library picks, 1 = single kernel, 2 = multi-launch passes
+int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, const GemmPlan* plan = nullptr,
+                       bool keep_empty = false, int dispatch_policy = 0);
 
 int launch_topk_softmax(const mi355_topk_softmax_traits& t, const mi355_topk_softmax_args& a, hipStream_t stream);
 
-size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk);
+// matrix-core rate sustained on register operands (mfma_ceiling.hip)
+int mfma_sustained(int prec, int milliseconds, int zeros, double* tflops, hipStream_t stream);
+
+size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk, int32_t dispatch_policy = 0);
 
 } // namespace mi355

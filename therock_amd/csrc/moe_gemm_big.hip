@@ -37,6 +37,7 @@
 #include "moe_gemm_device.hpp"
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 namespace mi355 {
@@ -691,17 +692,21 @@ int launch_big_w(const GemmParams& p, int max_tiles, hipStream_t stream)
 {
     constexpr bool kMx  = MODE == kFp8 && !GEMM0;
     const size_t lds    = (GEMM0 && MODE != kBf16W8) ? kLdsBytesPair : kMx ? kLdsBytes : kYsOffset;
-    // the dynamic LDS limit is an attribute of the function on one device: set once per device
-    static bool attr_ok[64] = {};
+    // the dynamic LDS limit is an attribute of the function on one device: set once per device, whichever host
+    // thread gets there first (the others wait for it)
+    static std::once_flag attr_once[64];
     int dev = 0;
     (void)hipGetDevice(&dev);
-    if(dev < 0 || dev >= 64 || !attr_ok[dev])
-    {
-        MI355_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_big_kernel<MODE, GEMM0, WPERM>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        if(dev >= 0 && dev < 64)
-            attr_ok[dev] = true;
-    }
+    hipError_t attr = hipSuccess;
+    auto set_attr   = [&] {
+        attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_big_kernel<MODE, GEMM0, WPERM>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    };
+    if(dev >= 0 && dev < 64)
+        std::call_once(attr_once[dev], set_attr);
+    else
+        set_attr();
+    MI355_HIP_TRY(attr);
     const int grid = round_up(max_tiles * p.n_ntiles, 256); // whole rounds of 32-item chunks over the 8 XCDs
     if(grid <= 0)
         return MI355_MOE_OK;

@@ -17,6 +17,7 @@
 #include "device_utils.hpp"
 
 #include <algorithm>
+#include <mutex>
 
 namespace mi355 {
 namespace {
@@ -143,7 +144,8 @@ struct ScanShared
 __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, int Ep, int U,
                                   const int* __restrict__ mask, int T, int K,
                                   int* __restrict__ sorted_ids, float* __restrict__ sorted_w,
-                                  int* __restrict__ sorted_eid, int* __restrict__ total, const GemmPlan& plan)
+                                  int* __restrict__ sorted_eid, int* __restrict__ total, const GemmPlan& plan,
+                                  bool keep_empty)
 {
     const int tid   = threadIdx.x;
     const int e     = tid & (Ep - 1);
@@ -191,13 +193,15 @@ __device__ inline void scan_phase(ScanShared& s, int* counts, int nseg, int E, i
     __syncthreads();
 
     // an expert that is masked out is skipped without consuming an output expert id; an expert
-    // with no token is skipped but does consume one (reference_moe_sorting.hpp:84-98)
+    // with no token is skipped but does consume one (reference_moe_sorting.hpp:84-98), or, with
+    // skip_experts_with_zero_token = false (keep_empty), owns one tile of padding like the reference's
+    // expert_slices[e] = 1 (:43, :100-112)
     const bool on_rank = tid < E && (mask == nullptr || mask[tid] != 0);
     const int my_cnt   = tid < E ? s.cnt[tid] : 0;
-    const int my_tiles = on_rank ? ceil_div(my_cnt, U) : 0;
+    const int my_tiles = on_rank ? max(ceil_div(my_cnt, U), keep_empty ? 1 : 0) : 0;
     // one pass of block scans for the first output tile of each expert, the output expert ids and the number of
     // experts that have tokens
-    const int scan_in[3] = {my_tiles, on_rank ? 1 : 0, my_tiles > 0 ? 1 : 0};
+    const int scan_in[3] = {my_tiles, on_rank ? 1 : 0, on_rank && my_cnt > 0 ? 1 : 0};
     int scan_ex[3], scan_total[3];
     block_exclusive_scan_n<kScanWaves, 3>(scan_in, s.wave3, scan_ex, scan_total);
     const int tbase = scan_ex[0], oeid = scan_ex[1];
@@ -356,9 +360,13 @@ struct SortParams
     int* counts;           // workspace [nseg][E]
     GemmPlan plan;         // tile_map == nullptr: nothing to prepare
     int tokens, K, E, Ep, nbits, U, nseg, work_blocks;
+    int keep_empty; // experts without tokens own one tile of padding (SkipExpertsWithZeroTokens = false)
 };
 
-// ---- whole sort in one workgroup (block 0); the other blocks zero moe_buf
+// ---- whole sort in one workgroup (block 0); the other blocks zero moe_buf.
+// IN_REGS: the wave's entries fit kMaxSteps registers per lane and are read once; otherwise (a caller that forces the
+// single kernel on a large problem) both walks stream them from memory.
+template <bool IN_REGS>
 __global__ __launch_bounds__(kScanBlock) void moe_sorting_oneshot_kernel(SortParams p)
 {
     extern __shared__ int dyn_lds[]; // [kScanWaves][E]
@@ -384,34 +392,44 @@ __global__ __launch_bounds__(kScanBlock) void moe_sorting_oneshot_kernel(SortPar
     int* inv = p.plan.tile_map != nullptr ? p.plan.inv : nullptr;
     // The wave's entries are read once, all loads issued together, and stay in registers for both walks: fetched
     // step by step they would be a chain of dependent global loads in the one workgroup that does all the work.
-    constexpr int kMaxSteps = kOneShotMaxEntries / kScanBlock;
+    constexpr int kMaxSteps = IN_REGS ? kOneShotMaxEntries / kScanBlock : 1;
     int ev[kMaxSteps];
     float wv[kMaxSteps];
-#pragma unroll
-    for(int u = 0; u < kMaxSteps; u++)
+    if constexpr(IN_REGS)
     {
-        const int i = begin + u * kWave + lane;
-        ev[u]       = i < end ? p.ids[i] : -1;
-        wv[u]       = i < end ? p.weights[i] : 0.f;
-    }
 #pragma unroll
-    for(int u = 0; u < kMaxSteps; u++)
-        if(begin + u * kWave < end)
+        for(int u = 0; u < kMaxSteps; u++)
         {
             const int i = begin + u * kWave + lane;
-            walk_step<false>(i, ev[u], wv[u], i < end, p.K, p.E, p.nbits, cnt, nullptr, nullptr, nullptr);
+            ev[u]       = i < end ? p.ids[i] : -1;
+            wv[u]       = i < end ? p.weights[i] : 0.f;
         }
+#pragma unroll
+        for(int u = 0; u < kMaxSteps; u++)
+            if(begin + u * kWave < end)
+            {
+                const int i = begin + u * kWave + lane;
+                walk_step<false>(i, ev[u], wv[u], i < end, p.K, p.E, p.nbits, cnt, nullptr, nullptr, nullptr);
+            }
+    }
+    else
+        walk_segment<false>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, nullptr, nullptr);
     __syncthreads();
     scan_phase(sh, dyn_lds, kScanWaves, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
-               p.sorted_eid, p.total, p.plan);
+               p.sorted_eid, p.total, p.plan, p.keep_empty != 0);
     __syncthreads();
+    if constexpr(IN_REGS)
+    {
 #pragma unroll
-    for(int u = 0; u < kMaxSteps; u++)
-        if(begin + u * kWave < end)
-        {
-            const int i = begin + u * kWave + lane;
-            walk_step<true>(i, ev[u], wv[u], i < end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w, inv);
-        }
+        for(int u = 0; u < kMaxSteps; u++)
+            if(begin + u * kWave < end)
+            {
+                const int i = begin + u * kWave + lane;
+                walk_step<true>(i, ev[u], wv[u], i < end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w, inv);
+            }
+    }
+    else
+        walk_segment<true>(p.ids, p.weights, begin, end, p.K, p.E, p.nbits, cnt, p.sorted_ids, p.sorted_w, inv);
 }
 
 // ---- pass 1: per-segment expert histogram; trailing blocks zero moe_buf
@@ -449,7 +467,7 @@ __global__ __launch_bounds__(kScanBlock) void moe_sorting_scan_kernel(SortParams
     __shared__ ScanShared sh;
     const int T = real_tokens(p.local_tokens, p.tokens);
     scan_phase(sh, p.counts, p.nseg, p.E, p.Ep, p.U, p.mask, T, p.K, p.sorted_ids, p.sorted_w,
-               p.sorted_eid, p.total, p.plan);
+               p.sorted_eid, p.total, p.plan, p.keep_empty != 0);
 }
 
 // ---- pass 3
@@ -480,18 +498,23 @@ inline bool use_oneshot(int64_t entries, int experts)
 
 } // namespace
 
-size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk)
+// dispatch_policy as in ck_tile's moe_sorting_get_workspace_size (moe_sorting_kernel.hpp:1407-1438): 0 = the library
+// picks, 1 = always the single kernel (no workspace), 2 = always the multi-launch passes
+size_t sorting_workspace_bytes(int32_t tokens, int32_t experts, int32_t topk, int32_t dispatch_policy)
 {
     if(tokens < 0 || experts <= 0 || topk <= 0)
         return 0;
     const int64_t n = (int64_t)tokens * topk;
-    if(use_oneshot(n, experts))
+    if(dispatch_policy == 1 || (dispatch_policy != 2 && use_oneshot(n, experts)))
         return 0;
-    return round_up<size_t>((size_t)ceil_div<int64_t>(n, kSeg) * experts * sizeof(int), 256);
+    return round_up<size_t>((size_t)std::max<int64_t>(ceil_div<int64_t>(n, kSeg), 1) * experts * sizeof(int), 256);
 }
 
-int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, const GemmPlan* plan)
+int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, const GemmPlan* plan, bool keep_empty,
+                       int dispatch_policy)
 {
+    if(dispatch_policy < 0 || dispatch_policy > 2)
+        return fail(MI355_MOE_E_INVALID, "moe_sorting: dispatch_policy=%d outside [0, 2]", dispatch_policy);
     if((a.tokens > 0 && (!a.p_topk_ids || !a.p_weights)) || !a.p_sorted_token_ids || !a.p_sorted_weights ||
        !a.p_sorted_expert_ids || !a.p_total_tokens_post_pad)
         return fail(MI355_MOE_E_INVALID, "moe_sorting: null input or output pointer");
@@ -519,6 +542,7 @@ int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, cons
     p.total        = static_cast<int*>(a.p_total_tokens_post_pad);
     if(plan != nullptr)
         p.plan = *plan;
+    p.keep_empty   = keep_empty ? 1 : 0;
     p.tokens       = a.tokens;
     p.K            = a.topk;
     p.E            = a.num_experts;
@@ -548,20 +572,38 @@ int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, cons
             zero_blocks = 1;
     }
 
-    if(use_oneshot(n, p.E))
+    if(dispatch_policy == 1 || (dispatch_policy == 0 && use_oneshot(n, p.E)))
     {
         p.nseg = kScanWaves;
         KernelTimer timer(MI355_MOE_K_SORT_ONESHOT, stream);
-        hipLaunchKernelGGL(moe_sorting_oneshot_kernel, dim3(1 + zero_blocks), dim3(kScanBlock),
-                           kScanWaves * p.E * sizeof(int), stream, p);
+        const size_t lds = kScanWaves * p.E * sizeof(int); // at most 64 KB beside the 30 KB of static LDS
+        if(use_oneshot(n, p.E))
+            hipLaunchKernelGGL(moe_sorting_oneshot_kernel<true>, dim3(1 + zero_blocks), dim3(kScanBlock), lds, stream, p);
+        else
+        {
+            static std::once_flag once[64];
+            int dev = 0;
+            (void)hipGetDevice(&dev);
+            hipError_t attr = hipSuccess;
+            auto set_attr = [&] {
+                attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_sorting_oneshot_kernel<false>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kScanWaves * kMaxExperts * (int)sizeof(int));
+            };
+            if(dev >= 0 && dev < 64)
+                std::call_once(once[dev], set_attr);
+            else
+                set_attr();
+            MI355_HIP_TRY(attr);
+            hipLaunchKernelGGL(moe_sorting_oneshot_kernel<false>, dim3(1 + zero_blocks), dim3(kScanBlock), lds, stream, p);
+        }
         MI355_HIP_TRY(hipGetLastError());
         return MI355_MOE_OK;
     }
     if(a.p_ws == nullptr)
         return fail(MI355_MOE_E_WORKSPACE, "moe_sorting: p_ws is null but %zu bytes are needed",
-                    sorting_workspace_bytes(a.tokens, a.num_experts, a.topk));
+                    sorting_workspace_bytes(a.tokens, a.num_experts, a.topk, dispatch_policy));
     p.counts      = static_cast<int*>(a.p_ws);
-    p.nseg        = (int)ceil_div<int64_t>(n, kSeg);
+    p.nseg        = (int)std::max<int64_t>(ceil_div<int64_t>(n, kSeg), 1);
     p.work_blocks = ceil_div(p.nseg, kWalkBlock / kWave);
     const size_t lds = (kWalkBlock / kWave) * p.E * sizeof(int);
     {

@@ -10,6 +10,8 @@
 // maximum, the sum and each of the k arg-max rounds are wave reductions.  The work is a single pass
 // over tokens * experts logits, so it is bound by reading them.
 #include "common.hpp"
+
+#include <type_traits>
 #include "device_utils.hpp"
 
 namespace mi355 {
@@ -59,8 +61,10 @@ __global__ __launch_bounds__(kRouterBlock) void topk_softmax_kernel(const Router
         float t     = -INFINITY;
         if(e < p.experts)
         {
-            if constexpr(sizeof(In) == 4)
+            if constexpr(std::is_same_v<In, float>)
                 t = x[e];
+            else if constexpr(std::is_same_v<In, _Float16>)
+                t = static_cast<float>(x[e]);
             else
                 t = bf16_bits_to_float(x[e]);
         }
@@ -158,8 +162,8 @@ int launch_t(const RouterParams& p, hipStream_t stream)
 
 int launch_topk_softmax(const mi355_topk_softmax_traits& t, const mi355_topk_softmax_args& a, hipStream_t stream)
 {
-    if(t.input_type != MI355_MOE_FP32 && t.input_type != MI355_MOE_BF16)
-        return fail(MI355_MOE_E_UNSUPPORTED, "topk_softmax: input type %d (fp32 and bf16 are implemented)", t.input_type);
+    if(t.input_type != MI355_MOE_FP32 && t.input_type != MI355_MOE_BF16 && t.input_type != MI355_MOE_FP16)
+        return fail(MI355_MOE_E_UNSUPPORTED, "topk_softmax: input type %d (fp32, bf16 and fp16 are implemented)", t.input_type);
     if(t.weight_type != MI355_MOE_FP32)
         return fail(MI355_MOE_E_UNSUPPORTED, "topk_softmax: weight type must be fp32");
     if(t.activation != 0 && t.activation != 1)
@@ -174,7 +178,9 @@ int launch_topk_softmax(const mi355_topk_softmax_traits& t, const mi355_topk_sof
         return fail(MI355_MOE_E_INVALID, "topk_softmax: null pointer");
     RouterParams p{a.p_input, static_cast<float*>(a.p_output), static_cast<int*>(a.p_indices), a.num_rows, a.num_experts,
                    a.topk,    a.stride_input, a.stride_output, t.activation, t.renormalize};
-    return t.input_type == MI355_MOE_FP32 ? launch_t<float>(p, stream) : launch_t<uint16_t>(p, stream);
+    if(t.input_type == MI355_MOE_FP32)
+        return launch_t<float>(p, stream);
+    return t.input_type == MI355_MOE_FP16 ? launch_t<_Float16>(p, stream) : launch_t<uint16_t>(p, stream);
 }
 
 } // namespace mi355

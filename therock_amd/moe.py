@@ -47,6 +47,11 @@ class moe_sorting_trait:
     index_type: str = "int32"
     weight_type: str = "fp32"
     local_expert_masking: bool = False
+    clear_workspace_inside_api: bool = False   # accepted: the workspace never needs clearing
+    dispatch_policy: int = 0                   # 0 the library picks, 1 single kernel, 2 multi-launch passes
+    # MoeSortingProblemEx::SkipExpertsWithZeroTokens (a template argument in ck_tile): False gives every expert of
+    # this rank that no token chose one unit of padding
+    skip_experts_with_zero_tokens: bool = True
 
 
 def _ptr(t) -> Optional[int]:
@@ -127,19 +132,21 @@ def moe_max_num_tokens_padded(tokens: int, num_experts: int, topk: int, unit_siz
 
 
 def moe_sorting_get_workspace_size(tokens: int, num_experts: int, topk: int, dispatch_policy: int = 0) -> int:
-    return int(_lib.load().mi355_moe_sorting_workspace_size(tokens, num_experts, topk))
+    return int(_lib.load().mi355_moe_sorting_workspace_size2(tokens, num_experts, topk, dispatch_policy))
 
 
 def moe_sorting(trait: moe_sorting_trait, a: moe_sorting_args, stream=None) -> float:
     """Returns 0.0 on success, -1.0 when the trait has no kernel (as CK's dispatcher does)."""
     if trait.index_type != "int32" or trait.weight_type != "fp32":
         return -1.0
-    mask = a.p_local_expert_mask if trait.local_expert_masking else None
-    s = _lib.SortingArgs(_ptr(a.p_topk_ids), _ptr(a.p_weights), _ptr(mask), _ptr(a.p_local_tokens),
+    t = _lib.SortingTraits(_lib.DTYPES["int32"], _lib.DTYPES["fp32"], int(trait.local_expert_masking),
+                           int(trait.clear_workspace_inside_api), int(trait.dispatch_policy),
+                           int(trait.skip_experts_with_zero_tokens))
+    s = _lib.SortingArgs(_ptr(a.p_topk_ids), _ptr(a.p_weights), _ptr(a.p_local_expert_mask), _ptr(a.p_local_tokens),
                          _ptr(a.p_sorted_token_ids), _ptr(a.p_sorted_weights), _ptr(a.p_sorted_expert_ids),
                          _ptr(a.p_total_tokens_post_pad), _ptr(a.p_moe_buf), _ptr(a.p_ws), a.tokens, a.unit_size,
                          a.num_experts, a.topk, a.moe_buf_interm_dim, a.moe_buf_elem_bytes)
-    _check(_lib.load().mi355_moe_sorting(C.byref(s), _stream(stream)), "moe_sorting")
+    _check(_lib.load().mi355_moe_sorting2(C.byref(t), C.byref(s), _stream(stream)), "moe_sorting")
     return 0.0
 
 
@@ -324,13 +331,13 @@ def moe_smoothquant(x, smscale, topk_ids, q_dtype: str = "int8", stream=None, ou
 
 def topk_softmax(logits, topk: int, activation: str = "softmax", renormalize: bool = False, stream=None):
     """Router front-end (CK's topk_softmax(trait, kargs, stream)): softmax or sigmoid over the experts of
-    each row of `logits` [rows, experts] (fp32 or bf16), then the top-k weights (fp32, descending) and
+    each row of `logits` [rows, experts] (fp32, bf16 or fp16), then the top-k weights (fp32, descending) and
     expert ids (int32).  Returns (weights[rows, topk], ids[rows, topk])."""
     import torch
 
     rows, experts = logits.shape
     assert logits.stride(1) == 1
-    kind = {torch.float32: "fp32", torch.bfloat16: "bf16"}[logits.dtype]
+    kind = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}[logits.dtype]
     w = torch.empty((rows, topk), dtype=torch.float32, device=logits.device)
     ids = torch.empty((rows, topk), dtype=torch.int32, device=logits.device)
     t = _lib.TopkSoftmaxTraits(_lib.DTYPES[kind], _lib.DTYPES["fp32"], experts,
