@@ -411,6 +411,9 @@ def main():
     ap.add_argument("--fused-quant", type=int, default=0, choices=(0, 2),
                     help="int8 workloads: 2 = re-quantise the intermediate activations (down GEMM on int8 MFMAs)")
     ap.add_argument("--router", default="", help="routing instead of the workload's own (e.g. zipf)")
+    ap.add_argument("--hot-expert", action="store_true", help="expert 0 in every token's top-k")
+    ap.add_argument("--weight-permute", type=int, default=0, choices=(0, 1), help="1 = weights in ck_tile's pre-shuffled layout")
+    ap.add_argument("--name", default="", help="name to report the varied workload under")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures one GPU only; run with --gpus 1 (the path is single-GPU: across "
@@ -422,11 +425,12 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     cfg = mi.CONFIGS[a.workload]
-    if a.tokens or a.router:
-        cfg = cfg.scaled(name=f"{cfg.name}_t{a.tokens or cfg.tokens}{'_' + a.router if a.router else ''}",
+    if a.tokens or a.router or a.name:
+        cfg = cfg.scaled(name=a.name or f"{cfg.name}_t{a.tokens or cfg.tokens}{'_' + a.router if a.router else ''}",
                          tokens=a.tokens or cfg.tokens, router=a.router or cfg.router)
     log(f"[bench] {cfg}")
-    res, inp, buf = run_workload(cfg, a.steps, a.warmup, fused_quant=a.fused_quant)
+    res, inp, buf = run_workload(cfg, a.steps, a.warmup, fused_quant=a.fused_quant, hot_expert=a.hot_expert,
+                                 weight_permute=a.weight_permute)
     log(f"[bench] {cfg.name}: {res['ms_per_step']:.3f} ms/step, {res['tflops']:.1f} TFLOP/s, kernels {res['kernel_avg_ms']}")
     roof = roofline_of(cfg, res)
     if a.calibrate_copy:
@@ -497,8 +501,8 @@ def main():
     if not a.headline_only and not a.no_other_workloads:
         i8 = mi.CONFIGS["cfg4_decode_int8_t256"]
         cases = {
-            "cfg4_model_int8_t8192_fused_quant0": (i8.scaled(name="cfg4_model_int8_t8192", tokens=8192), {}),
-            "cfg4_model_int8_t8192_fused_quant2": (i8.scaled(name="cfg4_model_int8_t8192", tokens=8192), {"fused_quant": 2}),
+            "cfg4_model_int8_t8192_fused_quant0": (i8.scaled(name="cfg4_model_int8_t8192_fused_quant0", tokens=8192), {}),
+            "cfg4_model_int8_t8192_fused_quant2": (i8.scaled(name="cfg4_model_int8_t8192_fused_quant2", tokens=8192), {"fused_quant": 2}),
             # 40 rows per expert: the decode kernel with two token blocks per tile
             "cfg4_model_int8_t640": (i8.scaled(name="cfg4_model_int8_t640", tokens=640), {}),
             "cfg2_mixtral_bf16_t160": (mi.CONFIGS["cfg2_mixtral_bf16"].scaled(name="cfg2_mixtral_bf16_t160", tokens=160), {}),

@@ -302,6 +302,140 @@ __global__ __launch_bounds__(256) void moe_smoothquant_vec_kernel(const uint16_t
     }
 }
 
+// Expert-grouped form, for expert tables that do not stay in an XCD's L2 beside the rows streaming through it
+// (256 experts x 7168 columns of fp32 are 7.3 MB against 4 MB): a workgroup owns one expert and one range of
+// kSqRange tokens.  It keeps the expert's smooth scales in registers (read once per workgroup instead of once per
+// row), finds the range's routing entries that name its expert, and quantises those rows one after the other, the
+// next row's activations fetched while the current one is reduced and stored.  The workgroups of one token range sit
+// on one XCD and run together there (workgroup ids go round the eight XCDs: id = (range / 8 * experts + expert) * 8 +
+// range % 8), so that the range's activations come from HBM once and from that XCD's L2 for the other slots.  Each row
+// is computed by the same expressions as in the per-token form: the results are the same bits.
+constexpr int kSqRange   = 128;  // tokens per range
+constexpr int kSqMaxList = 8192; // routing entries of a range (kSqRange x topk)
+template <bool FP8>
+__global__ __launch_bounds__(256) void moe_smoothquant_grouped_kernel(const uint16_t* __restrict__ x,
+                                                                       const float* __restrict__ smscale,
+                                                                       const int* __restrict__ topk_ids, int tokens,
+                                                                       int hidden, int experts, int topk, int64_t x_stride,
+                                                                       int64_t y_stride, unsigned char* __restrict__ qy,
+                                                                       float* __restrict__ yscale)
+{
+    __shared__ float s_red[2][4];
+    __shared__ int s_count;
+    __shared__ int s_list[kSqMaxList];
+    const int xcd   = blockIdx.x & 7;
+    const int e     = (blockIdx.x >> 3) % experts;
+    const int range = (blockIdx.x >> 3) / experts * 8 + xcd;
+    const int t0    = range * kSqRange;
+    if(t0 >= tokens)
+        return;
+    const int nt     = min(kSqRange, tokens - t0);
+    const int chunks = hidden >> 3;
+    const float qmx  = FP8 ? 448.0f : 127.0f;
+    if(threadIdx.x == 0)
+        s_count = 0;
+    __syncthreads();
+    // entries of the range that name this expert (ids outside [0, experts) are clamped like in the other forms)
+    const int* ids = topk_ids + (int64_t)t0 * topk;
+    for(int i = threadIdx.x; i < nt * topk; i += 256)
+        if(min(max(ids[i], 0), experts - 1) == e)
+            s_list[atomicAdd(&s_count, 1)] = i;
+    __syncthreads();
+    const int n = s_count;
+    if(n == 0)
+        return;
+    const float* sr = smscale + (int64_t)e * hidden;
+    float4 sm[kQuantCache][2];
+#pragma unroll
+    for(int j = 0; j < kQuantCache; j++)
+        if(threadIdx.x + 256 * j < chunks)
+        {
+            sm[j][0] = *reinterpret_cast<const float4*>(sr + (threadIdx.x + 256 * j) * 8);
+            sm[j][1] = *reinterpret_cast<const float4*>(sr + (threadIdx.x + 256 * j) * 8 + 4);
+        }
+    auto unpack = [&](const uint4& r, float (&o)[8]) {
+        const uint32_t d[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for(int i = 0; i < 4; i++)
+        {
+            o[2 * i]     = __uint_as_float(d[i] << 16);
+            o[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+        }
+    };
+    auto times_sm = [&](int c, const float (&in)[8], float (&o)[8]) {
+        const float4 s0 = *reinterpret_cast<const float4*>(sr + c * 8);
+        const float4 s1 = *reinterpret_cast<const float4*>(sr + c * 8 + 4);
+        o[0] = in[0] * s0.x; o[1] = in[1] * s0.y; o[2] = in[2] * s0.z; o[3] = in[3] * s0.w;
+        o[4] = in[4] * s1.x; o[5] = in[5] * s1.y; o[6] = in[6] * s1.z; o[7] = in[7] * s1.w;
+    };
+    uint4 raw[kQuantCache];
+    auto fetch_row = [&](int entry) {
+        const uint16_t* xr = x + (int64_t)(t0 + entry / topk) * x_stride;
+#pragma unroll
+        for(int j = 0; j < kQuantCache; j++)
+            if(threadIdx.x + 256 * j < chunks)
+                raw[j] = *reinterpret_cast<const uint4*>(xr + (threadIdx.x + 256 * j) * 8);
+    };
+    fetch_row(s_list[0]);
+    for(int m = 0; m < n; m++)
+    {
+        const int entry    = s_list[m];
+        const int t        = t0 + entry / topk;
+        const int k        = entry - (entry / topk) * topk;
+        const uint16_t* xr = x + (int64_t)t * x_stride;
+        float v[kQuantCache][8];
+        float amax = 0.f;
+#pragma unroll
+        for(int j = 0; j < kQuantCache; j++)
+            if(threadIdx.x + 256 * j < chunks)
+            {
+                float xv[8];
+                unpack(raw[j], xv);
+                const float4 s0 = sm[j][0], s1 = sm[j][1];
+                v[j][0] = xv[0] * s0.x; v[j][1] = xv[1] * s0.y; v[j][2] = xv[2] * s0.z; v[j][3] = xv[3] * s0.w;
+                v[j][4] = xv[4] * s1.x; v[j][5] = xv[5] * s1.y; v[j][6] = xv[6] * s1.z; v[j][7] = xv[7] * s1.w;
+#pragma unroll
+                for(int i = 0; i < 8; i++)
+                    amax = fmaxf(amax, fabsf(v[j][i]));
+            }
+        if(m + 1 < n)
+            fetch_row(s_list[m + 1]);
+        for(int c = threadIdx.x + 256 * kQuantCache; c < chunks; c += 256)
+        {
+            float a[8], b[8];
+            unpack(*reinterpret_cast<const uint4*>(xr + c * 8), a);
+            times_sm(c, a, b);
+#pragma unroll
+            for(int i = 0; i < 8; i++)
+                amax = fmaxf(amax, fabsf(b[i]));
+        }
+        amax               = block_max_256(amax, s_red[m & 1]); // two buffers: one barrier per row suffices
+        const float ys_out = amax / qmx;
+        const float ys     = amax > 0.f ? ys_out : 1.0f; // a row of zeros: scale 0, codes 0 (not 0 / 0)
+        const int64_t r    = (int64_t)k * tokens + t;
+        if(threadIdx.x == 0)
+            yscale[r] = ys_out;
+        unsigned char* qr   = qy + r * y_stride;
+        const double ys_rcp = row_reciprocal(ys);
+        auto store = [&](int c, const float (&o)[8]) {
+            typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+            const uint2 q = quantise_8<FP8>(o, ys_rcp);
+            __builtin_nontemporal_store(u32x2_t{q.x, q.y}, reinterpret_cast<u32x2_t*>(qr + c * 8));
+        };
+#pragma unroll
+        for(int j = 0; j < kQuantCache; j++)
+            if(threadIdx.x + 256 * j < chunks)
+                store(threadIdx.x + 256 * j, v[j]);
+        for(int c = threadIdx.x + 256 * kQuantCache; c < chunks; c += 256)
+        {
+            float a[8], b[8];
+            unpack(*reinterpret_cast<const uint4*>(xr + c * 8), a);
+            times_sm(c, a, b);
+            store(c, b);
+        }
+    }
+}
+
 // Re-quantisation of the intermediate activations between the two GEMMs of the int8 path (fused_quant 1 / 2 of
 // ck_tile's fused_moe_traits; y_smooth_scale of FusedMoeGemmHostArgs, fused_moegemm_kernel.hpp:103): sorted row r
 // of Y (bf16, row-major) times the smooth scale of its expert (SMOOTH), per-row dynamic quantisation to int8:
@@ -485,7 +619,17 @@ int launch_moe_smoothquant(const mi355_moe_smoothquant_args& a, int32_t q_dtype,
                            static_cast<unsigned char*>(a.p_qy), static_cast<float*>(a.p_yscale));
     };
     const dim3 per_token((unsigned)a.tokens), per_row((unsigned)a.tokens, (unsigned)a.topk);
-    if(q_dtype == MI355_MOE_FP8)
+    // expert tables beyond 3 MB do not stay in the 4 MB L2 of an XCD: rows grouped by expert, scales in registers
+    const int64_t ranges8 = ceil_div<int64_t>(ceil_div(a.tokens, kSqRange), 8);
+    const bool grouped    = vec && (int64_t)a.experts * a.hidden_size * (int64_t)sizeof(float) > (3ll << 20) &&
+                         kSqRange * a.topk <= kSqMaxList && ranges8 * a.experts * 8 < (1ll << 31);
+    if(grouped)
+    {
+        const dim3 grid((unsigned)(ranges8 * a.experts * 8));
+        q_dtype == MI355_MOE_FP8 ? launch(moe_smoothquant_grouped_kernel<true>, grid)
+                                 : launch(moe_smoothquant_grouped_kernel<false>, grid);
+    }
+    else if(q_dtype == MI355_MOE_FP8)
         vec ? launch(moe_smoothquant_vec_kernel<true>, per_token) : launch(moe_smoothquant_kernel<true>, per_row);
     else
         vec ? launch(moe_smoothquant_vec_kernel<false>, per_token) : launch(moe_smoothquant_kernel<false>, per_row);
