@@ -120,6 +120,56 @@ def test_gate_up_then_down(T, E, K, H, I, unit, kind):
     assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
 
 
+def test_skewed_fp8_batch_takes_the_large_tiles_on_the_device():
+    """A decode-sized fp8 batch with Zipf routing: the host's average says 32-row tiles, the tile-list pass sees few
+    active experts with many rows each and builds the list for 320-row tiles (its choice is word 1 of the workspace);
+    a uniformly routed batch of the same size keeps the decode tiles.  Both against the oracle."""
+    import torch
+    import therock_amd as ta
+    from tests.gpu_util import run_sorting
+    from therock_amd import inputs as mi
+
+    T, E, K, H, I, unit = 256, 64, 4, 512, 2048, 32
+    for router, want in (("zipf", 320), ("softmax_renorm", 32)):
+        rng = np.random.default_rng(11)
+        ids, w = mi.route_np(rng.standard_normal((T, E), dtype=np.float32), K, router)
+        s_ids, s_w, s_eid, total = run_sorting(ids, w, E, unit, fill=True)
+        pp = int(total[0])
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+        x32 = rng.standard_normal((T, H)).astype(np.float32)
+        g32 = (rng.standard_normal((E, 2 * I, H)) * 0.05).astype(np.float32)
+        d32 = (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32)
+        xq, sa = oracle.rowwise_quant(x32, oracle.DT_E4M3)
+        gq, sg = oracle.rowwise_quant(g32.reshape(E * 2 * I, H), oracle.DT_E4M3)
+        dq, sd = oracle.rowwise_quant(d32.reshape(E * H, I), oracle.DT_E4M3)
+        gq, dq, sg, sd = gq.reshape(E, 2 * I, H), dq.reshape(E, H, I), sg.reshape(E, 2 * I), sd.reshape(E, H)
+        d_ids, d_w, d_eid, d_tot = dev(s_ids), dev(s_w), dev(s_eid), dev(total.astype(np.int32))
+        x, g, d = dev(xq), dev(gq), dev(dq)
+        y = torch.full((T * K, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+        ws = torch.empty((ta.moe_flatmm_get_workspace_size(ta.GEMM1_GATE_UP, x, g, y, d_ids, d_eid, d_tot, T, K, unit),),
+                         dtype=torch.uint8, device="cuda")
+        assert ta.moe_flatmm(ta.GEMM1_GATE_UP, x, g, y, d_ids, d_eid, d_tot, T, K, unit, scale_m=dev(sa), scale_n=dev(sg),
+                             workspace=ws) == 0.0
+        torch.cuda.synchronize()
+        assert int(ws.view(torch.int32)[1]) == want, router
+        y_ref = oracle.moe_gemm(1, s_ids, s_eid, s_w, pp, unit, oracle.to_f32(xq, oracle.DT_E4M3),
+                                oracle.to_f32(gq, oracle.DT_E4M3), np.zeros((T * K, I), np.uint16), T, K, sa, sg)
+        yg = y.float().cpu().numpy()
+        assert not np.isnan(yg).any() and _rel(yg, oracle.to_f32(y_ref, oracle.DT_BF16)) <= 3e-2
+        yq, sy = oracle.rowwise_quant(oracle.to_f32(y_ref, oracle.DT_BF16), oracle.DT_E4M3)
+        c = torch.zeros((T, H), dtype=torch.bfloat16, device="cuda")
+        c_ref = oracle.moe_gemm(2, s_ids, s_eid, s_w, pp, unit, oracle.to_f32(yq, oracle.DT_E4M3),
+                                oracle.to_f32(dq, oracle.DT_E4M3), _bits(c).copy(), T, K, sy, sd)
+        ws2 = torch.empty((ta.moe_flatmm_get_workspace_size(ta.GEMM2, dev(yq), d, c, d_ids, d_eid, d_tot, T, K, unit),),
+                          dtype=torch.uint8, device="cuda")
+        assert ta.moe_flatmm(ta.GEMM2, dev(yq), d, c, d_ids, d_eid, d_tot, T, K, unit, sorted_weights=d_w, scale_m=dev(sy),
+                             scale_n=dev(sd), workspace=ws2) == 0.0
+        torch.cuda.synchronize()
+        # the down GEMM has two column tiles per expert here: too few active experts to fill the chip, decode tiles
+        assert int(ws2.view(torch.int32)[1]) == 32
+        assert _rel(c.float().cpu().numpy(), oracle.to_f32(c_ref, oracle.DT_BF16)) <= 3e-2
+
+
 @pytest.mark.parametrize("T,E,K,H,I,unit", [(24, 16, 4, 512, 256, 32), (300, 8, 2, 256, 384, 32), (1024, 4, 2, 512, 384, 32)])
 @pytest.mark.parametrize("kind", ["bf16", "fp16", "int8", "fp8"])
 @pytest.mark.parametrize("act,with_bias", [("silu", True), ("swiglu", False), ("swiglu", True)])  # (silu, no bias) is the test above

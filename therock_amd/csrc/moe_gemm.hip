@@ -912,6 +912,7 @@ struct FlatmmLayout
     int64_t max_pad, ys_kb_stride;
     int32_t max_tiles;
     int mblk, hidden, inter;
+    int alt; // second tile height (32-row blocks) the tile-list pass may choose from the routing, 0: none (see alt_mblk)
     mi355_fused_moe_traits traits;
 };
 
@@ -969,6 +970,8 @@ int flatmm_layout(int kind, const mi355_moe_flatmm_args& a, FlatmmLayout& L)
                                                  "and B (32 elements for fp8)", k_eff);
         L.mblk = std::min(L.mblk, 4);
     }
+    // skewed decode-sized batches: the same choice between two tile heights as the fused entry points make
+    L.alt          = a.k_padded_zeros == 0 ? alt_mblk(L.traits, a.NumTokens, a.TopK, a.NumExperts, L.hidden, L.inter) : 0;
     L.max_pad      = (int64_t)a.TopK * a.NumTokens + (int64_t)a.NumExperts * a.block_m - a.TopK;
     L.max_tiles    = (int32_t)(a.NumExperts + L.max_pad / (L.mblk * 32) + 1);
     L.total        = 0;
@@ -1033,8 +1036,10 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     int* inv           = reinterpret_cast<int*>(wsb + L.inv_off);
     const int mblk     = L.mblk;
     const int prec     = L.traits.prec_i;
-    if((g1 ? T : (int64_t)T * K) * a.stride_A * a_b >= ((int64_t)1 << 32) && mblk > 4)
+    if((g1 ? T : (int64_t)T * K) * a.stride_A * a_b >= ((int64_t)1 << 32) && (mblk > 4 || L.alt != 0))
         return fail(MI355_MOE_E_UNSUPPORTED, "moe_flatmm: A of 4 GiB or more is not supported at this problem size");
+    const int alt           = L.alt;
+    const int alt_max_tiles = alt ? (int)std::min<int64_t>(L.max_tiles, E + L.max_pad / (alt * 32) + 1) : 0;
     {
         KernelTimer timer(MI355_MOE_K_PREP, stream);
         const int n_inv     = T * K;
@@ -1042,7 +1047,8 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
         hipLaunchKernelGGL(moe_prep_kernel, dim3(prep_grid), dim3(kPrepBlock), 0, stream,
                            static_cast<const int*>(a.p_sorted_expert_ids), static_cast<const int*>(a.p_max_token_id),
                            a.block_m, E, mblk * 32, (int)ceil_div<int64_t>(L.max_pad, a.block_m), L.max_tiles, tile_map,
-                           inv, n_inv, 0, 0, 0);
+                           inv, n_inv, alt * 32, kAltMinRows,
+                           ceil_div(device_info().num_cu, ceil_div(a.N, 256))); // enough tiles of this GEMM to fill the chip
         if(!g1)
             hipLaunchKernelGGL(moe_inv_kernel, dim3(std::min<int>(ceil_div<int64_t>(L.max_pad, 256), 1024)), dim3(256), 0,
                                stream, static_cast<const int*>(a.p_sorted_token_ids),
@@ -1055,6 +1061,7 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
     p.tile_map       = tile_map;
     p.tokens         = T;
     p.slot_rows      = K;
+    p.tile_rows      = alt ? mblk * 32 : 0;
     p.act            = a.activation == MI355_MOE_ACT_SWIGLU ? 2 : 1; // MoeSilu (ck_tile's default FusedActivation) or Swiglu
     p.swiglu_alpha   = a.swiglu_alpha;
     p.swiglu_limit   = a.swiglu_limit;
@@ -1080,7 +1087,15 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
         p.gate_only     = go;
         p.n_out         = I;
         p.n_total       = a.N;
-        return launch_grouped_gemm(prec, true, mblk, decode, p, L.max_tiles, stream);
+        KernelTimerGroup both(MI355_MOE_K_GEMM0, stream, alt != 0);
+        rc = launch_grouped_gemm(prec, true, mblk, decode, p, L.max_tiles, stream);
+        if(rc == MI355_MOE_OK && alt)
+        {
+            GemmParams pa = p;
+            pa.tile_rows  = alt * 32;
+            rc            = launch_grouped_gemm(prec, true, alt, false, pa, alt_max_tiles, stream);
+        }
+        return rc;
     }
     p.out           = wsb + L.p_off;
     p.out_row_bytes = (int64_t)H * 2;
@@ -1094,7 +1109,16 @@ int launch_moe_flatmm(int kind, const mi355_moe_flatmm_args& a, void* ws_ptr, si
         hipLaunchKernelGGL(fill_u32x4_kernel, dim3((unsigned)std::min<int64_t>(ceil_div<int64_t>(n16, 256), 4096)), dim3(256), 0,
                            stream, reinterpret_cast<uint4*>(p.y_scale), n16, 0x7f7f7f7fu);
     }
-    rc = launch_grouped_gemm(prec, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p, L.max_tiles, stream);
+    {
+        KernelTimerGroup both(MI355_MOE_K_GEMM1, stream, alt != 0);
+        rc = launch_grouped_gemm(prec, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p, L.max_tiles, stream);
+        if(rc == MI355_MOE_OK && alt)
+        {
+            GemmParams pa = p;
+            pa.tile_rows  = alt * 32;
+            rc            = launch_grouped_gemm(prec, false, alt, false, pa, alt_max_tiles, stream);
+        }
+    }
     if(rc != MI355_MOE_OK)
         return rc;
     {
