@@ -168,6 +168,74 @@ def roofline_of(cfg, res, gemm=0):
             "algorithmic_flop": flop, "mfma_TFLOPs": tflops, "mfma_frac": tflops / PEAK_MFMA[cfg.dtype]}
 
 
+def _smi_sample():
+    """One reading of the package power (W) and the shader clock (MHz) from amd-smi; None where it cannot be had."""
+    import re
+    import subprocess
+
+    try:
+        out = subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=20).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    pw = re.search(r"SOCKET_POWER:\s*([0-9.]+)\s*W", out)
+    ck = re.search(r"GFX_0:\s*\n\s*CLK:\s*([0-9.]+)\s*MHz", out)
+    if not pw:
+        return None
+    return float(pw.group(1)), (float(ck.group(1)) if ck else None)
+
+
+def _power_cap():
+    import re
+    import subprocess
+
+    try:
+        out = subprocess.run(["rocm-smi", "--showmaxpower"], capture_output=True, text=True, timeout=20).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    m = re.search(r"Max Graphics Package Power \(W\):\s*([0-9.]+)", out)
+    return float(m.group(1)) if m else None
+
+
+def run_power_probe(cfg, samples=3):
+    """Package power and shader clock while the headline path runs back to back: passes are queued a few hundred at a
+    time and amd-smi is read while the queue drains.  Outside the timed region; None when amd-smi gives no reading."""
+    import torch
+
+    import therock_amd as ta
+    from therock_amd import inputs as mi
+
+    if _smi_sample() is None:
+        return None
+    dev = torch.device("cuda:0")
+    inp = mi.make_inputs_torch(cfg, dev, 0)
+    traits = ta.fused_moe_traits(prec_i=cfg.dtype, prec_w=cfg.dtype, block_m=cfg.unit)
+    buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, dev)
+    args = ta.make_args(traits, buf, inp["a"], inp["g"], inp["d"], inp["topk_ids"], inp["topk_weight"],
+                        a_scale=inp["a_scale"], g_scale=inp["g_scale"], d_scale=inp["d_scale"])
+    t0 = time.perf_counter()
+    for _ in range(20):
+        ta.fused_moe(traits, args)
+    torch.cuda.synchronize()
+    per_pass = (time.perf_counter() - t0) / 20
+    chunk = max(10, int(1.2 / per_pass))  # about 1.2 s of queued work per reading
+    watts, clocks = [], []
+    for _ in range(samples):
+        for _ in range(chunk):
+            ta.fused_moe(traits, args)
+        time.sleep(0.25)  # the power controller needs a moment to settle
+        r = _smi_sample()
+        torch.cuda.synchronize()
+        if r:
+            watts.append(r[0])
+            if r[1]:
+                clocks.append(r[1])
+    if not watts:
+        return None
+    return {"socket_power_w": sum(watts) / len(watts), "power_cap_w": _power_cap(),
+            "gfx_clock_mhz": sum(clocks) / len(clocks) if clocks else None, "samples": len(watts),
+            "what": f"amd-smi while {cfg.name} passes run back to back"}
+
+
 def run_sustained(dtype):
     """The matrix-core rate this device sustains for the workload's MFMA instruction on register operands, with no
     memory traffic at all: with operands that toggle like real data (the ceiling of any kernel on this box, set by
@@ -357,7 +425,7 @@ def _workload_short(r):
     return {"ms": _r(r["ms_per_step"]), "rate": _r(r["hbm_GBps"]), "unit": "GB/s", "frac": _r(r["frac_hbm_peak"], 3)}
 
 
-def build_line(cfg, steps, warmup, res, roof, roof1, cpu, router, neighbours, workloads, sustained=None):
+def build_line(cfg, steps, warmup, res, roof, roof1, cpu, router, neighbours, workloads, sustained=None, power=None):
     """The one JSON line of the result: headline fields, the two roofline entries, the CPU baseline and one short
     record per other workload.  Kept under MAX_LINE_BYTES: readers that keep only the tail of stdout must still
     see a whole line."""
@@ -381,6 +449,9 @@ def build_line(cfg, steps, warmup, res, roof, roof1, cpu, router, neighbours, wo
         line["mfma_sustained"] = {"random_operands": _r(sustained["random_operands"], 5),
                                   "zero_operands": _r(sustained["zero_operands"], 5), "unit": sustained["unit"],
                                   "frac_of_sustained": _r(res["tflops"] / sustained["random_operands"])}
+    if power:
+        line["power"] = {"socket_power_w": _r(power["socket_power_w"]), "power_cap_w": power.get("power_cap_w"),
+                         "gfx_clock_mhz": _r(power.get("gfx_clock_mhz"))}
     if router and "avg_launch_ms" in router:
         line["router_ms"] = _r(router["avg_launch_ms"])
     if neighbours and "error" not in neighbours:
@@ -452,6 +523,14 @@ def main():
                     r["frac_of_sustained"] = r["achieved"] / sustained["random_operands"]
         except Exception as e:
             log(f"[bench] sustained MFMA rate failed: {e!r}")
+    power = None
+    if not a.no_sustained:
+        try:
+            power = run_power_probe(cfg)
+            log(f"[bench] power while the path runs: {power}")
+            torch.cuda.empty_cache()
+        except Exception as e:
+            log(f"[bench] power probe failed: {e!r}")
     cpu = None
     if not a.no_cpu_baseline:
         try:
@@ -538,7 +617,7 @@ def main():
     if sustained and roof1 and roof1["bound"] == "mfma":
         roof1["sustained_peak"] = sustained["random_operands"]
         roof1["frac_of_sustained"] = roof1["achieved"] / sustained["random_operands"]
-    line = build_line(cfg, a.steps, a.warmup, res, roof, roof1, cpu, router, neighbours, {**others, **extra}, sustained)
+    line = build_line(cfg, a.steps, a.warmup, res, roof, roof1, cpu, router, neighbours, {**others, **extra}, sustained, power)
     print(json.dumps(line, separators=(",", ":")), flush=True)
 
 
