@@ -171,11 +171,13 @@ typedef struct mi355_fused_moe_traits
     int32_t activation;  /* 0 = gelu (erf form, ck_tile::element_wise::Gelu), 1 = silu */
     int32_t gate_only;   /* 0 = gate and up (g [e, 2*inter, hidden]), 1 = gate only (g [e, inter, hidden], y = act(gate)) */
     int32_t fused_quant; /* 0 = none (quantised dtypes always take a_scale/g_scale/d_scale; the int8 path keeps the
-                            intermediate activations in bf16).  INT8 only: 2 = dynamic-quant, the intermediate
-                            activations are re-quantised to int8 per row between the GEMMs and the down GEMM runs on
-                            int8 MFMAs; 1 = smooth-dynamic-quant, the same after a multiplication by
-                            y_smooth_scale[expert], and the activations arrive as MoeSmoothquant leaves them: one int8
-                            row per (slot, token), a [topk, tokens, stride_token], a_scale [topk, tokens]
+                            intermediate activations in bf16, the fp8 path rounds them to e4m3 with a power-of-two
+                            scale per 32 columns inside the gate+up GEMM).  INT8 and FP8: 2 = dynamic-quant, the
+                            intermediate activations are re-quantised to int8 (e4m3) with one fp32 scale per row in a
+                            pass between the GEMMs and the down GEMM runs on int8 (fp8) MFMAs; 1 =
+                            smooth-dynamic-quant, the same after a multiplication by y_smooth_scale[expert], and the
+                            activations arrive as MoeSmoothquant leaves them: one quantised row per (slot, token),
+                            a [topk, tokens, stride_token], a_scale [topk, tokens]
                             (UseSmoothQuant of fused_moegemm_traits.hpp:19-35; layouts moe_sorting_kernel.hpp:82-83) */
     int32_t local_expert_masking; /* 1 = apply local_expert_mask_ptr in the sort */
     int32_t weight_permute; /* layout of g and d, FusedMoeGemmWeightPermuteEnum (fused_moegemm_traits.hpp:10-17; a

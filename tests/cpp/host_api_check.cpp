@@ -136,6 +136,48 @@ int main()
     std::vector<uint16_t> o2(T * H);
     HIP_OK(hipMemcpy(o2.data(), args2.o_ptr, o2.size() * 2, hipMemcpyDeviceToHost));
     if(std::memcmp(o.data(), o2.data(), o.size() * 2) != 0) { std::fprintf(stderr, "pre-shuffled weights give other bits\n"); return 6; }
+    // moe_sorting() with the example's trait: experts without tokens keep a unit of padding (expert E - 1 gets no token
+    // here), once per dispatch policy; sizes as reference_moe_sorting lays them out without the skip
+    {
+        std::vector<int32_t> ids2(ids);
+        for(auto& v : ids2) v = v % (E - 1);
+        for(int t = 0; t < T; t++)
+            if(ids2[t * K + 1] == ids2[t * K]) ids2[t * K + 1] = (ids2[t * K] + 1) % (E - 1);
+        const int cells = T * K + E * U, units = cells / U + 1;
+        std::vector<int32_t> r_ids(cells, -1), r_eid(units, -1);
+        std::vector<float> r_w(cells, -1.f);
+        int32_t r_pp = 0;
+        moe_oracle_sorting(ids2.data(), w.data(), nullptr, T, K, E, U, /*skip_empty=*/0, r_ids.data(), r_w.data(), r_eid.data(), &r_pp);
+        for(int policy = 0; policy < 3; policy++)
+        {
+            mi355::moe_sorting_trait st;
+            st.dispatch_policy = policy;
+            st.skip_experts_with_zero_tokens = false;
+            mi355::moe_sorting_args sa{};
+            std::vector<int32_t> q_ids(cells, -1), q_eid(units, -1), q_tot(2, 0);
+            std::vector<float> q_w(cells, -1.f);
+            sa.p_topk_ids = to_device(ids2);
+            sa.p_weights = to_device(w);
+            sa.p_sorted_token_ids = to_device(q_ids);
+            sa.p_sorted_weights = to_device(q_w);
+            sa.p_sorted_expert_ids = to_device(q_eid);
+            sa.p_total_tokens_post_pad = to_device(q_tot);
+            const int ws_bytes = mi355::moe_sorting_get_workspace_size(T, E, K, policy);
+            if((ws_bytes == 0) != (policy != 2)) { std::fprintf(stderr, "workspace size %d with policy %d\n", ws_bytes, policy); return 7; }
+            void* ws = nullptr;
+            if(ws_bytes > 0) HIP_OK(hipMalloc(&ws, ws_bytes));
+            sa.p_ws = ws;
+            sa.tokens = T; sa.unit_size = U; sa.num_experts = E; sa.topk = K;
+            if(mi355::moe_sorting(st, sa) != 0.f) { std::fprintf(stderr, "moe_sorting failed\n"); return 7; }
+            HIP_OK(hipDeviceSynchronize());
+            HIP_OK(hipMemcpy(q_ids.data(), sa.p_sorted_token_ids, q_ids.size() * 4, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(q_eid.data(), sa.p_sorted_expert_ids, q_eid.size() * 4, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(q_tot.data(), sa.p_total_tokens_post_pad, 8, hipMemcpyDeviceToHost));
+            if(q_tot[0] != r_pp || std::memcmp(q_ids.data(), r_ids.data(), sizeof(int32_t) * r_pp) != 0 ||
+               std::memcmp(q_eid.data(), r_eid.data(), sizeof(int32_t) * (r_pp / U)) != 0 || q_eid[r_pp / U - 1] != E - 1)
+            { std::fprintf(stderr, "moe_sorting without the empty-expert skip differs from the oracle (policy %d)\n", policy); return 8; }
+        }
+    }
     // unsupported traits report -1 like CK's dispatcher; timing returns milliseconds
     mi355::fused_moe_traits bad = traits; bad.prec_i = "fp16"; bad.prec_w = "fp16";
     const float unsupported = mi355::fused_moe(bad, args);

@@ -182,8 +182,8 @@ def test_host_only_entry_points():
         for wp, ok in ((0, 1), (1, 1), (2, 0), (-1, 0)):
             t = _lib.FusedMoeTraits(prec, prec, 0, 3, 3, 3, 3, 32, 1, 0, 0, 0, wp)
             assert lib.mi355_fused_moe_supported(C.byref(t)) == ok
-    # fused_quant 1 / 2 (re-quantised intermediate activations) exist for int8 only and need a larger workspace
-    for prec, fq, ok in ((2, 1, 1), (2, 2, 1), (2, 3, 0), (0, 2, 0), (1, 1, 0)):
+    # fused_quant 1 / 2 (re-quantised intermediate activations) exist for int8 and fp8 and need a larger workspace
+    for prec, fq, ok in ((2, 1, 1), (2, 2, 1), (2, 3, 0), (0, 2, 0), (1, 1, 1), (1, 2, 1), (5, 2, 0)):
         t = _lib.FusedMoeTraits(prec, prec, 0, 3, 3, 3, 3, 32, 1, 0, fq, 0)
         assert lib.mi355_fused_moe_supported(C.byref(t)) == ok
     w0, w2 = (lib.mi355_fused_moe_workspace_size(C.byref(_lib.FusedMoeTraits(2, 2, 0, 3, 3, 3, 3, 32, 1, 0, fq, 0)),

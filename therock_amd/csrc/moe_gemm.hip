@@ -388,7 +388,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
                                                            int64_t out_row_bytes, int accumulate,
                                                            const float* __restrict__ slot_scale,
                                                            const float* __restrict__ bias,
-                                                           const int* __restrict__ sorted_eid, int unit, int f16)
+                                                           const int* __restrict__ sorted_eid, int unit, int f16,
+                                                           const float* __restrict__ row_scale = nullptr)
 {
     // f16: the partial rows and the output are fp16 instead of bf16 (a uniform branch)
     const int t  = blockIdx.x;
@@ -428,6 +429,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
                 w[j] = sorted_w[pos[j]];
                 if(slot_scale) // per-row scale of the stand-alone down GEMM's quantised input, row = token * topk + slot
                     w[j] *= slot_scale[t * topk + k0 + j];
+                if(row_scale) // per-row scale of re-quantised e4m3 intermediate activations, in sorted-row order
+                    w[j] *= row_scale[pos[j]];
                 v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(part + ((int64_t)pos[j] * hidden + h0) * 2));
             }
         }
@@ -627,9 +630,10 @@ int check_traits(const mi355_fused_moe_traits& t)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: activation=%d (0 = gelu, 1 = silu)", t.activation);
     if(t.gate_only != 0 && t.gate_only != 1)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: gate_only=%d (0 or 1)", t.gate_only);
-    if(t.fused_quant < 0 || t.fused_quant > 2 || (t.fused_quant != 0 && t.prec_i != MI355_MOE_INT8))
+    if(t.fused_quant < 0 || t.fused_quant > 2 ||
+       (t.fused_quant != 0 && t.prec_i != MI355_MOE_INT8 && t.prec_i != MI355_MOE_FP8))
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: fused_quant=%d with precision %d (1 = smooth-dynamic-quant and "
-                                             "2 = dynamic-quant of the intermediate activations exist for int8)",
+                                             "2 = dynamic-quant of the intermediate activations exist for int8 and fp8)",
                     t.fused_quant, t.prec_i);
     if(t.block_m < 1 || t.block_m > 1024)
         return fail(MI355_MOE_E_UNSUPPORTED, "fused_moe: block_m=%d", t.block_m);
@@ -663,10 +667,10 @@ WorkspaceLayout workspace_layout(const mi355_fused_moe_traits& t, int32_t tokens
     const int mblk   = pick_mblk(t, tokens, topk, experts, hidden, inter);
     w.max_pad        = (int64_t)topk * tokens + (int64_t)experts * t.block_m - topk;
     w.max_tiles      = (int32_t)(experts + w.max_pad / (mblk * 32) + 1);
-    // gemm0 writes e4m3 on the fp8 path and bf16 otherwise; with fused_quant the int8 path re-quantises that bf16
-    // Y into a second buffer the down GEMM reads
-    const bool requant = t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0;
-    const int y_b      = t.prec_i == MI355_MOE_FP8 ? 1 : 2;
+    // gemm0 writes e4m3 on the fp8 path (bf16 with fused_quant) and bf16 otherwise; with fused_quant the int8 and fp8
+    // paths re-quantise that bf16 Y, one scale per row, into a second buffer the down GEMM reads
+    const bool requant = (t.prec_i == MI355_MOE_INT8 || t.prec_i == MI355_MOE_FP8) && t.fused_quant != 0;
+    const int y_b      = (t.prec_i == MI355_MOE_FP8 && !requant) ? 1 : 2;
     w.sort_off       = bump(sorting_workspace_bytes(tokens, experts, topk));
     w.map_off        = bump(sizeof(int) * (kMapHdr + (size_t)kMapEnt * w.max_tiles));
     w.inv_off        = bump(sizeof(int) * (size_t)tokens * topk);
@@ -803,8 +807,10 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     p.w_permuted = t.weight_permute;
 
     // ---- gemm0: gate+up, SiLU*up
-    const bool requant = t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0;
-    const int y_b      = t.prec_i == MI355_MOE_FP8 ? 1 : 2; // bytes per element of what gemm0 writes
+    const bool requant  = quant && t.fused_quant != 0;
+    const bool requant8 = requant && t.prec_i == MI355_MOE_FP8; // e4m3 rows with one scale each instead of one per 32 columns
+    const int y_b       = (t.prec_i == MI355_MOE_FP8 && !requant) ? 1 : 2; // bytes per element of what gemm0 writes
+    p.y_bf16            = requant8 ? 1 : 0;
     p.x_slot_major     = t.fused_quant == 1 ? 1 : 0;
     p.x               = static_cast<const unsigned char*>(a.a_ptr);
     p.x_row_bytes     = (int64_t)a.stride_token * eb;
@@ -847,21 +853,29 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
         }
     }
     p.x_slot_major = 0;
+    p.y_bf16       = 0;
     if(requant)
     {
         rc = launch_requant_y(wsb + ws.y_off, I, static_cast<const float*>(a.y_smooth_scale_ptr), p.sorted_ids,
                               static_cast<const int*>(a.sorted_expert_ids_ptr),
                               static_cast<const int*>(a.num_sorted_tiles_ptr), t.block_m, T, y_slab, ws.max_pad,
-                              wsb + ws.yq_off, reinterpret_cast<float*>(wsb + ws.yrs_off), stream);
+                              wsb + ws.yq_off, reinterpret_cast<float*>(wsb + ws.yrs_off), stream, requant8);
         if(rc != MI355_MOE_OK)
             return rc;
+        if(requant8)
+        {
+            // the down GEMM runs the block-scaled MFMA: every block scale is 2^0, the row scales go into the combine
+            const int64_t n16 = (ws.ys_kb_stride * (I / 32) + 15) / 16; // the buffer is a multiple of 256 bytes
+            hipLaunchKernelGGL(fill_u32x4_kernel, dim3((unsigned)std::min<int64_t>(ceil_div<int64_t>(n16, 256), 4096)),
+                               dim3(256), 0, stream, reinterpret_cast<uint4*>(wsb + ws.ys_off), n16, 0x7f7f7f7fu);
+        }
     }
 
     // ---- gemm1: down, * top-k weight, bf16 partial per (token, slot)
     p.y_slab         = y_slab;
     p.x              = requant ? wsb + ws.yq_off : wsb + ws.y_off;
     p.x_row_bytes    = (int64_t)I * yq_b;
-    p.x_scale        = requant ? reinterpret_cast<const float*>(wsb + ws.yrs_off) : nullptr;
+    p.x_scale        = requant && !requant8 ? reinterpret_cast<const float*>(wsb + ws.yrs_off) : nullptr;
     p.gate_only      = 0;
     p.w              = static_cast<const unsigned char*>(a.d_ptr);
     p.w_row_bytes    = (int64_t)I * eb;
@@ -876,7 +890,7 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     {
         KernelTimerGroup both(MI355_MOE_K_GEMM1, stream, alt != 0);
         rc = launch_grouped_gemm(t.prec_i, false, mblk, decode && down_gemm_wants_decode(E, (int64_t)T * K, H), p,
-                                 ws.max_tiles, stream, requant);
+                                 ws.max_tiles, stream, requant && !requant8);
         if(rc != MI355_MOE_OK)
             return rc;
         if(alt)
@@ -896,7 +910,8 @@ int launch_fused_moegemm(const mi355_fused_moe_traits& t, const mi355_fused_moeg
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T, ceil_div(H, 256 * 8)), dim3(256), 0, stream, wsb + ws.p_off, inv,
                        static_cast<const float*>(a.sorted_weight_ptr), static_cast<unsigned char*>(a.o_ptr), K, H,
                        (int64_t)a.stride_token * 2, 0, static_cast<const float*>(nullptr), static_cast<const float*>(nullptr),
-                       static_cast<const int*>(nullptr), 1, t.prec_i == MI355_MOE_FP16 ? 1 : 0);
+                       static_cast<const int*>(nullptr), 1, t.prec_i == MI355_MOE_FP16 ? 1 : 0,
+                       requant8 ? reinterpret_cast<const float*>(wsb + ws.yrs_off) : static_cast<const float*>(nullptr));
     }
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;

@@ -76,7 +76,7 @@ int launch_moe_smoothquant(const mi355_moe_smoothquant_args& a, int32_t q_dtype,
 // total[0] = rows of the sorted prefix; segs > 0: slab-major output)
 int launch_requant_y(const void* y, int32_t inter, const float* smooth, const int* sorted_ids, const int* sorted_expert_ids,
                      const int* total, int32_t unit, int32_t tokens, int32_t segs, int64_t max_rows, void* yq, float* yscale,
-                     hipStream_t stream);
+                     hipStream_t stream, bool fp8 = false);
 
 int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stride_x, int32_t q_dtype,
                          void* q, void* scale, hipStream_t stream);

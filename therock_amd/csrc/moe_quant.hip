@@ -445,7 +445,9 @@ __global__ __launch_bounds__(256) void moe_smoothquant_grouped_kernel(const uint
 // input.  One wave per row; a row of up to 2048 columns is read once.
 // Output row-major, or slab-major when segs > 0 (y_slab_offset); padding rows become zeros with scale 0, rows past
 // the sorted prefix are left alone.
-template <bool SMOOTH>
+// FP8 (the fp8 path with fused_quant): e4m3 codes instead, scale = amax / 448, rounded to nearest even by the
+// conversion instruction.
+template <bool SMOOTH, bool FP8>
 __global__ __launch_bounds__(256) void moe_requant_y_kernel(const uint16_t* __restrict__ y, int inter,
                                                              const float* __restrict__ smooth,
                                                              const int* __restrict__ sorted_ids,
@@ -514,17 +516,22 @@ __global__ __launch_bounds__(256) void moe_requant_y_kernel(const uint16_t* __re
 #pragma unroll
     for(int d = 32; d > 0; d >>= 1)
         amax = fmaxf(amax, __shfl_xor(amax, d));
-    const float ys_out = amax / 127.0f;
+    const float ys_out = amax / (FP8 ? 448.0f : 127.0f);
     const float ys     = amax > 0.f ? ys_out : 1.0f; // a row of zeros: scale 0, codes 0
     if(lane == 0)
         yscale[row] = ys_out;
     const double ys_rcp = row_reciprocal(ys);
     auto store = [&](int c, const float (&o)[8]) {
-        uint32_t w[2] = {0u, 0u};
+        if constexpr(FP8)
+            *reinterpret_cast<uint2*>(dst(c)) = quantise_8<true>(o, ys_rcp);
+        else
+        {
+            uint32_t w[2] = {0u, 0u};
 #pragma unroll
-        for(int i = 0; i < 8; i++)
-            w[i >> 2] |= (static_cast<uint32_t>(static_cast<int>(__builtin_rintf(div_by_row_scale(o[i], ys_rcp)))) & 0xffu) << (8 * (i & 3));
-        *reinterpret_cast<uint2*>(dst(c)) = make_uint2(w[0], w[1]);
+            for(int i = 0; i < 8; i++)
+                w[i >> 2] |= (static_cast<uint32_t>(static_cast<int>(__builtin_rintf(div_by_row_scale(o[i], ys_rcp)))) & 0xffu) << (8 * (i & 3));
+            *reinterpret_cast<uint2*>(dst(c)) = make_uint2(w[0], w[1]);
+        }
     };
 #pragma unroll
     for(int j = 0; j < kQuantCache; j++)
@@ -665,7 +672,7 @@ int launch_rowwise_quant(const void* x, int64_t rows, int32_t cols, int64_t stri
 
 int launch_requant_y(const void* y, int32_t inter, const float* smooth, const int* sorted_ids, const int* sorted_expert_ids,
                      const int* total, int32_t unit, int32_t tokens, int32_t segs, int64_t max_rows, void* yq, float* yscale,
-                     hipStream_t stream)
+                     hipStream_t stream, bool fp8)
 {
     if(max_rows <= 0)
         return MI355_MOE_OK;
@@ -675,7 +682,10 @@ int launch_requant_y(const void* y, int32_t inter, const float* smooth, const in
         hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(y), inter, smooth, sorted_ids,
                            sorted_expert_ids, total, unit, tokens, segs, static_cast<unsigned char*>(yq), yscale);
     };
-    smooth != nullptr ? launch(moe_requant_y_kernel<true>) : launch(moe_requant_y_kernel<false>);
+    if(fp8)
+        smooth != nullptr ? launch(moe_requant_y_kernel<true, true>) : launch(moe_requant_y_kernel<false, true>);
+    else
+        smooth != nullptr ? launch(moe_requant_y_kernel<true, false>) : launch(moe_requant_y_kernel<false, false>);
     MI355_HIP_TRY(hipGetLastError());
     return MI355_MOE_OK;
 }
