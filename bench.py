@@ -170,15 +170,22 @@ def roofline_of(cfg, res, gemm=0):
 
 def _smi_sample():
     """One reading of the package power (W) and the shader clock (MHz) from amd-smi; None where it cannot be had."""
-    import re
     import subprocess
 
     try:
         out = subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=20).stdout
     except (OSError, subprocess.SubprocessError):
         return None
-    pw = re.search(r"SOCKET_POWER:\s*([0-9.]+)\s*W", out)
-    ck = re.search(r"GFX_0:\s*\n\s*CLK:\s*([0-9.]+)\s*MHz", out)
+    return parse_smi(out)
+
+
+def parse_smi(text):
+    """(socket power in W, clock of the first shader engine in MHz or None) from `amd-smi metric -p -c`; None without
+    a power reading."""
+    import re
+
+    pw = re.search(r"SOCKET_POWER:\s*([0-9.]+)\s*W", text)
+    ck = re.search(r"GFX_0:\s*\n\s*CLK:\s*([0-9.]+)\s*MHz", text)
     if not pw:
         return None
     return float(pw.group(1)), (float(ck.group(1)) if ck else None)

@@ -60,3 +60,28 @@ def test_line_sheds_optional_parts_before_it_outgrows_the_limit():
     text = json.dumps(line, separators=(",", ":"))
     assert len(text) < bench.MAX_LINE_BYTES
     assert "workloads" not in line and line["roofline"] and line["cpu_baseline"]
+
+
+def test_power_reading_is_parsed_and_reported():
+    text = """GPU: 0
+    POWER:
+        SOCKET_POWER: 1395 W
+        GFX_VOLTAGE: N/A
+    CLOCK:
+        GFX_0:
+            CLK: 1921 MHz
+            MIN_CLK: 500 MHz
+        GFX_1:
+            CLK: 1874 MHz
+"""
+    assert bench.parse_smi(text) == (1395.0, 1921.0)
+    assert bench.parse_smi("ERROR:root:Unable to get devices") is None
+    assert bench.parse_smi("        SOCKET_POWER: 640 W\n") == (640.0, None)
+    cfg = mi.CONFIGS[bench.HEADLINE]
+    res = _stub_result(cfg, 3.3)
+    line = bench.build_line(cfg, 20, 3, res, bench.roofline_of(cfg, res), bench.roofline_of(cfg, res, 1), None, None, None, {},
+                            {"random_operands": 3912.4, "zero_operands": 4948.1, "unit": "TFLOP/s"},
+                            {"socket_power_w": 1389.7, "power_cap_w": 1400.0, "gfx_clock_mhz": 1905.3})
+    assert line["power"] == {"socket_power_w": 1390.0, "power_cap_w": 1400.0, "gfx_clock_mhz": 1905.0}
+    assert abs(line["mfma_sustained"]["frac_of_sustained"] - res["tflops"] / 3912.4) < 1e-3
+    assert len(json.dumps(line, separators=(",", ":"))) < bench.MAX_LINE_BYTES
