@@ -204,8 +204,8 @@ def _power_cap():
 
 
 def run_power_probe(cfg, samples=3):
-    """Package power and shader clock while the headline path runs back to back: passes are queued a few hundred at a
-    time and amd-smi is read while the queue drains.  Outside the timed region; None when amd-smi gives no reading."""
+    """Package power and shader clock while the headline path runs back to back.  Outside the timed region; None when
+    amd-smi gives no reading."""
     import torch
 
     import therock_amd as ta
@@ -219,19 +219,30 @@ def run_power_probe(cfg, samples=3):
     buf = ta.MoeBuffers(traits, cfg.tokens, cfg.experts, cfg.topk, cfg.hidden, cfg.inter, dev)
     args = ta.make_args(traits, buf, inp["a"], inp["g"], inp["d"], inp["topk_ids"], inp["topk_weight"],
                         a_scale=inp["a_scale"], g_scale=inp["g_scale"], d_scale=inp["d_scale"])
-    t0 = time.perf_counter()
-    for _ in range(20):
-        ta.fused_moe(traits, args)
+    # The readings are taken by a child process that is started while the device is idle and then runs amd-smi a few
+    # times on its own; this process meanwhile does nothing but queue passes.  (It must not start a process while it
+    # is submitting work: a fork makes the pages of the submitting process copy-on-write, and a launch that writes
+    # its kernel arguments into such a page while the child still exists moves the page away from under the GPU.)
+    import subprocess
+
     torch.cuda.synchronize()
-    per_pass = (time.perf_counter() - t0) / 20
-    chunk = max(10, int(1.2 / per_pass))  # about 1.2 s of queued work per reading
-    watts, clocks = [], []
-    for _ in range(samples):
-        for _ in range(chunk):
+    script = f"sleep 1.5; for i in $(seq {samples}); do amd-smi metric -p -c; echo ====; sleep 0.3; done"
+    try:
+        child = subprocess.Popen(["bash", "-c", script], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)
+    except OSError:
+        return None
+    deadline = time.perf_counter() + 30.0
+    while child.poll() is None and time.perf_counter() < deadline:
+        for _ in range(8):
             ta.fused_moe(traits, args)
-        time.sleep(0.25)  # the power controller needs a moment to settle
-        r = _smi_sample()
         torch.cuda.synchronize()
+    torch.cuda.synchronize()
+    if child.poll() is None:
+        child.kill()
+    out = child.communicate()[0]
+    watts, clocks = [], []
+    for part in out.split("===="):
+        r = parse_smi(part)
         if r:
             watts.append(r[0])
             if r[1]:
