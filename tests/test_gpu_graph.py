@@ -17,7 +17,10 @@ pytestmark = pytest.mark.gpu
     ("cfg4_decode_int8_t64", dict(tokens=160, hidden=1024, inter=512, experts=32), 0),
     # with the re-quantisation pass between the GEMMs (decode kernel / large-tile kernel)
     ("cfg4_decode_int8_t64", dict(hidden=1024, inter=512), 2),
-    ("cfg4_decode_int8_t64", dict(tokens=2048, hidden=512, inter=256, experts=8), 2)])
+    ("cfg4_decode_int8_t64", dict(tokens=2048, hidden=512, inter=256, experts=8), 2),
+    # fp8 with re-quantised rows: the pass between the GEMMs, the fill of the unit block scales, row scales in the combine
+    ("cfg3_dsv3_fp8", dict(tokens=64, hidden=512, inter=256, experts=16, topk=4), 2),
+    ("cfg3_dsv3_fp8", dict(tokens=2048, hidden=512, inter=256, experts=8), 2)])
 def test_capture_and_replay(name, scale, fused_quant):
     import torch
 
