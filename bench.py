@@ -226,7 +226,7 @@ def run_power_probe(cfg, samples=3):
     import subprocess
 
     torch.cuda.synchronize()
-    script = f"sleep 1.5; for i in $(seq {samples}); do amd-smi metric -p -c; echo ====; sleep 0.3; done"
+    script = f"sleep 1.5; for i in $(seq {samples}); do timeout -k 2 8 amd-smi metric -p -c; echo ====; sleep 0.3; done"
     try:
         child = subprocess.Popen(["bash", "-c", script], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)
     except OSError:
@@ -239,7 +239,10 @@ def run_power_probe(cfg, samples=3):
     torch.cuda.synchronize()
     if child.poll() is None:
         child.kill()
-    out = child.communicate()[0]
+    try:
+        out = child.communicate(timeout=15)[0]
+    except subprocess.TimeoutExpired:
+        return None
     watts, clocks = [], []
     for part in out.split("===="):
         r = parse_smi(part)
