@@ -71,6 +71,8 @@ def test_random_shapes_masks_and_local_tokens(seed):
 
 def test_empty_and_skew():
     check(np.zeros((0, 2), np.int32), np.zeros((0, 2), np.float32), 8, 32)
+    # an empty batch whose output arrays have no cell at all (max_num_tokens_padded = 0): only the totals are written
+    check(np.zeros((0, 1), np.int32), np.zeros((0, 1), np.float32), 1, 1)
     # every token picks the same experts: one giant bucket, the rest empty
     T = 20000
     ids = np.tile(np.array([[5, 2]], dtype=np.int32), (T, 1))

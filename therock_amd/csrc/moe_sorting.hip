@@ -515,8 +515,11 @@ int launch_moe_sorting(const mi355_moe_sorting_args& a, hipStream_t stream, cons
 {
     if(dispatch_policy < 0 || dispatch_policy > 2)
         return fail(MI355_MOE_E_INVALID, "moe_sorting: dispatch_policy=%d outside [0, 2]", dispatch_policy);
-    if((a.tokens > 0 && (!a.p_topk_ids || !a.p_weights)) || !a.p_sorted_token_ids || !a.p_sorted_weights ||
-       !a.p_sorted_expert_ids || !a.p_total_tokens_post_pad)
+    // (an empty batch writes nothing but the totals unless experts without tokens keep a unit: its arrays may be
+    // empty, and an empty device array has no address)
+    const bool writes_rows = a.tokens > 0 || keep_empty;
+    if((a.tokens > 0 && (!a.p_topk_ids || !a.p_weights)) || !a.p_total_tokens_post_pad ||
+       (writes_rows && (!a.p_sorted_token_ids || !a.p_sorted_weights || !a.p_sorted_expert_ids)))
         return fail(MI355_MOE_E_INVALID, "moe_sorting: null input or output pointer");
     if(a.tokens < 0 || a.tokens >= (1 << 24))
         return fail(MI355_MOE_E_INVALID, "moe_sorting: tokens=%d outside [0, 2^24)", a.tokens);
