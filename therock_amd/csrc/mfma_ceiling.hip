@@ -136,9 +136,20 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(int iters, uint32_t s
 template <int MODE>
 int run(int ms_target, int zeros, double* tflops, hipStream_t stream)
 {
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    MI355_HIP_TRY(hipEventCreate(&e0));
-    MI355_HIP_TRY(hipEventCreate(&e1));
+    struct Events // destroyed on every way out
+    {
+        hipEvent_t a = nullptr, b = nullptr;
+        ~Events()
+        {
+            if(a)
+                (void)hipEventDestroy(a);
+            if(b)
+                (void)hipEventDestroy(b);
+        }
+    } ev;
+    MI355_HIP_TRY(hipEventCreate(&ev.a));
+    MI355_HIP_TRY(hipEventCreate(&ev.b));
+    const hipEvent_t e0 = ev.a, e1 = ev.b;
     const int grid  = device_info().num_cu;
     // MFMAs of one K step of 64 bytes per tile, FLOP of each
     constexpr int kPerStep     = ModeTraits<MODE>::kOpB == 16 ? 2 : 1;
@@ -168,8 +179,6 @@ int run(int ms_target, int zeros, double* tflops, hipStream_t stream)
                 iters *= 2; // launches of a few milliseconds: the launch gap does not show
         }
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     *tflops = flop / (total_ms * 1e-3) / 1e12;
     return MI355_MOE_OK;
 }
