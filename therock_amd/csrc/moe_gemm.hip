@@ -473,8 +473,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const unsigned char* _
     *reinterpret_cast<uint4*>(out + (int64_t)t * out_row_bytes + (int64_t)h0 * 2) = o;
 }
 
-// bytes per element of the intermediate activations the down GEMM reads: e4m3 on the fp8 path, int8 when the
-// int8 path re-quantises them (fused_quant 1 / 2), bf16 otherwise
+// bytes per element of the intermediate activations the down GEMM reads: e4m3 on the fp8 path (per 32 columns from
+// gemm0, or per row from the re-quantisation pass with fused_quant 1 / 2), int8 when the int8 path re-quantises them,
+// bf16 otherwise
 inline int y_bytes(const mi355_fused_moe_traits& t)
 {
     return (t.prec_i == MI355_MOE_FP8 || (t.prec_i == MI355_MOE_INT8 && t.fused_quant != 0)) ? 1 : 2;

@@ -14,8 +14,8 @@ struct WorkspaceLayout
     size_t y_off;      // intermediate activations Y [max_pad, inter] (bf16 or e4m3)
     size_t ys_off;     // e8m0 block scales of Y [inter / 32][ys_kb_stride] (fp8 path only)
     int64_t ys_kb_stride;
-    size_t yq_off;     // int8 copy of Y [max_pad, inter] and ...
-    size_t yrs_off;    // ... its fp32 per-row scales [max_pad] (int8 path with fused_quant 1 / 2 only)
+    size_t yq_off;     // int8 (e4m3) copy of Y [max_pad, inter] and ...
+    size_t yrs_off;    // ... its fp32 per-row scales [max_pad] (int8 and fp8 paths with fused_quant 1 / 2 only)
     size_t p_off;      // partial outputs per sorted row [max_pad, hidden] bf16
     size_t total;
     int64_t max_pad;
