@@ -72,6 +72,20 @@ def test_argument_blocks_have_the_layout_of_the_ck_tile_structs(tmp_path):
     assert r.returncode != 0 and "static assertion failed" in r.stderr
 
 
+def test_tile_order_of_the_large_tile_kernel_visits_every_tile_once(tmp_path):
+    """blocked_tile_of (the index arithmetic a workgroup of the large-tile kernel uses to find its tile) on the host:
+    a bijection for every (row tiles, column tiles) pair, with the locality it is there for."""
+    import shutil
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc is not installed")
+    exe = tmp_path / "tile_order_check"
+    subprocess.run([hipcc, "-std=c++17", "--cuda-host-only", "-I/opt/rocm/include", "-Wno-everything", "-o", str(exe),
+                    os.path.join(ROOT, "tests", "cpp", "tile_order_check.cpp")], check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and "tile_order_check ok" in r.stdout, r.stdout
+
+
 def test_sizes_out_of_range_are_rejected_on_the_host():
     """No entry point divides by or indexes with a size before checking it (0 experts used to kill the process)."""
     lib = _lib.load()

@@ -107,6 +107,30 @@ struct KernelTimerGroup
 constexpr int kMapHdr = 8;
 constexpr int kMapEnt = 8;
 
+// Order of an expert's work items in the large-tile kernel: blocks of kTileRowBlock row tiles; inside a block column
+// tile by column tile, the block's row tiles adjacent; the expert's last rows % kTileRowBlock row tiles form a
+// narrower block of their own.  rel = item number inside the expert (0 .. rows * cols - 1) -> column tile, row tile.
+constexpr int kTileRowBlock = 4;
+__host__ __device__ inline void blocked_tile_of(int rel, int rows, int cols, int& col, int& row)
+{
+    const int full    = rows / kTileRowBlock * kTileRowBlock; // row tiles in whole blocks
+    const int in_full = full * cols;
+    if(rel < in_full)
+    {
+        const int blk = rel / (kTileRowBlock * cols);
+        const int r2  = rel - blk * (kTileRowBlock * cols);
+        col           = r2 / kTileRowBlock;
+        row           = blk * kTileRowBlock + (r2 - col * kTileRowBlock);
+    }
+    else
+    {
+        const int rest = rows - full; // 1 .. kTileRowBlock - 1 row tiles, or the expert's only ones
+        const int r2   = rel - in_full;
+        col            = r2 / (rest > 0 ? rest : 1);
+        row            = full + (r2 - col * rest);
+    }
+}
+
 // what the sort can prepare for the GEMMs while it has the per-expert counts at hand
 struct GemmPlan
 {

@@ -170,30 +170,13 @@ __device__ __attribute__((always_inline)) inline TileRef lookup_tile(const int* 
     int j;
     if constexpr(CHUNKED)
     {
-        // An expert's items in blocks of kRowBlock row tiles: inside a block column tile by column tile, the block's
-        // row tiles adjacent.  The 32 consecutive items that run together on one XCD are then 4 row tiles x 8 column
-        // tiles: every K slice of their tokens is fetched into that L2 once for 8 column tiles and every weight slice
-        // once for 4 row tiles.  With all row tiles of a column tile adjacent (the order of the other kernels) an
-        // expert of 100 row tiles re-read its tokens from beyond L2 for every column tile: 9.2 GB of fetches against
-        // 0.9 GB of operands on the Zipf-routed workload.
-        constexpr int kRowBlock = 4;
-        const int rows   = max(b.x, 1);
-        const int full   = rows / kRowBlock * kRowBlock; // row tiles in whole blocks
-        const int in_full = full * n_ntiles;
-        if(rel < in_full)
-        {
-            const int blk = rel / (kRowBlock * n_ntiles);
-            const int r2  = rel - blk * (kRowBlock * n_ntiles);
-            t.nt          = r2 / kRowBlock;
-            j             = blk * kRowBlock + (r2 - t.nt * kRowBlock);
-        }
-        else
-        {
-            const int rest = rows - full; // 1 .. kRowBlock - 1 row tiles, or the expert's only ones
-            const int r2   = rel - in_full;
-            t.nt           = r2 / rest;
-            j              = full + (r2 - t.nt * rest);
-        }
+        // An expert's items in blocks of four row tiles (blocked_tile_of): inside a block column tile by column tile,
+        // the block's row tiles adjacent.  The 32 consecutive items that run together on one XCD are then 4 row tiles
+        // x 8 column tiles: every K slice of their tokens is fetched into that L2 once for 8 column tiles and every
+        // weight slice once for 4 row tiles.  With all row tiles of a column tile adjacent (the order of the other
+        // kernels) an expert of 100 row tiles re-read its tokens from beyond L2 for every column tile: 9.2 GB of
+        // fetches against 0.9 GB of operands on the Zipf-routed workload.
+        blocked_tile_of(rel, max(b.x, 1), n_ntiles, t.nt, j);
     }
     else
     {
